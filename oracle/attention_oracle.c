@@ -1,0 +1,285 @@
+/*
+ * TEST INFRASTRUCTURE — NOT PRODUCT CODE.
+ *
+ * CPU restatement of the grouped-query attention with sinks and sliding window that
+ * jaylauffer/loadngo runs on the CPU. Only tests, the smoke check and the benchmark's
+ * cpu_baseline leg may link or call this file; the shipped HIP path never does.
+ *
+ * The reference is Rust and cannot be built where this file is built (no rustc), so
+ * this is a restatement, function by function, of:
+ *
+ *   gpt-oss/src/model.rs:434-464            f32 attention of Model::step (the parity target)
+ *   gpt-oss/src/config.rs:99-103            even layers slide, odd layers see everything
+ *   metal-compute/tests/attention_grouped.rs:65-100   float64 definition (t, start, window, sinks)
+ *   metal-compute/tests/attention_grouped.rs:25-35    xorshift input generator `values`
+ *   metal-compute/tests/attention_grouped.rs:47-63    ring layout of a cache (`ring`)
+ *   metal-compute/src/apple.rs:1243-1256,1356-1369    accepted / rejected shapes
+ *   weights/src/dtype.rs:95-116             bf16 widen / round-to-nearest-even narrow
+ *
+ * What pins each function (tests/test_oracle_*.py): the three literal bf16 vectors and the
+ * round trip over all codes from dtype.rs:183-202; the integer generator reproduced
+ * independently in Python; the f32 restatement against the f64 definition; the f64
+ * definition against torch's scaled_dot_product_attention with an explicit mask and with
+ * the sink written as one extra key of value zero; closed forms (zero queries, constant
+ * values, window of one); ring independence; NaN poisoning of rows outside the window.
+ *
+ * Build: make -C oracle   (gcc -O2 -fno-fast-math -ffp-contract=off -fopenmp)
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define LNG_ORACLE_FULL UINT64_MAX
+
+/* ---- weights/src/dtype.rs:95-97 ------------------------------------------------------ */
+float lng_oracle_bf16_to_f32(uint16_t bits) {
+    uint32_t wide = (uint32_t)bits << 16;
+    float out;
+    memcpy(&out, &wide, 4);
+    return out;
+}
+
+/* ---- weights/src/dtype.rs:101-109: nearest, ties to even; NaN stays a quiet NaN ------- */
+uint16_t lng_oracle_f32_to_bf16(float value) {
+    uint32_t bits;
+    memcpy(&bits, &value, 4);
+    if (value != value) {
+        return (uint16_t)((bits >> 16) | 0x40);
+    }
+    uint32_t bias = 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)((bits + bias) >> 16);
+}
+
+void lng_oracle_widen(const uint16_t *src, float *dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) dst[i] = lng_oracle_bf16_to_f32(src[i]);
+}
+
+void lng_oracle_narrow(const float *src, uint16_t *dst, size_t n) {
+    for (size_t i = 0; i < n; ++i) dst[i] = lng_oracle_f32_to_bf16(src[i]);
+}
+
+/* ---- metal-compute/tests/attention_grouped.rs:25-35 ---------------------------------- */
+void lng_oracle_values(uint64_t seed, size_t n, float *out) {
+    uint64_t s = seed | 1u;
+    for (size_t i = 0; i < n; ++i) {
+        s ^= s << 13;
+        s ^= s >> 7;
+        s ^= s << 17;
+        out[i] = (float)(s >> 40) / (float)((uint64_t)1 << 23) - 1.0f;
+    }
+}
+
+/*
+ * ---- metal-compute/tests/attention_grouped.rs:47-63 ----------------------------------
+ * `all` holds a row of `row` floats for every absolute position below start + t. `out`
+ * receives the cache a decoder would hold after reaching start + t: position p in row
+ * p % slots. Rows the plain operator must never read are NaN; the tiled operator's padded
+ * rows are zero. Returns the number of rows written (rows * row floats must fit `out`).
+ */
+size_t lng_oracle_ring_rows(uint64_t t, uint64_t start, uint64_t slots, int tiled) {
+    uint64_t end = start + t;
+    if (!tiled) return slots < end ? slots : end;
+    if (slots < end) return slots;
+    return (end + 31) / 32 * 32;
+}
+
+size_t lng_oracle_ring(const float *all, size_t row, uint64_t t, uint64_t start,
+                       uint64_t slots, int tiled, float *out) {
+    uint64_t end = start + t;
+    size_t rows = lng_oracle_ring_rows(t, start, slots, tiled);
+    float fill = tiled ? 0.0f : NAN;
+    for (size_t i = 0; i < rows * row; ++i) out[i] = fill;
+    uint64_t from = end > slots ? end - slots : 0;
+    for (uint64_t p = from; p < end; ++p) {
+        memcpy(out + (p % slots) * row, all + p * row, row * sizeof(float));
+    }
+    return rows;
+}
+
+/*
+ * ---- metal-compute/src/apple.rs:1243-1256 (plain) and 1356-1369 (tiled) ---------------
+ * 1 when the reference would record the dispatch, 0 when it answers Error::Dispatch.
+ */
+int lng_oracle_accepts(uint64_t t, uint64_t start, uint64_t heads, uint64_t kv_heads,
+                       uint64_t dim, uint64_t window, uint64_t slots, int tiled) {
+    uint64_t end = start + t;
+    uint64_t need = window > UINT64_MAX - t ? UINT64_MAX : window + t; /* saturating_add */
+    if (t == 0 || kv_heads == 0 || heads % kv_heads != 0 || dim == 0 || dim > 512 ||
+        window == 0 || slots == 0) {
+        return 0;
+    }
+    if (!tiled) {
+        if (dim % 32 != 0) return 0;
+        if (slots < end && slots < need) return 0;
+    } else {
+        if (dim % 16 != 0) return 0;
+        if (slots < end && (slots % 32 != 0 || slots < need)) return 0;
+    }
+    /* apple.rs:1257-1272: every count must fit u32 */
+    uint64_t win = window < end ? window : end;
+    uint64_t groups = tiled ? (t + 31) / 32 * heads : t * heads;
+    if (t > UINT32_MAX || start > UINT32_MAX || heads > UINT32_MAX || kv_heads > UINT32_MAX ||
+        win > UINT32_MAX || slots > UINT32_MAX || groups > UINT32_MAX) {
+        return 0;
+    }
+    return 1;
+}
+
+/*
+ * ---- gpt-oss/src/model.rs:434-464, generalised to (t, start, window, slots) -----------
+ * q   [t][heads][dim] f32
+ * k,v [rows][kv_heads][dim] f32, position p in row p % slots (a flat Vec in model.rs,
+ *     i.e. slots = infinity; the ring is how metal-compute's callers hold it)
+ * sinks [heads] or NULL (NULL: the sink logit is -inf, exp(-inf) = 0)
+ * out [t][heads][dim] f32
+ *
+ * Operation order is the reference's: the score is a sequential f32 sum over the head
+ * dimension, times scale (445-448); max folds from the sink (449-450); total starts at
+ * exp(sink - max) and adds exp(score - max) in position order (451-455); each output
+ * element accumulates weight / total * value in position order from 0 (456-463).
+ * `threads` > 1 spreads (query, head) pairs over OpenMP threads without changing any
+ * per-pair arithmetic; the reference itself walks heads on one thread.
+ */
+static void attend_f32(const float *query, const float *k, const float *v, const float *sink_at,
+                       float *target, uint64_t pos, uint64_t kv, uint64_t kv_heads, uint64_t dim,
+                       uint64_t window, uint64_t slots, float scale) {
+    const uint64_t first = (window == LNG_ORACLE_FULL || pos + 1 <= window) ? 0 : pos + 1 - window;
+    const uint64_t count = pos + 1 - first;
+    float *scores = (float *)malloc(count * sizeof(float));
+    for (uint64_t p = first; p <= pos; ++p) {
+        const float *key = k + ((p % slots) * kv_heads + kv) * dim;
+        float sum = 0.0f;
+        for (uint64_t d = 0; d < dim; ++d) sum += query[d] * key[d];
+        scores[p - first] = sum * scale;
+    }
+    const float sink = sink_at ? *sink_at : -INFINITY;
+    float max = sink;
+    for (uint64_t j = 0; j < count; ++j) max = fmaxf(max, scores[j]);
+    float total = expf(sink - max);
+    for (uint64_t j = 0; j < count; ++j) {
+        scores[j] = expf(scores[j] - max);
+        total += scores[j];
+    }
+    for (uint64_t d = 0; d < dim; ++d) target[d] = 0.0f;
+    for (uint64_t p = first; p <= pos; ++p) {
+        const float *value = v + ((p % slots) * kv_heads + kv) * dim;
+        const float weight = scores[p - first];
+        for (uint64_t d = 0; d < dim; ++d) target[d] += weight / total * value[d];
+    }
+    free(scores);
+}
+
+void lng_oracle_attention_f32(const float *q, const float *k, const float *v,
+                              const float *sinks, float *out, uint64_t t, uint64_t start,
+                              uint64_t heads, uint64_t kv_heads, uint64_t dim, uint64_t window,
+                              uint64_t slots, float scale, int threads) {
+    const uint64_t group = heads / kv_heads;
+    const int64_t pairs = (int64_t)(t * heads);
+    if (threads < 1) threads = 1;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads) if (threads > 1)
+    for (int64_t pair = 0; pair < pairs; ++pair) {
+        const uint64_t i = (uint64_t)pair / heads;
+        const uint64_t head = (uint64_t)pair % heads;
+        attend_f32(q + (i * heads + head) * dim, k, v, sinks ? sinks + head : NULL,
+                   out + (i * heads + head) * dim, start + i, head / group, kv_heads, dim, window,
+                   slots, scale);
+    }
+}
+
+/*
+ * ---- metal-compute/tests/attention_grouped.rs:65-100 ---------------------------------
+ * The float64 definition the reference's operator tests compare against; same layouts as
+ * above (the test indexes a flat array of all positions; slots >= start + t gives that).
+ * Every term is exp(x - m) / z * v in f64, summed in position order, then cast to f32.
+ */
+void lng_oracle_attention_f64(const float *q, const float *k, const float *v,
+                              const float *sinks, float *out, uint64_t t, uint64_t start,
+                              uint64_t heads, uint64_t kv_heads, uint64_t dim, uint64_t window,
+                              uint64_t slots, float scale, int threads) {
+    const uint64_t group = heads / kv_heads;
+    const int64_t pairs = (int64_t)(t * heads);
+    if (threads < 1) threads = 1;
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads) if (threads > 1)
+    for (int64_t pair = 0; pair < pairs; ++pair) {
+        const uint64_t i = (uint64_t)pair / heads;
+        const uint64_t h = (uint64_t)pair % heads;
+        const uint64_t last = start + i;
+        const uint64_t first = (window == LNG_ORACLE_FULL || last + 1 <= window) ? 0 : last + 1 - window;
+        const uint64_t g = h / group;
+        const float *qt = q + (i * heads + h) * dim;
+        const uint64_t count = last + 1 - first;
+        double *scores = (double *)malloc(count * sizeof(double));
+        for (uint64_t p = first; p <= last; ++p) {
+            const float *kr = k + ((p % slots) * kv_heads + g) * dim;
+            double sum = 0.0;
+            for (uint64_t d = 0; d < dim; ++d) sum += (double)qt[d] * (double)kr[d];
+            scores[p - first] = sum * (double)scale;
+        }
+        const double sink = sinks ? (double)sinks[h] : -INFINITY;
+        double m = sink;
+        for (uint64_t j = 0; j < count; ++j) m = fmax(m, scores[j]);
+        double z = 0.0;
+        for (uint64_t j = 0; j < count; ++j) z += exp(scores[j] - m);
+        z += exp(sink - m);
+        for (uint64_t d = 0; d < dim; ++d) {
+            double acc = 0.0;
+            for (uint64_t p = first; p <= last; ++p) {
+                acc += exp(scores[p - first] - m) / z *
+                       (double)v[((p % slots) * kv_heads + g) * dim + d];
+            }
+            out[(i * heads + h) * dim + d] = (float)acc;
+        }
+        free(scores);
+    }
+}
+
+/*
+ * bf16 in, bf16 out, f32 accumulate: inputs are widened exactly (dtype.rs:95-97), the f32
+ * restatement above runs on them, and the output is rounded to nearest even
+ * (dtype.rs:101-109). `rows` is the number of cache rows behind k and v. Sinks stay f32.
+ */
+void lng_oracle_attention_bf16(const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                               const float *sinks, uint16_t *out, uint64_t rows, uint64_t t,
+                               uint64_t start, uint64_t heads, uint64_t kv_heads, uint64_t dim,
+                               uint64_t window, uint64_t slots, float scale, int threads) {
+    const size_t nq = (size_t)(t * heads * dim);
+    const size_t nk = (size_t)(rows * kv_heads * dim);
+    float *qf = (float *)malloc(nq * sizeof(float));
+    float *kf = (float *)malloc(nk * sizeof(float));
+    float *vf = (float *)malloc(nk * sizeof(float));
+    float *of = (float *)malloc(nq * sizeof(float));
+    lng_oracle_widen(q, qf, nq);
+    lng_oracle_widen(k, kf, nk);
+    lng_oracle_widen(v, vf, nk);
+    lng_oracle_attention_f32(qf, kf, vf, sinks, of, t, start, heads, kv_heads, dim, window, slots,
+                             scale, threads);
+    lng_oracle_narrow(of, out, nq);
+    free(qf);
+    free(kf);
+    free(vf);
+    free(of);
+}
+
+/*
+ * The same, for a subset of query rows: row i of the output is the attention of query row
+ * i at absolute position positions[i] (each its own `start`, t = 1). Lets a long prefill be
+ * checked, and timed as a CPU baseline, on a sample of rows instead of all of them.
+ */
+void lng_oracle_attention_rows_f32(const float *q, const float *k, const float *v,
+                                   const float *sinks, float *out, const uint64_t *positions,
+                                   uint64_t n_rows, uint64_t heads, uint64_t kv_heads, uint64_t dim,
+                                   uint64_t window, uint64_t slots, float scale, int threads) {
+    const uint64_t group = heads / kv_heads;
+    if (threads < 1) threads = 1;
+    const int64_t pairs = (int64_t)(n_rows * heads);
+#pragma omp parallel for schedule(dynamic, 1) num_threads(threads) if (threads > 1)
+    for (int64_t pair = 0; pair < pairs; ++pair) {
+        const uint64_t i = (uint64_t)pair / heads;
+        const uint64_t head = (uint64_t)pair % heads;
+        attend_f32(q + (i * heads + head) * dim, k, v, sinks ? sinks + head : NULL,
+                   out + (i * heads + head) * dim, positions[i], head / group, kv_heads, dim,
+                   window, slots, scale);
+    }
+}

@@ -1,0 +1,170 @@
+"""TEST INFRASTRUCTURE — NOT PRODUCT CODE.
+
+ctypes access to ``liblng_oracle.so`` (built from ``attention_oracle.c``, which cites the
+reference lines each function restates). Only ``tests/``, ``__graft_entry__.smoke`` and the
+``cpu_baseline`` leg of ``bench.py`` import this module; ``loadngo_amd`` never does.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liblng_oracle.so")
+FULL = 2**64 - 1  # GroupedShape.window = usize::MAX: every earlier position is visible
+
+_u64 = ctypes.c_uint64
+_fp = ctypes.POINTER(ctypes.c_float)
+_hp = ctypes.POINTER(ctypes.c_uint16)
+
+
+def build():
+    """Compiles the oracle with the committed Makefile."""
+    subprocess.check_call(["make", "-C", _HERE, "-B", "liblng_oracle.so"], stdout=subprocess.DEVNULL)
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.lng_oracle_bf16_to_f32.restype = ctypes.c_float
+    lib.lng_oracle_bf16_to_f32.argtypes = [ctypes.c_uint16]
+    lib.lng_oracle_f32_to_bf16.restype = ctypes.c_uint16
+    lib.lng_oracle_f32_to_bf16.argtypes = [ctypes.c_float]
+    lib.lng_oracle_widen.argtypes = [_hp, _fp, ctypes.c_size_t]
+    lib.lng_oracle_narrow.argtypes = [_fp, _hp, ctypes.c_size_t]
+    lib.lng_oracle_values.argtypes = [_u64, ctypes.c_size_t, _fp]
+    lib.lng_oracle_ring_rows.restype = ctypes.c_size_t
+    lib.lng_oracle_ring_rows.argtypes = [_u64, _u64, _u64, ctypes.c_int]
+    lib.lng_oracle_ring.restype = ctypes.c_size_t
+    lib.lng_oracle_ring.argtypes = [_fp, ctypes.c_size_t, _u64, _u64, _u64, ctypes.c_int, _fp]
+    lib.lng_oracle_accepts.restype = ctypes.c_int
+    lib.lng_oracle_accepts.argtypes = [_u64] * 7 + [ctypes.c_int]
+    attn = [_fp, _fp, _fp, _fp, _fp] + [_u64] * 7 + [ctypes.c_float, ctypes.c_int]
+    lib.lng_oracle_attention_f32.argtypes = attn
+    lib.lng_oracle_attention_f64.argtypes = attn
+    lib.lng_oracle_attention_bf16.argtypes = (
+        [_hp, _hp, _hp, _fp, _hp] + [_u64] * 8 + [ctypes.c_float, ctypes.c_int]
+    )
+    lib.lng_oracle_attention_rows_f32.argtypes = (
+        [_fp, _fp, _fp, _fp, _fp, ctypes.POINTER(_u64)] + [_u64] * 6 + [ctypes.c_float, ctypes.c_int]
+    )
+    return lib
+
+
+_lib = _load()
+
+
+def _f(a):
+    return a.ctypes.data_as(_fp)
+
+
+def _h(a):
+    return a.ctypes.data_as(_hp)
+
+
+def bf16_to_f32(bits):
+    """weights/src/dtype.rs:95-97. ``bits``: uint16 array or scalar."""
+    a = np.ascontiguousarray(bits, dtype=np.uint16)
+    out = np.empty(a.shape, dtype=np.float32)
+    _lib.lng_oracle_widen(_h(a.reshape(-1)), _f(out.reshape(-1)), a.size)
+    return out
+
+
+def f32_to_bf16(values):
+    """weights/src/dtype.rs:101-109. Returns uint16 bit patterns."""
+    a = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(a.shape, dtype=np.uint16)
+    _lib.lng_oracle_narrow(_f(a.reshape(-1)), _h(out.reshape(-1)), a.size)
+    return out
+
+
+def values(seed, n):
+    """metal-compute/tests/attention_grouped.rs:25-35."""
+    out = np.empty(n, dtype=np.float32)
+    _lib.lng_oracle_values(seed, n, _f(out))
+    return out
+
+
+def ring(all_rows, t, start, slots, tiled):
+    """metal-compute/tests/attention_grouped.rs:47-63. ``all_rows``: [start+t][row] f32."""
+    all_rows = np.ascontiguousarray(all_rows, dtype=np.float32)
+    row = all_rows.shape[1]
+    rows = _lib.lng_oracle_ring_rows(t, start, slots, int(tiled))
+    out = np.empty((rows, row), dtype=np.float32)
+    _lib.lng_oracle_ring(_f(all_rows), row, t, start, slots, int(tiled), _f(out))
+    return out
+
+
+def accepts(t, start, heads, kv_heads, dim, window, slots, tiled=False):
+    """metal-compute/src/apple.rs:1243-1272 and 1356-1385."""
+    return bool(_lib.lng_oracle_accepts(t, start, heads, kv_heads, dim, window, slots, int(tiled)))
+
+
+def _attention(fn, q, k, v, sinks, start, window, slots, scale, threads):
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    t, heads, dim = q.shape
+    kv_heads = k.shape[1]
+    assert k.shape == v.shape and k.shape[2] == dim
+    assert k.shape[0] >= min(slots, start + t), "cache holds too few rows"
+    out = np.empty_like(q)
+    s = None if sinks is None else np.ascontiguousarray(sinks, dtype=np.float32)
+    fn(_f(q), _f(k), _f(v), None if s is None else _f(s), _f(out), t, start, heads, kv_heads, dim,
+       window, slots, scale, threads)
+    return out
+
+
+def attention_f32(q, k, v, sinks, start, window=FULL, slots=None, scale=None, threads=1):
+    """gpt-oss/src/model.rs:434-464 over q [t][H][D], k/v [rows][G][D] (row = pos % slots)."""
+    slots = k.shape[0] if slots is None else slots
+    scale = 1.0 / np.sqrt(np.float32(q.shape[2])) if scale is None else scale
+    return _attention(_lib.lng_oracle_attention_f32, q, k, v, sinks, start, window, slots,
+                      float(scale), threads)
+
+
+def attention_f64(q, k, v, sinks, start, window=FULL, slots=None, scale=None, threads=1):
+    """metal-compute/tests/attention_grouped.rs:65-100."""
+    slots = k.shape[0] if slots is None else slots
+    scale = 1.0 / np.sqrt(np.float32(q.shape[2])) if scale is None else scale
+    return _attention(_lib.lng_oracle_attention_f64, q, k, v, sinks, start, window, slots,
+                      float(scale), threads)
+
+
+def attention_bf16(q, k, v, sinks, start, window=FULL, slots=None, scale=None, threads=1):
+    """bf16 bit patterns in and out (uint16 arrays), f32 arithmetic of model.rs:434-464."""
+    q = np.ascontiguousarray(q, dtype=np.uint16)
+    k = np.ascontiguousarray(k, dtype=np.uint16)
+    v = np.ascontiguousarray(v, dtype=np.uint16)
+    t, heads, dim = q.shape
+    rows, kv_heads, _ = k.shape
+    slots = rows if slots is None else slots
+    scale = 1.0 / np.sqrt(np.float32(dim)) if scale is None else scale
+    assert rows >= min(slots, start + t), "cache holds too few rows"
+    out = np.empty_like(q)
+    s = None if sinks is None else np.ascontiguousarray(sinks, dtype=np.float32)
+    _lib.lng_oracle_attention_bf16(_h(q), _h(k), _h(v), None if s is None else _f(s), _h(out), rows,
+                                   t, start, heads, kv_heads, dim, window, slots, float(scale),
+                                   threads)
+    return out
+
+
+def attention_rows_f32(q, k, v, sinks, positions, window=FULL, slots=None, scale=None, threads=1):
+    """Row i of q attends from absolute position positions[i] (a sample of a long pass)."""
+    q = np.ascontiguousarray(q, dtype=np.float32)
+    k = np.ascontiguousarray(k, dtype=np.float32)
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    n, heads, dim = q.shape
+    kv_heads = k.shape[1]
+    slots = k.shape[0] if slots is None else slots
+    scale = 1.0 / np.sqrt(np.float32(dim)) if scale is None else scale
+    pos = np.ascontiguousarray(positions, dtype=np.uint64)
+    assert pos.shape == (n,)
+    out = np.empty_like(q)
+    s = None if sinks is None else np.ascontiguousarray(sinks, dtype=np.float32)
+    _lib.lng_oracle_attention_rows_f32(_f(q), _f(k), _f(v), None if s is None else _f(s), _f(out),
+                                       pos.ctypes.data_as(ctypes.POINTER(_u64)), n, heads, kv_heads,
+                                       dim, window, slots, float(scale), threads)
+    return out
