@@ -1,0 +1,200 @@
+/*
+ * lng_hip.h — C ABI of the MI355X (gfx950) grouped-attention operator library.
+ *
+ * One shared library, liblng_hip.so, replaces the part of loadngo's `metal-compute` crate
+ * that the gpt-oss attention path uses. Every entry point names the reference interface it
+ * stands in for (paths relative to the reference repository). Plain pointers and sizes
+ * only; errors are negative codes plus a thread-local message.
+ *
+ * Differences from the Metal original that a binding must know:
+ *  - Device memory is not CPU-visible: Buffer::as_f32()/as_bytes_mut() become
+ *    lng_hip_download()/lng_hip_upload().
+ *  - Every attention entry point takes an element type (f32 as in the reference, or bf16
+ *    in/out with f32 accumulation). Sinks are always f32.
+ *  - Counts are 64-bit throughout (the reference narrows to u32 and refuses what does not
+ *    fit; the same refusals are kept so behaviour is identical).
+ */
+#ifndef LNG_HIP_H
+#define LNG_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GroupedShape.window = usize::MAX: a query sees every earlier position. */
+#define LNG_WINDOW_FULL UINT64_MAX
+/* lng_decode_item.sinks_offset when the item has no sinks. */
+#define LNG_NO_SINKS UINT64_MAX
+
+/* metal-compute/src/lib.rs:41-53 — enum Error {NoDevice, Compile, Alloc, Dispatch, Gpu}. */
+typedef enum lng_status {
+    LNG_OK = 0,
+    LNG_ERR_NO_DEVICE = -1, /* Error::NoDevice */
+    LNG_ERR_COMPILE = -2,   /* Error::Compile(String): code object missing or a kernel not found */
+    LNG_ERR_ALLOC = -3,     /* Error::Alloc(usize) */
+    LNG_ERR_DISPATCH = -4,  /* Error::Dispatch(String): refused before anything is recorded */
+    LNG_ERR_GPU = -5        /* Error::Gpu(String): the submitted work failed */
+} lng_status;
+
+typedef enum lng_dtype {
+    LNG_F32 = 0, /* the reference's only element type */
+    LNG_BF16 = 1 /* weights/src/dtype.rs:95-116 convention: high half of an f32, RNE narrowing */
+} lng_dtype;
+
+typedef struct lng_gpu lng_gpu;       /* apple.rs:105   struct Gpu */
+typedef struct lng_buffer lng_buffer; /* apple.rs:391   struct Buffer, and apple.rs:465 Resident */
+typedef struct lng_batch lng_batch;   /* apple.rs:541   struct Batch */
+
+/* apple.rs:507-521 — Slice {buffer, offset, len}: bytes offset..offset+len of the batch's
+ * buffer number `buffer`: its own buffers first, then the residents it attached, in order. */
+typedef struct lng_slice {
+    uint64_t buffer;
+    uint64_t offset;
+    uint64_t len;
+} lng_slice;
+
+/* apple.rs:598-614 — GroupedShape. `window` counts the query itself; position s of the
+ * cache is in row s % slots. */
+typedef struct lng_grouped_shape {
+    uint64_t t;        /* new positions (queries) */
+    uint64_t start;    /* absolute position of the first of them */
+    uint64_t heads;    /* query heads */
+    uint64_t kv_heads; /* key/value heads; heads is a multiple of it */
+    uint64_t dim;      /* width of every head: multiple of 32 (16 for tiled), at most 512 */
+    uint64_t window;   /* positions each query sees, itself included; LNG_WINDOW_FULL for all */
+    uint64_t slots;    /* rows in the key and value buffers */
+    float scale;
+} lng_grouped_shape;
+
+/* apple.rs:536-539 — Completed {buffers, gpu_time}: handed to the completion callback.
+ * `status` is LNG_OK or LNG_ERR_GPU (then `message` says why); the buffers the batch owned
+ * are the caller's again when the callback runs. */
+typedef struct lng_completed {
+    int status;
+    double gpu_seconds;
+    const char *message; /* valid during the callback only */
+} lng_completed;
+
+typedef void (*lng_on_done)(const lng_completed *done, void *user);
+
+/* The message of the calling thread's most recent failed call ("" if none). */
+const char *lng_hip_last_error(void);
+
+/* ---- device --------------------------------------------------------------------------- */
+
+/* apple.rs:105 Gpu::new — opens HIP device `device`, loads the gfx950 code object embedded
+ * in the library and resolves every kernel. LNG_ERR_NO_DEVICE / LNG_ERR_COMPILE. */
+int lng_hip_open(int device, lng_gpu **gpu);
+/* Drop of Gpu. Waits for submitted batches; buffers must have been freed before. */
+void lng_hip_close(lng_gpu *gpu);
+/* Device name (e.g. "gfx950..."), copied into `name` (NUL-terminated, truncated to `cap`). */
+int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
+
+/* ---- memory --------------------------------------------------------------------------- */
+
+/* apple.rs:255 Gpu::buffer(len) — device memory, contents unspecified. len == 0 is
+ * LNG_ERR_ALLOC ("Alloc(0)", apple.rs:256-258). */
+int lng_hip_buffer(lng_gpu *gpu, size_t len, lng_buffer **buffer);
+/* apple.rs:297 Gpu::resident(bytes) — read-only memory filled once; may be attached to any
+ * number of batches at once and is never an output (apple.rs:896-900). */
+int lng_hip_resident(lng_gpu *gpu, const void *bytes, size_t len, lng_buffer **resident);
+/* Drop of Buffer / Arc<Resident>. LNG_ERR_DISPATCH while a batch owns or has attached it. */
+int lng_hip_buffer_free(lng_buffer *buffer);
+size_t lng_hip_buffer_len(const lng_buffer *buffer);
+/* Raw device address, for callers that share the memory with other HIP code. */
+void *lng_hip_buffer_device_ptr(lng_buffer *buffer);
+/* Buffer::as_bytes_mut()[offset..offset+len].copy_from_slice(src) (apple.rs:409-416).
+ * Refused while a batch owns the buffer and for residents. Blocking. */
+int lng_hip_upload(lng_buffer *buffer, size_t offset, const void *src, size_t len);
+/* Buffer::as_bytes()[offset..offset+len] (apple.rs:401-407). Refused while owned. Blocking. */
+int lng_hip_download(lng_buffer *buffer, size_t offset, void *dst, size_t len);
+/* Fills bytes [offset, offset+len) with `byte`. Refused while owned. Blocking. */
+int lng_hip_fill(lng_buffer *buffer, size_t offset, int byte, size_t len);
+
+/* ---- batches -------------------------------------------------------------------------- */
+
+/* apple.rs:365 Gpu::batch(buffers, Dispatch::Serial) — starts recording a batch that owns
+ * `buffers` until it completes or is dropped; dispatches name them by position. */
+int lng_hip_batch(lng_gpu *gpu, lng_buffer *const *buffers, size_t n_buffers, lng_batch **batch);
+/* apple.rs:835 Batch::attach(&resident) -> Slice covering the whole resident. */
+int lng_hip_batch_attach(lng_batch *batch, lng_buffer *resident, lng_slice *whole);
+/* apple.rs:829 Batch::dispatches(). */
+size_t lng_hip_batch_dispatches(const lng_batch *batch);
+/* apple.rs:2194 Batch::barrier(). Dispatches of a batch already run in order here. */
+int lng_hip_batch_barrier(lng_batch *batch);
+/* apple.rs:2202 Batch::commit(proactor, on_done) — submits without blocking. `on_done` runs
+ * once on a library thread when the GPU has finished (the Rust shim re-posts it to the
+ * caller's proactor, as apple.rs:2231-2232 does); it may be NULL. The batch handle stays
+ * valid for lng_hip_batch_wait / lng_hip_batch_drop. */
+int lng_hip_batch_commit(lng_batch *batch, lng_on_done on_done, void *user);
+/* Blocks until a committed batch has finished; gpu_seconds (may be NULL) receives the time
+ * between its first and last dispatch on the device (Completed.gpu_time, apple.rs:2219-2221). */
+int lng_hip_batch_wait(lng_batch *batch, double *gpu_seconds);
+/* Drop of Batch: an uncommitted batch runs nothing (apple.rs:553-561); a committed one is
+ * waited for. Its buffers are the caller's again. */
+void lng_hip_batch_drop(lng_batch *batch);
+
+/* ---- the attention operator ------------------------------------------------------------ */
+
+/* Shape rules alone, with no device: LNG_OK or LNG_ERR_DISPATCH, exactly the refusals of
+ * apple.rs:1243-1272 (tiled == 0) and apple.rs:1356-1385 (tiled != 0). */
+int lng_hip_check_grouped(const lng_grouped_shape *shape, int tiled);
+
+/* apple.rs:1199 Batch::attention_grouped and apple.rs:1213 attention_grouped_with_sinks
+ * (`sinks` NULL for the former). q, out: [t][heads][dim]; k, v: [rows][kv_heads][dim] with
+ * rows = min(slots, start + t); sinks: [heads] f32. Slice lengths must be exactly what the
+ * shape implies (apple.rs:868-873), inside their buffers (874-879), offsets aligned to the
+ * element size; the output must not be resident memory nor overlap an input (896-906). */
+int lng_hip_attention_grouped(lng_batch *batch, lng_slice q, lng_slice k, lng_slice v, lng_slice out,
+                              const lng_slice *sinks, const lng_grouped_shape *shape, int dtype);
+
+/* apple.rs:1311 Batch::attention_grouped_tiled and apple.rs:1324 ..._tiled_with_sinks: the
+ * prompt-pass form. q and out hold t rounded up to 32 rows; k and v hold `slots` rows when
+ * positions wrap (slots < start + t; then slots % 32 == 0) and start + t rounded up to 32
+ * otherwise. Padded rows are never read here (the reference multiplies them by zero). */
+int lng_hip_attention_grouped_tiled(lng_batch *batch, lng_slice q, lng_slice k, lng_slice v,
+                                    lng_slice out, const lng_slice *sinks,
+                                    const lng_grouped_shape *shape, int dtype);
+
+/* apple.rs:1762 Batch::copy_rows((src, src_stride), (dst, dst_stride), rows, width): how
+ * gpt-oss/src/gpu.rs:744-759 writes new K and V rows into a cache. Strides and width count
+ * elements. src_dtype != dst_dtype converts (f32 -> bf16 rounds to nearest even): the new
+ * rows of an f32 projection go straight into a bf16 cache. */
+int lng_hip_copy_rows(lng_batch *batch, lng_slice src, uint64_t src_stride, int src_dtype,
+                      lng_slice dst, uint64_t dst_stride, int dst_dtype, uint64_t rows,
+                      uint64_t width);
+
+/* One decoding query per item, many sequences and layers in one dispatch. No counterpart
+ * in the reference, which records one attention_grouped_with_sinks per sequence and layer
+ * (gpt-oss/src/gpu.rs:794-805); each item computes exactly what that call computes with
+ * t = 1. Offsets are bytes into the named buffers of the batch. */
+typedef struct lng_decode_item {
+    uint64_t q_offset;     /* [heads][dim] */
+    uint64_t out_offset;   /* [heads][dim] */
+    uint64_t k_offset;     /* [min(slots, start+1)][kv_heads][dim] */
+    uint64_t v_offset;
+    uint64_t sinks_offset; /* [heads] f32, or LNG_NO_SINKS */
+    uint64_t start;        /* absolute position of the query */
+    uint64_t window;       /* LNG_WINDOW_FULL for all */
+    uint64_t slots;
+} lng_decode_item;
+
+int lng_hip_attention_decode_batched(lng_batch *batch, uint64_t q_buffer, uint64_t k_buffer,
+                                     uint64_t v_buffer, uint64_t out_buffer, uint64_t sinks_buffer,
+                                     const lng_decode_item *items, size_t n_items, uint64_t heads,
+                                     uint64_t kv_heads, uint64_t dim, float scale, int dtype);
+
+/* Deterministic synthetic data written on the device (benchmarks and full-size tests):
+ * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
+ * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The
+ * same integers are documented in the library source so a host can reproduce any element. */
+int lng_hip_fill_synthetic(lng_batch *batch, lng_slice dst, int dtype, uint64_t seed, float scale,
+                           uint64_t period);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LNG_HIP_H */

@@ -1,0 +1,50 @@
+"""Builds liblng_hip.so in-tree: the gfx950 code object from csrc/lng_kernels.hip
+(``hipcc --genco``), embedded into the host library compiled from csrc/lng_hip.cpp.
+
+    python -m loadngo_amd.build
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "liblng_hip.so")
+HSACO = os.path.join(HERE, "lng_kernels.hsaco")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+# Packed-FP32 instruction selection is switched off for every kernel.
+DEVICE_FLAGS = [
+    "--genco", "--offload-arch=gfx950", "-O3", "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout)
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+    return proc.stdout
+
+
+def build(verbose=False):
+    """Compiles the kernels and the host library. Always recompiles."""
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    out = _run([hipcc] + DEVICE_FLAGS + [os.path.join(CSRC, "lng_kernels.hip"), "-o", HSACO])
+    if verbose and out:
+        print(out)
+    out = _run([
+        "g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-result", "-pthread",
+        "-D__HIP_PLATFORM_AMD__", "-DLNG_HSACO_PATH=\"%s\"" % HSACO,
+        "-I" + os.path.join(ROCM, "include"),
+        os.path.join(CSRC, "lng_hip.cpp"), "-o", LIB,
+        "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
+    ])
+    if verbose and out:
+        print(out)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

@@ -1,0 +1,395 @@
+"""Host-side mirror of loadngo's ``metal-compute`` operator interface for the attention
+path, over the C ABI of ``liblng_hip.so`` (``include/lng_hip.h``).
+
+Names, argument meaning and error behaviour follow metal-compute/src/apple.rs and lib.rs:
+``Gpu`` (apple.rs:105), ``Buffer`` (391), ``Resident`` (465), ``Slice`` (507), ``Batch`` (541),
+``GroupedShape`` (598), ``Completed`` (536), ``Error`` (lib.rs:41-53). Device memory is not
+CPU-visible here, so ``Buffer.as_f32()`` style access is ``Buffer.write`` / ``Buffer.read``.
+
+There is no CPU fallback: without the built library, or without a HIP device, construction
+fails (``Error.Compile`` / ``Error.NoDevice``).
+"""
+import ctypes
+import os
+import threading
+
+import numpy as np
+
+FULL = 2**64 - 1  # GroupedShape.window = usize::MAX
+NO_SINKS = 2**64 - 1
+F32, BF16 = 0, 1
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liblng_hip.so")
+
+
+class Error(Exception):
+    """metal-compute/src/lib.rs:41-53."""
+
+
+class NoDevice(Error):
+    pass
+
+
+class Compile(Error):
+    pass
+
+
+class Alloc(Error):
+    pass
+
+
+class Dispatch(Error):
+    pass
+
+
+class GpuFailure(Error):  # Error::Gpu
+    pass
+
+
+Error.NoDevice, Error.Compile, Error.Alloc, Error.Dispatch, Error.Gpu = (
+    NoDevice, Compile, Alloc, Dispatch, GpuFailure)
+_ERRORS = {-1: NoDevice, -2: Compile, -3: Alloc, -4: Dispatch, -5: GpuFailure}
+
+
+class _Slice(ctypes.Structure):
+    _fields_ = [("buffer", ctypes.c_uint64), ("offset", ctypes.c_uint64), ("len", ctypes.c_uint64)]
+
+
+class _Shape(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in ("t", "start", "heads", "kv_heads", "dim", "window", "slots")]
+    _fields_.append(("scale", ctypes.c_float))
+
+
+class _Item(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in
+                ("q_offset", "out_offset", "k_offset", "v_offset", "sinks_offset", "start", "window", "slots")]
+
+
+class _Completed(ctypes.Structure):
+    _fields_ = [("status", ctypes.c_int), ("gpu_seconds", ctypes.c_double), ("message", ctypes.c_char_p)]
+
+
+_ON_DONE = ctypes.CFUNCTYPE(None, ctypes.POINTER(_Completed), ctypes.c_void_p)
+
+# Every symbol include/lng_hip.h declares: (restype, argtypes)
+_P = ctypes.c_void_p
+_U64 = ctypes.c_uint64
+SYMBOLS = {
+    "lng_hip_last_error": (ctypes.c_char_p, []),
+    "lng_hip_open": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_P)]),
+    "lng_hip_close": (None, [_P]),
+    "lng_hip_device_name": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.c_size_t]),
+    "lng_hip_buffer": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.POINTER(_P)]),
+    "lng_hip_resident": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.POINTER(_P)]),
+    "lng_hip_buffer_free": (ctypes.c_int, [_P]),
+    "lng_hip_buffer_len": (ctypes.c_size_t, [_P]),
+    "lng_hip_buffer_device_ptr": (_P, [_P]),
+    "lng_hip_upload": (ctypes.c_int, [_P, ctypes.c_size_t, _P, ctypes.c_size_t]),
+    "lng_hip_download": (ctypes.c_int, [_P, ctypes.c_size_t, _P, ctypes.c_size_t]),
+    "lng_hip_fill": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.c_int, ctypes.c_size_t]),
+    "lng_hip_batch": (ctypes.c_int, [_P, ctypes.POINTER(_P), ctypes.c_size_t, ctypes.POINTER(_P)]),
+    "lng_hip_batch_attach": (ctypes.c_int, [_P, _P, ctypes.POINTER(_Slice)]),
+    "lng_hip_batch_dispatches": (ctypes.c_size_t, [_P]),
+    "lng_hip_batch_barrier": (ctypes.c_int, [_P]),
+    "lng_hip_batch_commit": (ctypes.c_int, [_P, _ON_DONE, _P]),
+    "lng_hip_batch_wait": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_double)]),
+    "lng_hip_batch_drop": (None, [_P]),
+    "lng_hip_check_grouped": (ctypes.c_int, [ctypes.POINTER(_Shape), ctypes.c_int]),
+    "lng_hip_attention_grouped": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, ctypes.POINTER(_Slice),
+                                                 ctypes.POINTER(_Shape), ctypes.c_int]),
+    "lng_hip_attention_grouped_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, ctypes.POINTER(_Slice),
+                                                       ctypes.POINTER(_Shape), ctypes.c_int]),
+    "lng_hip_copy_rows": (ctypes.c_int, [_P, _Slice, _U64, ctypes.c_int, _Slice, _U64, ctypes.c_int, _U64, _U64]),
+    "lng_hip_attention_decode_batched": (ctypes.c_int, [_P, _U64, _U64, _U64, _U64, _U64, ctypes.POINTER(_Item),
+                                                        ctypes.c_size_t, _U64, _U64, _U64, ctypes.c_float,
+                                                        ctypes.c_int]),
+    "lng_hip_fill_synthetic": (ctypes.c_int, [_P, _Slice, ctypes.c_int, _U64, ctypes.c_float, _U64]),
+}
+
+_lib = None
+_lib_lock = threading.Lock()
+
+
+def library():
+    """The loaded C-ABI library. Raises ``Compile`` when it has not been built."""
+    global _lib
+    with _lib_lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise Compile("liblng_hip.so is not built: run `python -m loadngo_amd.build`")
+            lib = ctypes.CDLL(LIB_PATH)
+            for name, (restype, argtypes) in SYMBOLS.items():
+                fn = getattr(lib, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _lib = lib
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        message = library().lng_hip_last_error().decode("utf-8", "replace")
+        raise _ERRORS.get(rc, Error)(message)
+
+
+class Slice:
+    """apple.rs:507-521: bytes ``offset..offset+len`` of the batch's buffer number ``buffer``."""
+
+    __slots__ = ("buffer", "offset", "len")
+
+    def __init__(self, buffer, offset, len):
+        self.buffer, self.offset, self.len = buffer, offset, len
+
+    def _c(self):
+        return _Slice(self.buffer, self.offset, self.len)
+
+    def __repr__(self):
+        return "Slice(buffer=%d, offset=%d, len=%d)" % (self.buffer, self.offset, self.len)
+
+    def __eq__(self, other):
+        return (self.buffer, self.offset, self.len) == (other.buffer, other.offset, other.len)
+
+
+class GroupedShape:
+    """apple.rs:598-614."""
+
+    __slots__ = ("t", "start", "heads", "kv_heads", "dim", "window", "slots", "scale")
+
+    def __init__(self, t, start, heads, kv_heads, dim, window, slots, scale):
+        self.t, self.start, self.heads, self.kv_heads = t, start, heads, kv_heads
+        self.dim, self.window, self.slots, self.scale = dim, window, slots, scale
+
+    def _c(self):
+        return _Shape(self.t, self.start, self.heads, self.kv_heads, self.dim, self.window, self.slots, self.scale)
+
+    def __repr__(self):
+        return "GroupedShape(%s)" % ", ".join("%s=%r" % (n, getattr(self, n)) for n in self.__slots__)
+
+
+def check_grouped(shape, tiled=False):
+    """The shape rules alone (apple.rs:1243-1272, 1356-1385); raises ``Dispatch``. No device needed."""
+    _check(library().lng_hip_check_grouped(ctypes.byref(shape._c()), int(tiled)))
+
+
+class DecodeItem:
+    """One decoding query of a batched dispatch: byte offsets into the named buffers."""
+
+    __slots__ = ("q_offset", "out_offset", "k_offset", "v_offset", "sinks_offset", "start", "window", "slots")
+
+    def __init__(self, q_offset, out_offset, k_offset, v_offset, sinks_offset, start, window, slots):
+        self.q_offset, self.out_offset, self.k_offset, self.v_offset = q_offset, out_offset, k_offset, v_offset
+        self.sinks_offset = NO_SINKS if sinks_offset is None else sinks_offset
+        self.start, self.window, self.slots = start, window, slots
+
+
+class Completed:
+    """apple.rs:536-539: the batch's buffers, and the GPU time or why it failed."""
+
+    def __init__(self, buffers, gpu_time):
+        self.buffers = buffers
+        self.gpu_time = gpu_time  # seconds (float) or an Error instance
+
+
+class Buffer:
+    """apple.rs:391-430, in device memory."""
+
+    resident = False
+
+    def __init__(self, gpu, handle, len):
+        self._gpu, self._h, self.len = gpu, handle, len
+
+    def __len__(self):
+        return self.len
+
+    def device_ptr(self):
+        return library().lng_hip_buffer_device_ptr(self._h)
+
+    def write(self, array, offset=0):
+        """``as_bytes_mut()[offset..].copy_from_slice(array bytes)``."""
+        a = np.ascontiguousarray(array)
+        _check(library().lng_hip_upload(self._h, offset, a.ctypes.data_as(_P), a.nbytes))
+
+    def read(self, dtype=np.uint8, offset=0, count=None):
+        """``as_bytes()[offset..]`` viewed as ``dtype``."""
+        dtype = np.dtype(dtype)
+        nbytes = self.len - offset if count is None else count * dtype.itemsize
+        out = np.empty(nbytes // dtype.itemsize, dtype=dtype)
+        _check(library().lng_hip_download(self._h, offset, out.ctypes.data_as(_P), out.nbytes))
+        return out
+
+    def fill(self, byte, offset=0, len=None):
+        _check(library().lng_hip_fill(self._h, offset, byte, self.len - offset if len is None else len))
+
+    def free(self):
+        if self._h:
+            _check(library().lng_hip_buffer_free(self._h))
+            self._h = None
+
+    def __del__(self):
+        try:
+            if self._h and library():
+                library().lng_hip_buffer_free(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class Resident(Buffer):
+    """apple.rs:465-503: read-only memory that many batches may read at once."""
+
+    resident = True
+
+
+class Gpu:
+    """apple.rs:100-389."""
+
+    def __init__(self, device=0):
+        lib = library()
+        handle = _P()
+        _check(lib.lng_hip_open(device, ctypes.byref(handle)))
+        self._h = handle
+
+    @classmethod
+    def new(cls):
+        return cls()
+
+    def name(self):
+        buf = ctypes.create_string_buffer(128)
+        _check(library().lng_hip_device_name(self._h, buf, 128))
+        return buf.value.decode()
+
+    def buffer(self, len):
+        h = _P()
+        _check(library().lng_hip_buffer(self._h, len, ctypes.byref(h)))
+        return Buffer(self, h, len)
+
+    def resident(self, data):
+        a = np.ascontiguousarray(data)
+        h = _P()
+        _check(library().lng_hip_resident(self._h, a.ctypes.data_as(_P), a.nbytes, ctypes.byref(h)))
+        return Resident(self, h, a.nbytes)
+
+    def upload(self, array):
+        """A buffer holding ``array`` (the tests' ``upload`` helper, attention_grouped.rs:37-41)."""
+        a = np.ascontiguousarray(array)
+        b = self.buffer(max(a.nbytes, 4))
+        if a.nbytes:
+            b.write(a)
+        return b
+
+    def batch(self, buffers, dispatch="serial"):
+        return Batch(self, list(buffers))
+
+    def close(self):
+        if self._h:
+            library().lng_hip_close(self._h)
+            self._h = None
+
+
+class Batch:
+    """apple.rs:541-2240: one recorded submission. Dispatches run in order."""
+
+    def __init__(self, gpu, buffers):
+        self._gpu = gpu
+        self.buffers = buffers
+        self._residents = []
+        arr = (_P * max(len(buffers), 1))(*[b._h for b in buffers])
+        h = _P()
+        _check(library().lng_hip_batch(gpu._h, arr, len(buffers), ctypes.byref(h)))
+        self._h = h
+        self._callback = None
+        self._committed = False
+
+    def dispatches(self):
+        return library().lng_hip_batch_dispatches(self._h)
+
+    def attach(self, resident):
+        s = _Slice()
+        _check(library().lng_hip_batch_attach(self._h, resident._h, ctypes.byref(s)))
+        if resident not in self._residents:
+            self._residents.append(resident)
+        return Slice(s.buffer, s.offset, s.len)
+
+    def barrier(self):
+        _check(library().lng_hip_batch_barrier(self._h))
+
+    def attention_grouped(self, q, k, v, out, shape, dtype=F32):
+        _check(library().lng_hip_attention_grouped(self._h, q._c(), k._c(), v._c(), out._c(), None,
+                                                   ctypes.byref(shape._c()), dtype))
+
+    def attention_grouped_with_sinks(self, qkv, sinks, out, shape, dtype=F32):
+        q, k, v = qkv
+        _check(library().lng_hip_attention_grouped(self._h, q._c(), k._c(), v._c(), out._c(),
+                                                   ctypes.byref(sinks._c()), ctypes.byref(shape._c()), dtype))
+
+    def attention_grouped_tiled(self, q, k, v, out, shape, dtype=F32):
+        _check(library().lng_hip_attention_grouped_tiled(self._h, q._c(), k._c(), v._c(), out._c(), None,
+                                                         ctypes.byref(shape._c()), dtype))
+
+    def attention_grouped_tiled_with_sinks(self, qkv, sinks, out, shape, dtype=F32):
+        q, k, v = qkv
+        _check(library().lng_hip_attention_grouped_tiled(self._h, q._c(), k._c(), v._c(), out._c(),
+                                                         ctypes.byref(sinks._c()), ctypes.byref(shape._c()), dtype))
+
+    def copy_rows(self, src, dst, rows, width, src_dtype=F32, dst_dtype=None):
+        """``copy_rows((src, src_stride), (dst, dst_stride), rows, width)`` (apple.rs:1762)."""
+        (s, s_stride), (d, d_stride) = src, dst
+        dst_dtype = src_dtype if dst_dtype is None else dst_dtype
+        _check(library().lng_hip_copy_rows(self._h, s._c(), s_stride, src_dtype, d._c(), d_stride, dst_dtype,
+                                           rows, width))
+
+    def attention_decode_batched(self, q_buffer, k_buffer, v_buffer, out_buffer, sinks_buffer, items, heads,
+                                 kv_heads, dim, scale, dtype=BF16):
+        arr = (_Item * len(items))(*[
+            _Item(i.q_offset, i.out_offset, i.k_offset, i.v_offset, i.sinks_offset, i.start, i.window, i.slots)
+            for i in items])
+        _check(library().lng_hip_attention_decode_batched(self._h, q_buffer, k_buffer, v_buffer, out_buffer,
+                                                          sinks_buffer, arr, len(items), heads, kv_heads, dim,
+                                                          scale, dtype))
+
+    def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
+        _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))
+
+    def commit(self, on_done=None):
+        """apple.rs:2202: submits; ``on_done(Completed)`` runs on a library thread when the GPU
+        has finished (a Rust caller re-posts it to its proactor)."""
+        if on_done is not None:
+            def trampoline(done, _user):
+                d = done.contents
+                if d.status == 0:
+                    gpu_time = d.gpu_seconds
+                else:
+                    gpu_time = _ERRORS.get(d.status, Error)((d.message or b"").decode("utf-8", "replace"))
+                on_done(Completed(self.buffers, gpu_time))
+            self._callback = _ON_DONE(trampoline)
+        else:
+            self._callback = ctypes.cast(None, _ON_DONE)
+        self._committed = True
+        _check(library().lng_hip_batch_commit(self._h, self._callback, None))
+
+    def wait(self):
+        """Blocks until a committed batch has finished; returns ``Completed``."""
+        seconds = ctypes.c_double()
+        rc = library().lng_hip_batch_wait(self._h, ctypes.byref(seconds))
+        if rc == -5:
+            return Completed(self.buffers, GpuFailure(library().lng_hip_last_error().decode()))
+        _check(rc)
+        return Completed(self.buffers, seconds.value)
+
+    def run(self):
+        """commit + wait: what the reference's tests do with their proactor loop
+        (attention_grouped.rs:11-23)."""
+        self.commit()
+        return self.wait()
+
+    def drop(self):
+        if self._h:
+            library().lng_hip_batch_drop(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.drop()
+        except Exception:
+            pass

@@ -1,0 +1,951 @@
+// Host side of liblng_hip.so: the C ABI declared in include/lng_hip.h.
+//
+// Plain HIP driver-style calls only (hipMalloc, hipModuleLoadData, hipModuleLaunchKernel,
+// events): the gfx950 code object built from lng_kernels.hip is embedded in this library.
+// A batch records dispatches on the host and submits them in order on one stream at
+// commit, so an uncommitted batch runs nothing (metal-compute/src/apple.rs:553-561) and a
+// refused dispatch leaves nothing behind (apple.rs:1243-1256 run before any encoding).
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <atomic>
+#include <condition_variable>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <deque>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "lng_kernel_args.h"
+
+// The code object, placed in .rodata by the assembler (path given by the build).
+#ifndef LNG_HSACO_PATH
+#error "LNG_HSACO_PATH must name the gfx950 code object to embed"
+#endif
+__asm__(".section .rodata\n"
+        ".balign 4096\n"
+        ".global lng_hsaco_begin\n"
+        "lng_hsaco_begin:\n"
+        ".incbin \"" LNG_HSACO_PATH "\"\n"
+        ".global lng_hsaco_end\n"
+        "lng_hsaco_end:\n"
+        ".byte 0\n"
+        ".previous\n");
+extern "C" const char lng_hsaco_begin[];
+extern "C" const char lng_hsaco_end[];
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char *fmt, ...) {
+    char text[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(text, sizeof text, fmt, ap);
+    va_end(ap);
+    g_error = text;
+    return code;
+}
+
+const char *hip_text(hipError_t e) { return hipGetErrorString(e); }
+
+size_t elem_size(int dtype) { return dtype == LNG_BF16 ? 2 : 4; }
+
+struct Table { // one pinned-host / device pair holding row tables of batched dispatches
+    char *host = nullptr;
+    char *dev = nullptr;
+    size_t cap = 0;
+    size_t used = 0;
+};
+
+struct Cmd {
+    hipFunction_t fn = nullptr;
+    unsigned grid[3] = {1, 1, 1};
+    unsigned block = 256;
+    std::vector<char> args;
+    // optional host->device copy enqueued before the launch (row tables)
+    const void *copy_src = nullptr;
+    void *copy_dst = nullptr;
+    size_t copy_len = 0;
+};
+
+} // namespace
+
+struct lng_buffer {
+    lng_gpu *gpu = nullptr;
+    void *ptr = nullptr;
+    size_t len = 0;
+    bool resident = false;
+    std::atomic<int> holds{0}; // batches owning (buffer) or having attached (resident) it
+};
+
+struct lng_gpu {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipModule_t module = nullptr;
+    hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
+                  decode_combine = nullptr, prefill_bf16_d64 = nullptr, copy_rows = nullptr,
+                  fill_synthetic = nullptr;
+    std::string name;
+    unsigned cus = 256;
+
+    std::mutex mu;
+    std::vector<Table> free_tables;
+    float *scratch_o = nullptr;  // split-K partial outputs, grown on demand
+    float *scratch_ml = nullptr; // split-K partial (max, sum)
+    size_t scratch_o_len = 0, scratch_ml_len = 0;
+    std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
+    std::atomic<long> live_buffers{0};
+    unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
+
+    // completion thread (only for batches committed with a callback)
+    std::thread worker;
+    std::mutex qmu;
+    std::condition_variable qcv;
+    std::deque<lng_batch *> queue;
+    bool stopping = false;
+};
+
+struct lng_batch {
+    lng_gpu *gpu = nullptr;
+    std::vector<lng_buffer *> buffers;
+    std::vector<lng_buffer *> residents;
+    std::vector<Cmd> cmds;
+    std::vector<Table> tables;
+    size_t dispatches = 0;
+    enum State { Recording, Committed, Done } state = Recording;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    lng_on_done on_done = nullptr;
+    void *user = nullptr;
+    int status = LNG_OK;
+    double seconds = 0.0;
+    std::string message;
+    std::mutex mu;
+    std::condition_variable cv;
+    bool released = false;
+};
+
+namespace {
+
+struct Operand { // a checked slice resolved to its buffer
+    lng_buffer *buf;
+    uint64_t index;
+    uint64_t offset;
+    uint64_t len;
+};
+
+lng_buffer *buffer_at(lng_batch *b, uint64_t index) {
+    if (index < b->buffers.size()) return b->buffers[index];
+    index -= b->buffers.size();
+    if (index < b->residents.size()) return b->residents[index];
+    return nullptr;
+}
+
+// apple.rs:860-887 Batch::check
+int check_slice(lng_batch *b, const char *what, const lng_slice &s, uint64_t len, uint64_t align,
+                Operand *out) {
+    lng_buffer *buf = buffer_at(b, s.buffer);
+    if (!buf) {
+        return fail(LNG_ERR_DISPATCH, "%s: no buffer %llu (batch has %zu)", what,
+                    (unsigned long long)s.buffer, b->buffers.size() + b->residents.size());
+    }
+    if (s.len != len) {
+        return fail(LNG_ERR_DISPATCH, "%s: %llu bytes, the shape needs %llu", what,
+                    (unsigned long long)s.len, (unsigned long long)len);
+    }
+    if (s.offset > buf->len || s.len > buf->len - s.offset) {
+        return fail(LNG_ERR_DISPATCH, "%s: bytes %llu..%llu outside a %zu-byte buffer", what,
+                    (unsigned long long)s.offset, (unsigned long long)(s.offset + s.len), buf->len);
+    }
+    if (s.offset % align != 0) {
+        return fail(LNG_ERR_DISPATCH, "%s: offset %llu is not a multiple of %llu", what,
+                    (unsigned long long)s.offset, (unsigned long long)align);
+    }
+    *out = Operand{buf, s.buffer, s.offset, s.len};
+    return LNG_OK;
+}
+
+bool overlaps(const Operand &a, const Operand &b) {
+    return a.index == b.index && a.offset < b.offset + b.len && b.offset < a.offset + a.len;
+}
+
+// apple.rs:889-906 Batch::check_output
+int check_output(lng_batch *b, const Operand &y, std::initializer_list<const Operand *> inputs) {
+    if (y.index >= b->buffers.size()) {
+        return fail(LNG_ERR_DISPATCH, "output is in read-only resident memory");
+    }
+    for (const Operand *in : inputs) {
+        if (overlaps(y, *in)) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+    }
+    return LNG_OK;
+}
+
+std::string shape_text(const lng_grouped_shape &s) {
+    char text[256];
+    snprintf(text, sizeof text,
+             "GroupedShape { t: %llu, start: %llu, heads: %llu, kv_heads: %llu, dim: %llu, window: %llu, "
+             "slots: %llu, scale: %g }",
+             (unsigned long long)s.t, (unsigned long long)s.start, (unsigned long long)s.heads,
+             (unsigned long long)s.kv_heads, (unsigned long long)s.dim, (unsigned long long)s.window,
+             (unsigned long long)s.slots, (double)s.scale);
+    return text;
+}
+
+bool fits_u32(uint64_t n) { return n <= 0xffffffffull; }
+
+// apple.rs:1243-1272 (plain) and 1356-1385 (tiled)
+int check_shape(const lng_grouped_shape &s, bool tiled) {
+    const uint64_t end = s.start + s.t;
+    const uint64_t need = s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t;
+    const bool ring = s.slots < end;
+    bool bad = s.t == 0 || s.kv_heads == 0 || (s.kv_heads && s.heads % s.kv_heads != 0) || s.dim == 0 ||
+               s.dim > 512 || s.window == 0 || s.slots == 0 || end < s.start;
+    if (!tiled) {
+        bad = bad || s.dim % 32 != 0 || (ring && s.slots < need);
+    } else {
+        bad = bad || s.dim % 16 != 0 || (ring && (s.slots % 32 != 0 || s.slots < need));
+    }
+    if (bad) {
+        return fail(LNG_ERR_DISPATCH, "unsupported %sgrouped attention shape %s", tiled ? "tiled " : "",
+                    shape_text(s).c_str());
+    }
+    const uint64_t window = std::min(s.window, end);
+    const uint64_t groups = tiled ? (s.t + 31) / 32 * s.heads : s.t * s.heads;
+    for (uint64_t n : {s.t, s.start, s.heads, s.kv_heads, s.dim, window, s.slots, groups}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (s.heads == 0) return fail(LNG_ERR_DISPATCH, "unsupported grouped attention shape %s", shape_text(s).c_str());
+    return LNG_OK;
+}
+
+int need_recording(lng_batch *b) {
+    if (!b) return fail(LNG_ERR_DISPATCH, "no batch");
+    if (b->state != lng_batch::Recording) return fail(LNG_ERR_DISPATCH, "the batch was already committed");
+    return LNG_OK;
+}
+
+template <typename A> void set_args(Cmd &c, const A &a) {
+    c.args.resize(sizeof(A));
+    memcpy(c.args.data(), &a, sizeof(A));
+}
+
+// Device scratch for split-K partials, shared by every dispatch of the gpu: dispatches run
+// in order on one stream, so the next one starts after the previous combine has read it.
+int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats) {
+    std::lock_guard<std::mutex> lock(g->mu);
+    if (o_floats > g->scratch_o_len) {
+        void *p = nullptr;
+        const size_t want = std::max(o_floats, g->scratch_o_len * 2);
+        if (hipMalloc(&p, want * sizeof(float)) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte scratch buffer", want * sizeof(float));
+        if (g->scratch_o) g->retired.push_back(g->scratch_o);
+        g->scratch_o = (float *)p;
+        g->scratch_o_len = want;
+    }
+    if (ml_floats > g->scratch_ml_len) {
+        void *p = nullptr;
+        const size_t want = std::max(ml_floats, g->scratch_ml_len * 2);
+        if (hipMalloc(&p, want * sizeof(float)) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte scratch buffer", want * sizeof(float));
+        if (g->scratch_ml) g->retired.push_back(g->scratch_ml);
+        g->scratch_ml = (float *)p;
+        g->scratch_ml_len = want;
+    }
+    return LNG_OK;
+}
+
+// Space for a row table: pinned host memory now, its device twin filled at commit.
+int reserve_table(lng_batch *b, size_t bytes, char **host, char **dev) {
+    lng_gpu *g = b->gpu;
+    if (b->tables.empty() || b->tables.back().cap - b->tables.back().used < bytes) {
+        Table t;
+        {
+            std::lock_guard<std::mutex> lock(g->mu);
+            for (size_t i = 0; i < g->free_tables.size(); ++i) {
+                if (g->free_tables[i].cap >= bytes) {
+                    t = g->free_tables[i];
+                    g->free_tables.erase(g->free_tables.begin() + i);
+                    break;
+                }
+            }
+        }
+        if (!t.host) {
+            t.cap = std::max<size_t>(bytes, 64 * 1024);
+            if (hipHostMalloc((void **)&t.host, t.cap, hipHostMallocDefault) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte pinned table", t.cap);
+            if (hipMalloc((void **)&t.dev, t.cap) != hipSuccess) {
+                hipHostFree(t.host);
+                return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte device table", t.cap);
+            }
+        }
+        t.used = 0;
+        b->tables.push_back(t);
+    }
+    Table &t = b->tables.back();
+    *host = t.host + t.used;
+    *dev = t.dev + t.used;
+    t.used += (bytes + 255) / 256 * 256;
+    if (t.used > t.cap) t.used = t.cap;
+    return LNG_OK;
+}
+
+void release(lng_batch *b) { // buffers and tables go back; idempotent
+    if (b->released) return;
+    b->released = true;
+    for (lng_buffer *buf : b->buffers) buf->holds.fetch_sub(1);
+    for (lng_buffer *buf : b->residents) buf->holds.fetch_sub(1);
+    std::lock_guard<std::mutex> lock(b->gpu->mu);
+    for (Table &t : b->tables) b->gpu->free_tables.push_back(t);
+    b->tables.clear();
+}
+
+// Waits for the GPU, fills status/seconds, hands the buffers back. Called once per batch.
+void finish(lng_batch *b) {
+    hipSetDevice(b->gpu->device);
+    hipError_t e = hipEventSynchronize(b->ev1);
+    if (e == hipSuccess) {
+        float ms = 0.0f;
+        e = hipEventElapsedTime(&ms, b->ev0, b->ev1);
+        if (e == hipSuccess) b->seconds = std::max(0.0, (double)ms * 1e-3);
+    }
+    if (e != hipSuccess) {
+        b->status = LNG_ERR_GPU;
+        b->message = hip_text(e);
+    }
+    release(b);
+}
+
+void worker_loop(lng_gpu *g) {
+    for (;;) {
+        lng_batch *b = nullptr;
+        {
+            std::unique_lock<std::mutex> lock(g->qmu);
+            g->qcv.wait(lock, [&] { return g->stopping || !g->queue.empty(); });
+            if (g->queue.empty()) return;
+            b = g->queue.front();
+            g->queue.pop_front();
+        }
+        finish(b);
+        if (b->on_done) {
+            lng_completed done{b->status, b->seconds, b->message.c_str()};
+            b->on_done(&done, b->user);
+        }
+        {
+            std::lock_guard<std::mutex> lock(b->mu);
+            b->state = lng_batch::Done;
+        }
+        b->cv.notify_all();
+    }
+}
+
+// Rows of one dispatch, and how to split them over workgroups.
+struct DecodePlan {
+    uint32_t chunk = 128;
+    uint32_t n_chunks = 1;
+};
+
+uint64_t visible_from_tile(const lng_k_row &r) { // positions from the tile-aligned window start
+    const uint64_t last = r.start;
+    const uint64_t first = (r.window != LNG_WINDOW_FULL && last + 1 > r.window) ? last + 1 - r.window : 0;
+    return last + 1 - (first & ~(uint64_t)31);
+}
+
+DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_uniform, uint32_t kv_heads) {
+    // rows == the table, or one row standing for t_uniform consecutive queries of one cache
+    uint64_t total = 0, longest = 0;
+    if (t_uniform) {
+        for (uint64_t i = 0; i < t_uniform; ++i) {
+            lng_k_row r = rows[0];
+            r.start += i;
+            const uint64_t v = visible_from_tile(r);
+            total += v;
+            longest = std::max(longest, v);
+        }
+    } else {
+        for (size_t i = 0; i < n; ++i) {
+            const uint64_t v = visible_from_tile(rows[i]);
+            total += v;
+            longest = std::max(longest, v);
+        }
+    }
+    DecodePlan p;
+    const uint64_t per_wg = (total * kv_heads + g->decode_wgs - 1) / g->decode_wgs;
+    uint64_t chunk = (per_wg + 127) / 128 * 128;
+    chunk = std::max<uint64_t>(chunk, 128);
+    chunk = std::min<uint64_t>(chunk, 1u << 20);
+    p.chunk = (uint32_t)chunk;
+    p.n_chunks = (uint32_t)((longest + chunk - 1) / chunk);
+    return p;
+}
+
+// Records the kernels for a set of single-query rows (decode, and short passes row by row).
+int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n_rows, uint64_t t_uniform,
+                bool aligned16) {
+    lng_gpu *g = b->gpu;
+    const uint32_t group = a.heads / a.kv_heads;
+    const bool fast = a.dtype == LNG_BF16 && a.dim == 64 && group <= 16 && aligned16;
+    if (!fast) {
+        Cmd c;
+        c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;
+        c.grid[0] = (unsigned)(n_rows * a.heads);
+        c.block = 256;
+        set_args(c, a);
+        if (a.rows) { // table upload rides on the first command
+            c.copy_src = host_rows;
+            c.copy_dst = (void *)a.rows;
+            c.copy_len = n_rows * sizeof(lng_k_row);
+        }
+        b->cmds.push_back(std::move(c));
+        return LNG_OK;
+    }
+    const DecodePlan plan = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads);
+    a.chunk = plan.chunk;
+    a.n_chunks = plan.n_chunks;
+    if (plan.n_chunks > 1) {
+        const size_t slots = n_rows * a.kv_heads * (size_t)plan.n_chunks * group;
+        if (int rc = reserve_scratch(g, slots * 64, slots * 2)) return rc;
+        a.partial_o = g->scratch_o;
+        a.partial_ml = g->scratch_ml;
+    }
+    Cmd c;
+    c.fn = g->decode_bf16_d64;
+    c.grid[0] = plan.n_chunks;
+    c.grid[1] = (unsigned)(n_rows * a.kv_heads);
+    c.block = 256;
+    set_args(c, a);
+    if (a.rows) {
+        c.copy_src = host_rows;
+        c.copy_dst = (void *)a.rows;
+        c.copy_len = n_rows * sizeof(lng_k_row);
+    }
+    b->cmds.push_back(std::move(c));
+    if (plan.n_chunks > 1) {
+        Cmd m;
+        m.fn = g->decode_combine;
+        m.grid[0] = (unsigned)(n_rows * a.heads);
+        m.block = 64;
+        set_args(m, a);
+        b->cmds.push_back(std::move(m));
+    }
+    return LNG_OK;
+}
+
+int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out, const lng_slice *sinks,
+              const lng_grouped_shape *shape, int dtype, bool tiled) {
+    if (int rc = need_recording(b)) return rc;
+    if (!shape) return fail(LNG_ERR_DISPATCH, "no shape");
+    if (dtype != LNG_F32 && dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", dtype);
+    const lng_grouped_shape &s = *shape;
+    if (int rc = check_shape(s, tiled)) return rc;
+    const uint64_t es = elem_size(dtype);
+    const uint64_t end = s.start + s.t;
+    uint64_t q_rows, kv_rows;
+    if (!tiled) {
+        q_rows = s.t; // apple.rs:1273-1277
+        kv_rows = std::min(s.slots, end);
+    } else {
+        q_rows = (s.t + 31) / 32 * 32; // apple.rs:1386-1395
+        kv_rows = s.slots < end ? s.slots : (end + 31) / 32 * 32;
+    }
+    Operand oq, ok, ov, oo, os{};
+    if (int rc = check_slice(b, "q", q, q_rows * s.heads * s.dim * es, es, &oq)) return rc;
+    if (int rc = check_slice(b, "k", k, kv_rows * s.kv_heads * s.dim * es, es, &ok)) return rc;
+    if (int rc = check_slice(b, "v", v, kv_rows * s.kv_heads * s.dim * es, es, &ov)) return rc;
+    if (int rc = check_slice(b, "out", out, q_rows * s.heads * s.dim * es, es, &oo)) return rc;
+    if (int rc = check_output(b, oo, {&oq, &ok, &ov})) return rc;
+    if (sinks) {
+        if (int rc = check_slice(b, "sinks", *sinks, s.heads * 4, 4, &os)) return rc;
+    }
+    lng_gpu *g = b->gpu;
+    const bool aligned16 = ((q.offset | k.offset | v.offset | out.offset) & 15u) == 0;
+
+    if (tiled && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 16 && aligned16 && g->prefill_bf16_d64) {
+        lng_k_prefill p{};
+        p.q = (const char *)oq.buf->ptr + q.offset;
+        p.k = (const char *)ok.buf->ptr + k.offset;
+        p.v = (const char *)ov.buf->ptr + v.offset;
+        p.out = (char *)oo.buf->ptr + out.offset;
+        p.sinks = sinks ? (const float *)((const char *)os.buf->ptr + sinks->offset) : nullptr;
+        p.t = s.t;
+        p.start = s.start;
+        p.window = s.window;
+        p.slots = s.slots;
+        p.heads = (uint32_t)s.heads;
+        p.kv_heads = (uint32_t)s.kv_heads;
+        p.dim = (uint32_t)s.dim;
+        p.q_tiles = (uint32_t)((s.t + 127) / 128);
+        p.scale = s.scale;
+        Cmd c;
+        c.fn = g->prefill_bf16_d64;
+        c.grid[0] = p.q_tiles;
+        c.grid[1] = (unsigned)s.kv_heads;
+        c.block = 256;
+        set_args(c, p);
+        b->cmds.push_back(std::move(c));
+        b->dispatches += 1;
+        return LNG_OK;
+    }
+
+    lng_k_attn a{};
+    a.q = (const char *)oq.buf->ptr;
+    a.k = (const char *)ok.buf->ptr;
+    a.v = (const char *)ov.buf->ptr;
+    a.out = (char *)oo.buf->ptr;
+    a.sinks = sinks ? (const char *)os.buf->ptr : nullptr;
+    a.rows = nullptr;
+    a.first.q_offset = q.offset;
+    a.first.out_offset = out.offset;
+    a.first.k_offset = k.offset;
+    a.first.v_offset = v.offset;
+    a.first.sinks_offset = sinks ? sinks->offset : LNG_NO_SINKS;
+    a.first.start = s.start;
+    a.first.window = s.window;
+    a.first.slots = s.slots;
+    a.n_rows = (uint32_t)s.t;
+    a.heads = (uint32_t)s.heads;
+    a.kv_heads = (uint32_t)s.kv_heads;
+    a.dim = (uint32_t)s.dim;
+    a.chunk = 128;
+    a.n_chunks = 1;
+    a.dtype = (uint32_t)dtype;
+    a.scale = s.scale;
+    if (int rc = record_rows(b, a, &a.first, s.t, s.t, aligned16)) return rc;
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+} // namespace
+
+// ================================== C ABI =====================================================
+
+extern "C" const char *lng_hip_last_error(void) { return g_error.c_str(); }
+
+extern "C" int lng_hip_open(int device, lng_gpu **out) {
+    if (!out) return fail(LNG_ERR_DISPATCH, "no place for the gpu handle");
+    *out = nullptr;
+    int count = 0;
+    if (hipInit(0) != hipSuccess || hipGetDeviceCount(&count) != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(LNG_ERR_NO_DEVICE, "no HIP device");
+    }
+    if (device < 0 || device >= count) return fail(LNG_ERR_NO_DEVICE, "no HIP device %d (%d present)", device, count);
+    if (hipSetDevice(device) != hipSuccess) return fail(LNG_ERR_NO_DEVICE, "cannot select HIP device %d", device);
+    lng_gpu *g = new lng_gpu;
+    g->device = device;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
+        g->name = prop.gcnArchName;
+        g->cus = (unsigned)prop.multiProcessorCount;
+    }
+    hipError_t e = hipModuleLoadData(&g->module, lng_hsaco_begin);
+    if (e != hipSuccess) {
+        const int rc = fail(LNG_ERR_COMPILE, "the gfx950 code object does not load on %s: %s", g->name.c_str(), hip_text(e));
+        delete g;
+        return rc;
+    }
+    struct { const char *name; hipFunction_t *fn; bool required; } wanted[] = {
+        {"lng_attn_generic_f32", &g->generic_f32, true},
+        {"lng_attn_generic_bf16", &g->generic_bf16, true},
+        {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
+        {"lng_decode_combine", &g->decode_combine, true},
+        {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, false},
+        {"lng_copy_rows", &g->copy_rows, true},
+        {"lng_fill_synthetic", &g->fill_synthetic, true},
+    };
+    for (auto &w : wanted) {
+        e = hipModuleGetFunction(w.fn, g->module, w.name);
+        if (e != hipSuccess && w.required) {
+            const int rc = fail(LNG_ERR_COMPILE, "kernel %s missing: %s", w.name, hip_text(e));
+            hipModuleUnload(g->module);
+            delete g;
+            return rc;
+        }
+    }
+    if (hipStreamCreateWithFlags(&g->stream, hipStreamNonBlocking) != hipSuccess) {
+        hipModuleUnload(g->module);
+        delete g;
+        return fail(LNG_ERR_NO_DEVICE, "cannot create a stream");
+    }
+    if (const char *env = getenv("LNG_DECODE_WGS")) {
+        const long n = atol(env);
+        if (n >= 1 && n <= (1 << 20)) g->decode_wgs = (unsigned)n;
+    }
+    *out = g;
+    return LNG_OK;
+}
+
+extern "C" void lng_hip_close(lng_gpu *g) {
+    if (!g) return;
+    hipSetDevice(g->device);
+    if (g->worker.joinable()) {
+        {
+            std::lock_guard<std::mutex> lock(g->qmu);
+            g->stopping = true;
+        }
+        g->qcv.notify_all();
+        g->worker.join();
+    }
+    hipStreamSynchronize(g->stream);
+    for (Table &t : g->free_tables) {
+        hipHostFree(t.host);
+        hipFree(t.dev);
+    }
+    for (void *p : g->retired) hipFree(p);
+    if (g->scratch_o) hipFree(g->scratch_o);
+    if (g->scratch_ml) hipFree(g->scratch_ml);
+    hipStreamDestroy(g->stream);
+    hipModuleUnload(g->module);
+    delete g;
+}
+
+extern "C" int lng_hip_device_name(lng_gpu *g, char *name, size_t cap) {
+    if (!g || !name || cap == 0) return fail(LNG_ERR_DISPATCH, "no gpu or no room for the name");
+    snprintf(name, cap, "%s", g->name.c_str());
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_buffer(lng_gpu *g, size_t len, lng_buffer **out) {
+    if (!g || !out) return fail(LNG_ERR_DISPATCH, "no gpu");
+    *out = nullptr;
+    if (len == 0) return fail(LNG_ERR_ALLOC, "could not allocate a 0-byte buffer");
+    hipSetDevice(g->device);
+    void *p = nullptr;
+    if (hipMalloc(&p, len) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte buffer", len);
+    }
+    lng_buffer *b = new lng_buffer;
+    b->gpu = g;
+    b->ptr = p;
+    b->len = len;
+    g->live_buffers.fetch_add(1);
+    *out = b;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_resident(lng_gpu *g, const void *bytes, size_t len, lng_buffer **out) {
+    if (!bytes && len) return fail(LNG_ERR_DISPATCH, "no bytes");
+    if (int rc = lng_hip_buffer(g, len, out)) return rc;
+    if (hipMemcpy((*out)->ptr, bytes, len, hipMemcpyHostToDevice) != hipSuccess) {
+        lng_hip_buffer_free(*out);
+        *out = nullptr;
+        return fail(LNG_ERR_GPU, "could not fill a %zu-byte resident", len);
+    }
+    (*out)->resident = true;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_buffer_free(lng_buffer *b) {
+    if (!b) return LNG_OK;
+    if (b->holds.load() != 0) return fail(LNG_ERR_DISPATCH, "the buffer belongs to a batch that has not finished");
+    hipSetDevice(b->gpu->device);
+    hipFree(b->ptr);
+    b->gpu->live_buffers.fetch_sub(1);
+    delete b;
+    return LNG_OK;
+}
+
+extern "C" size_t lng_hip_buffer_len(const lng_buffer *b) { return b ? b->len : 0; }
+
+extern "C" void *lng_hip_buffer_device_ptr(lng_buffer *b) { return b ? b->ptr : nullptr; }
+
+static int host_access(lng_buffer *b, size_t offset, size_t len, bool write) {
+    if (!b) return fail(LNG_ERR_DISPATCH, "no buffer");
+    if (write && b->resident) return fail(LNG_ERR_DISPATCH, "resident memory is read-only");
+    if (!b->resident && b->holds.load() != 0) return fail(LNG_ERR_DISPATCH, "the buffer belongs to a batch that has not finished");
+    if (offset > b->len || len > b->len - offset) return fail(LNG_ERR_DISPATCH, "bytes %zu..%zu outside a %zu-byte buffer", offset, offset + len, b->len);
+    hipSetDevice(b->gpu->device);
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_upload(lng_buffer *b, size_t offset, const void *src, size_t len) {
+    if (int rc = host_access(b, offset, len, true)) return rc;
+    if (len == 0) return LNG_OK;
+    const hipError_t e = hipMemcpy((char *)b->ptr + offset, src, len, hipMemcpyHostToDevice);
+    return e == hipSuccess ? LNG_OK : fail(LNG_ERR_GPU, "upload failed: %s", hip_text(e));
+}
+
+extern "C" int lng_hip_download(lng_buffer *b, size_t offset, void *dst, size_t len) {
+    if (int rc = host_access(b, offset, len, false)) return rc;
+    if (len == 0) return LNG_OK;
+    const hipError_t e = hipMemcpy(dst, (const char *)b->ptr + offset, len, hipMemcpyDeviceToHost);
+    return e == hipSuccess ? LNG_OK : fail(LNG_ERR_GPU, "download failed: %s", hip_text(e));
+}
+
+extern "C" int lng_hip_fill(lng_buffer *b, size_t offset, int byte, size_t len) {
+    if (int rc = host_access(b, offset, len, true)) return rc;
+    if (len == 0) return LNG_OK;
+    hipError_t e = hipMemset((char *)b->ptr + offset, byte, len);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    return e == hipSuccess ? LNG_OK : fail(LNG_ERR_GPU, "fill failed: %s", hip_text(e));
+}
+
+extern "C" int lng_hip_batch(lng_gpu *g, lng_buffer *const *buffers, size_t n, lng_batch **out) {
+    if (!g || !out || (n && !buffers)) return fail(LNG_ERR_DISPATCH, "no gpu or no buffers");
+    *out = nullptr;
+    for (size_t i = 0; i < n; ++i) {
+        if (!buffers[i] || buffers[i]->gpu != g) return fail(LNG_ERR_DISPATCH, "buffer %zu is not of this gpu", i);
+        if (buffers[i]->resident) return fail(LNG_ERR_DISPATCH, "buffer %zu is resident memory: attach it instead", i);
+        for (size_t j = 0; j < i; ++j) {
+            if (buffers[j] == buffers[i]) return fail(LNG_ERR_DISPATCH, "buffer %zu is given twice", i);
+        }
+    }
+    // take ownership of all or none
+    size_t taken = 0;
+    for (; taken < n; ++taken) {
+        int expected = 0;
+        if (!buffers[taken]->holds.compare_exchange_strong(expected, 1)) break;
+    }
+    if (taken < n) {
+        for (size_t i = 0; i < taken; ++i) buffers[i]->holds.store(0);
+        return fail(LNG_ERR_DISPATCH, "buffer %zu belongs to a batch that has not finished", taken);
+    }
+    lng_batch *b = new lng_batch;
+    b->gpu = g;
+    b->buffers.assign(buffers, buffers + n);
+    *out = b;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_batch_attach(lng_batch *b, lng_buffer *resident, lng_slice *whole) {
+    if (int rc = need_recording(b)) return rc;
+    if (!resident || !whole) return fail(LNG_ERR_DISPATCH, "no resident");
+    if (!resident->resident || resident->gpu != b->gpu) return fail(LNG_ERR_DISPATCH, "not a resident of this gpu");
+    size_t index = 0;
+    for (; index < b->residents.size(); ++index) {
+        if (b->residents[index] == resident) break;
+    }
+    if (index == b->residents.size()) {
+        resident->holds.fetch_add(1);
+        b->residents.push_back(resident);
+    }
+    *whole = lng_slice{b->buffers.size() + index, 0, resident->len};
+    return LNG_OK;
+}
+
+extern "C" size_t lng_hip_batch_dispatches(const lng_batch *b) { return b ? b->dispatches : 0; }
+
+extern "C" int lng_hip_batch_barrier(lng_batch *b) { return need_recording(b); }
+
+extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *user) {
+    if (int rc = need_recording(b)) return rc;
+    lng_gpu *g = b->gpu;
+    hipSetDevice(g->device);
+    hipError_t e = hipEventCreate(&b->ev0);
+    if (e == hipSuccess) e = hipEventCreate(&b->ev1);
+    if (e == hipSuccess) e = hipEventRecord(b->ev0, g->stream);
+    for (size_t i = 0; e == hipSuccess && i < b->cmds.size(); ++i) {
+        Cmd &c = b->cmds[i];
+        if (c.copy_len) {
+            e = hipMemcpyAsync(c.copy_dst, c.copy_src, c.copy_len, hipMemcpyHostToDevice, g->stream);
+            if (e != hipSuccess) break;
+        }
+        size_t size = c.args.size();
+        void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, c.args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                          HIP_LAUNCH_PARAM_END};
+        e = hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block, 1, 1, 0, g->stream, nullptr, config);
+    }
+    if (e == hipSuccess) e = hipEventRecord(b->ev1, g->stream);
+    b->on_done = on_done;
+    b->user = user;
+    b->state = lng_batch::Committed;
+    if (e != hipSuccess) {
+        // What was submitted before the failure still runs; wait for it, then report.
+        hipStreamSynchronize(g->stream);
+        b->status = LNG_ERR_GPU;
+        b->message = hip_text(e);
+        release(b);
+        b->state = lng_batch::Done;
+        if (on_done) {
+            lng_completed done{b->status, 0.0, b->message.c_str()};
+            on_done(&done, user);
+        }
+        return fail(LNG_ERR_GPU, "submission failed: %s", b->message.c_str());
+    }
+    if (on_done) {
+        std::lock_guard<std::mutex> lock(g->qmu);
+        if (!g->worker.joinable()) g->worker = std::thread(worker_loop, g);
+        g->queue.push_back(b);
+        g->qcv.notify_one();
+    }
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_batch_wait(lng_batch *b, double *gpu_seconds) {
+    if (!b) return fail(LNG_ERR_DISPATCH, "no batch");
+    if (b->state == lng_batch::Recording) return fail(LNG_ERR_DISPATCH, "the batch was not committed");
+    if (b->on_done) { // the completion thread finishes it
+        std::unique_lock<std::mutex> lock(b->mu);
+        b->cv.wait(lock, [&] { return b->state == lng_batch::Done; });
+    } else if (b->state != lng_batch::Done) {
+        finish(b);
+        b->state = lng_batch::Done;
+    }
+    if (gpu_seconds) *gpu_seconds = b->seconds;
+    if (b->status != LNG_OK) return fail(b->status, "the batch failed on the GPU: %s", b->message.c_str());
+    return LNG_OK;
+}
+
+extern "C" void lng_hip_batch_drop(lng_batch *b) {
+    if (!b) return;
+    if (b->state == lng_batch::Recording) {
+        release(b);
+    } else {
+        lng_hip_batch_wait(b, nullptr);
+    }
+    if (b->ev0) hipEventDestroy(b->ev0);
+    if (b->ev1) hipEventDestroy(b->ev1);
+    delete b;
+}
+
+extern "C" int lng_hip_check_grouped(const lng_grouped_shape *shape, int tiled) {
+    if (!shape) return fail(LNG_ERR_DISPATCH, "no shape");
+    return check_shape(*shape, tiled != 0);
+}
+
+extern "C" int lng_hip_attention_grouped(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out,
+                                         const lng_slice *sinks, const lng_grouped_shape *shape, int dtype) {
+    return attention(b, q, k, v, out, sinks, shape, dtype, false);
+}
+
+extern "C" int lng_hip_attention_grouped_tiled(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out,
+                                               const lng_slice *sinks, const lng_grouped_shape *shape, int dtype) {
+    return attention(b, q, k, v, out, sinks, shape, dtype, true);
+}
+
+extern "C" int lng_hip_copy_rows(lng_batch *b, lng_slice src, uint64_t src_stride, int src_dtype, lng_slice dst,
+                                 uint64_t dst_stride, int dst_dtype, uint64_t rows, uint64_t width) {
+    if (int rc = need_recording(b)) return rc;
+    for (int d : {src_dtype, dst_dtype}) {
+        if (d != LNG_F32 && d != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", d);
+    }
+    // apple.rs:1769-1781
+    if (rows == 0 || width == 0 || src_stride < width || dst_stride < width) {
+        return fail(LNG_ERR_DISPATCH, "unsupported copy: %llu x %llu, strides %llu and %llu", (unsigned long long)rows,
+                    (unsigned long long)width, (unsigned long long)src_stride, (unsigned long long)dst_stride);
+    }
+    for (uint64_t n : {rows, width, src_stride, dst_stride}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (!fits_u32(rows * std::max(src_stride, dst_stride))) {
+        return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)(rows * std::max(src_stride, dst_stride)));
+    }
+    const uint64_t ss = elem_size(src_dtype), ds = elem_size(dst_dtype);
+    Operand os, od;
+    if (int rc = check_slice(b, "src", src, ((rows - 1) * src_stride + width) * ss, ss, &os)) return rc;
+    if (int rc = check_slice(b, "dst", dst, ((rows - 1) * dst_stride + width) * ds, ds, &od)) return rc;
+    if (int rc = check_output(b, od, {&os})) return rc;
+    lng_k_copy a{};
+    a.src = (const char *)os.buf->ptr + src.offset;
+    a.dst = (char *)od.buf->ptr + dst.offset;
+    a.rows = rows;
+    a.width = width;
+    a.src_stride = src_stride;
+    a.dst_stride = dst_stride;
+    a.src_dtype = (uint32_t)src_dtype;
+    a.dst_dtype = (uint32_t)dst_dtype;
+    Cmd c;
+    c.fn = b->gpu->copy_rows;
+    c.grid[0] = (unsigned)((rows * width + 255) / 256);
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_attention_decode_batched(lng_batch *b, uint64_t q_buffer, uint64_t k_buffer, uint64_t v_buffer,
+                                                uint64_t out_buffer, uint64_t sinks_buffer, const lng_decode_item *items,
+                                                size_t n_items, uint64_t heads, uint64_t kv_heads, uint64_t dim,
+                                                float scale, int dtype) {
+    if (int rc = need_recording(b)) return rc;
+    if (dtype != LNG_F32 && dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", dtype);
+    if (!items || n_items == 0) return fail(LNG_ERR_DISPATCH, "no items");
+    if (!fits_u32(n_items) || !fits_u32(n_items * heads)) return fail(LNG_ERR_DISPATCH, "%zu items do not fit in u32", n_items);
+    lng_buffer *bq = buffer_at(b, q_buffer), *bk = buffer_at(b, k_buffer), *bv = buffer_at(b, v_buffer),
+               *bo = buffer_at(b, out_buffer);
+    if (!bq || !bk || !bv || !bo) return fail(LNG_ERR_DISPATCH, "no such buffer (batch has %zu)", b->buffers.size() + b->residents.size());
+    if (out_buffer >= b->buffers.size()) return fail(LNG_ERR_DISPATCH, "output is in read-only resident memory");
+    const uint64_t es = elem_size(dtype);
+    bool any_sinks = false, aligned16 = true;
+    for (size_t i = 0; i < n_items; ++i) {
+        const lng_decode_item &it = items[i];
+        // every item is the reference's plain dispatch with t = 1
+        lng_grouped_shape s{1, it.start, heads, kv_heads, dim, it.window, it.slots, scale};
+        if (int rc = check_shape(s, false)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        const uint64_t rows = std::min(it.slots, it.start + 1);
+        const lng_slice sq{q_buffer, it.q_offset, heads * dim * es}, sk{k_buffer, it.k_offset, rows * kv_heads * dim * es},
+            sv{v_buffer, it.v_offset, rows * kv_heads * dim * es}, so{out_buffer, it.out_offset, heads * dim * es};
+        Operand oq, ok, ov, oo;
+        if (int rc = check_slice(b, "q", sq, sq.len, es, &oq)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        if (int rc = check_slice(b, "k", sk, sk.len, es, &ok)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        if (int rc = check_slice(b, "v", sv, sv.len, es, &ov)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        if (int rc = check_slice(b, "out", so, so.len, es, &oo)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        if (int rc = check_output(b, oo, {&oq, &ok, &ov})) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+        if (it.sinks_offset != LNG_NO_SINKS) {
+            Operand os;
+            const lng_slice ss{sinks_buffer, it.sinks_offset, heads * 4};
+            if (int rc = check_slice(b, "sinks", ss, ss.len, 4, &os)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+            any_sinks = true;
+        }
+        aligned16 = aligned16 && ((it.q_offset | it.k_offset | it.v_offset | it.out_offset) & 15u) == 0;
+    }
+    // outputs of different items must not overlap each other
+    {
+        std::vector<std::pair<uint64_t, uint64_t>> spans(n_items);
+        for (size_t i = 0; i < n_items; ++i) spans[i] = {items[i].out_offset, items[i].out_offset + heads * dim * es};
+        std::sort(spans.begin(), spans.end());
+        for (size_t i = 1; i < n_items; ++i) {
+            if (spans[i].first < spans[i - 1].second) return fail(LNG_ERR_DISPATCH, "outputs of two items overlap");
+        }
+    }
+    char *host = nullptr, *dev = nullptr;
+    if (int rc = reserve_table(b, n_items * sizeof(lng_k_row), &host, &dev)) return rc;
+    memcpy(host, items, n_items * sizeof(lng_k_row));
+    lng_k_attn a{};
+    a.q = (const char *)bq->ptr;
+    a.k = (const char *)bk->ptr;
+    a.v = (const char *)bv->ptr;
+    a.out = (char *)bo->ptr;
+    a.sinks = any_sinks ? (const char *)buffer_at(b, sinks_buffer)->ptr : nullptr;
+    a.rows = (const lng_k_row *)dev;
+    a.n_rows = (uint32_t)n_items;
+    a.heads = (uint32_t)heads;
+    a.kv_heads = (uint32_t)kv_heads;
+    a.dim = (uint32_t)dim;
+    a.chunk = 128;
+    a.n_chunks = 1;
+    a.dtype = (uint32_t)dtype;
+    a.scale = scale;
+    if (int rc = record_rows(b, a, (const lng_k_row *)host, n_items, 0, aligned16)) return rc;
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, uint64_t seed, float scale,
+                                      uint64_t period) {
+    if (int rc = need_recording(b)) return rc;
+    if (dtype != LNG_F32 && dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", dtype);
+    const uint64_t es = elem_size(dtype);
+    if (dst.len == 0 || dst.len % es != 0) return fail(LNG_ERR_DISPATCH, "dst: %llu bytes is not a whole number of elements", (unsigned long long)dst.len);
+    Operand od;
+    if (int rc = check_slice(b, "dst", dst, dst.len, es, &od)) return rc;
+    if (od.index >= b->buffers.size()) return fail(LNG_ERR_DISPATCH, "output is in read-only resident memory");
+    lng_k_fill a{};
+    a.dst = (char *)od.buf->ptr + dst.offset;
+    a.n = dst.len / es;
+    a.seed = seed;
+    a.period = period;
+    a.factor = scale / LNG_SYNTH_STD;
+    a.dtype = (uint32_t)dtype;
+    Cmd c;
+    c.fn = b->gpu->fill_synthetic;
+    c.grid[0] = (unsigned)std::min<uint64_t>((a.n + 255) / 256, 256u * 64u);
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
+    b->dispatches += 1;
+    return LNG_OK;
+}

@@ -1,0 +1,83 @@
+/*
+ * Kernel argument blocks shared by the host library (lng_hip.cpp) and the gfx950 kernels
+ * (lng_kernels.hip). Each kernel takes exactly one of these structs by value; the host
+ * passes it as the raw kernarg buffer of hipModuleLaunchKernel.
+ */
+#ifndef LNG_KERNEL_ARGS_H
+#define LNG_KERNEL_ARGS_H
+
+#include <stdint.h>
+
+#include "../../include/lng_hip.h"
+
+/* One query row and the cache it attends over: the device-side form of lng_decode_item,
+ * byte offsets relative to the base pointers in lng_k_attn. */
+typedef lng_decode_item lng_k_row;
+
+typedef struct lng_k_attn {
+    const char *q;            /* base of the query buffer */
+    const char *k;            /* base of the key cache buffer */
+    const char *v;            /* base of the value cache buffer */
+    char *out;                /* base of the output buffer */
+    const char *sinks;        /* base of the sinks buffer (f32), unused when a row has none */
+    const lng_k_row *rows;    /* device table of n_rows rows, or NULL: derive row i from `first` */
+    float *partial_o;         /* split-K scratch: [row][kv_head][chunk][group][dim] f32 */
+    float *partial_ml;        /* split-K scratch: [row][kv_head][chunk][group][2] f32 (max, sum) */
+    lng_k_row first;          /* row 0 when rows == NULL; row i: q/out advance by one row, start by i */
+    uint32_t n_rows;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t dim;
+    uint32_t chunk;           /* positions per workgroup along the cache (multiple of 128) */
+    uint32_t n_chunks;        /* workgroups along the cache = ceil(longest visible run / chunk) */
+    uint32_t dtype;           /* lng_dtype of q, k, v, out */
+    float scale;
+} lng_k_attn;
+
+/* Prompt pass: t query rows from `start`, one cache. */
+typedef struct lng_k_prefill {
+    const char *q;
+    const char *k;
+    const char *v;
+    char *out;
+    const float *sinks; /* NULL when absent */
+    uint64_t t;
+    uint64_t start;
+    uint64_t window;
+    uint64_t slots;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t dim;
+    uint32_t q_tiles;   /* ceil(t / rows per workgroup) */
+    float scale;
+    uint32_t pad;
+} lng_k_prefill;
+
+typedef struct lng_k_copy {
+    const char *src;
+    char *dst;
+    uint64_t rows;
+    uint64_t width;
+    uint64_t src_stride;
+    uint64_t dst_stride;
+    uint32_t src_dtype;
+    uint32_t dst_dtype;
+} lng_k_copy;
+
+typedef struct lng_k_fill {
+    char *dst;
+    uint64_t n;      /* elements */
+    uint64_t seed;
+    uint64_t period; /* 0: none */
+    float factor;    /* scale / LNG_SYNTH_STD */
+    uint32_t dtype;
+} lng_k_fill;
+
+/* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with
+ * i' = period ? i % period : i; s = sum of the four 16-bit fields of z; value =
+ * (float)(s - 131070) * factor, one f32 multiply, then narrowed if the dtype is bf16.
+ * The sum of four independent uniform 16-bit integers has standard deviation
+ * sqrt(4 * (65536^2 - 1) / 12). */
+#define LNG_SYNTH_STD 37837.227f
+
+#endif /* LNG_KERNEL_ARGS_H */

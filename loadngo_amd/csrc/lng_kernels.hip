@@ -1,0 +1,463 @@
+// gfx950 (CDNA4) kernels of the grouped-attention operator: compiled to one code object
+// (hipcc --genco) that the host library embeds and loads with hipModuleLoadData.
+//
+// What every kernel here computes is the operator of metal-compute (apple.rs:1199-1401,
+// kernels.metal:500-720 and 1944-2032), itself the GPU twin of gpt-oss/src/model.rs:434-464:
+//   for each query i at absolute position last = start + i, head h, kv head g = h / (H/G):
+//     first = max(0, last + 1 - window);  s_p = (q . k_p) * scale for p in first..=last
+//     m = max(sink, max_p s_p);  Z = exp(sink - m) + sum_p exp(s_p - m)
+//     out = sum_p exp(s_p - m) / Z * v_p                      (position p is in row p % slots)
+// Nothing below is translated from the Metal kernels; the work split, layouts and reductions
+// are chosen for 64-wide wavefronts, MFMA and HBM streaming.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "lng_kernel_args.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+#define LNG_LOG2E 1.4426950408889634f
+#define LNG_NEG_INF (-__builtin_huge_valf())
+
+// ---- element helpers (weights/src/dtype.rs:95-116: widen is a shift, narrow is RNE) --------
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t bits) {
+    return __uint_as_float((uint32_t)bits << 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float value) {
+    uint32_t bits = __float_as_uint(value);
+    if (value != value) return (uint16_t)((bits >> 16) | 0x40);
+    uint32_t bias = 0x7fffu + ((bits >> 16) & 1u);
+    return (uint16_t)((bits + bias) >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float load_elem(const T *p);
+template <> __device__ __forceinline__ float load_elem<float>(const float *p) { return *p; }
+template <> __device__ __forceinline__ float load_elem<uint16_t>(const uint16_t *p) {
+    return bf16_bits_to_f32(*p);
+}
+template <typename T> __device__ __forceinline__ void store_elem(T *p, float x);
+template <> __device__ __forceinline__ void store_elem<float>(float *p, float x) { *p = x; }
+template <> __device__ __forceinline__ void store_elem<uint16_t>(uint16_t *p, float x) {
+    *p = f32_to_bf16_bits(x);
+}
+
+__device__ __forceinline__ lng_k_row row_of(const lng_k_attn &a, uint32_t r) {
+    if (a.rows) return a.rows[r];
+    lng_k_row it = a.first;
+    const uint64_t step = (uint64_t)a.heads * a.dim * (a.dtype == LNG_BF16 ? 2u : 4u);
+    it.q_offset += r * step;
+    it.out_offset += r * step;
+    it.start += r;
+    return it;
+}
+
+__device__ __forceinline__ uint64_t first_visible(uint64_t last, uint64_t window) {
+    return (window != LNG_WINDOW_FULL && last + 1 > window) ? last + 1 - window : 0;
+}
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) x += __shfl_xor(x, s, 64);
+    return x;
+}
+
+// =============================================================================================
+// Generic kernel: any element type, any head width up to 512, any group size. One workgroup
+// per (row, head); its four wavefronts take every fourth position, lanes split the head
+// dimension; per-wavefront online softmax, merged in LDS with the sink joining the merge.
+// Used for f32 (the reference's element type), for widths other than 64 and as the fallback
+// when an operand is not 16-byte aligned. Accurate exp/divide: this is the path held to
+// 1e-5 relative against the CPU reference.
+// =============================================================================================
+template <typename T>
+__device__ __forceinline__ void attn_generic(const lng_k_attn &a) {
+    __shared__ float s_m[4];
+    __shared__ float s_l[4];
+    __shared__ float s_acc[4][512];
+    const uint32_t row = blockIdx.x / a.heads;
+    const uint32_t head = blockIdx.x % a.heads;
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const lng_k_row it = row_of(a, row);
+    const uint32_t dim = a.dim;
+    const uint32_t g = head / (a.heads / a.kv_heads);
+    const T *q = (const T *)(a.q + it.q_offset) + (uint64_t)head * dim;
+    const T *kb = (const T *)(a.k + it.k_offset) + (uint64_t)g * dim;
+    const T *vb = (const T *)(a.v + it.v_offset) + (uint64_t)g * dim;
+    const uint64_t stride = (uint64_t)a.kv_heads * dim;
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+
+    float qv[8], acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t d = lane + 64u * i;
+        qv[i] = d < dim ? load_elem<T>(q + d) : 0.0f;
+        acc[i] = 0.0f;
+    }
+    float m = LNG_NEG_INF, l = 0.0f;
+    for (uint64_t p = first + wave; p <= last; p += 4) {
+        const uint64_t r = p % it.slots;
+        const T *kr = kb + r * stride;
+        const T *vr = vb + r * stride;
+        float part = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t d = lane + 64u * i;
+            if (d < dim) part += qv[i] * load_elem<T>(kr + d);
+        }
+        const float s = wave_sum(part) * a.scale;
+        const float next = fmaxf(m, s);
+        const float keep = m == LNG_NEG_INF ? 0.0f : expf(m - next);
+        const float w = expf(s - next);
+        l = l * keep + w;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t d = lane + 64u * i;
+            if (d < dim) acc[i] = acc[i] * keep + w * load_elem<T>(vr + d);
+        }
+        m = next;
+    }
+    if (lane == 0) {
+        s_m[wave] = m;
+        s_l[wave] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t d = lane + 64u * i;
+        if (d < dim) s_acc[wave][d] = acc[i];
+    }
+    __syncthreads();
+    const float sink = it.sinks_offset != LNG_NO_SINKS
+                           ? ((const float *)(a.sinks + it.sinks_offset))[head]
+                           : LNG_NEG_INF;
+    float top = sink;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) top = fmaxf(top, s_m[w]);
+    float total = sink == LNG_NEG_INF ? 0.0f : expf(sink - top);
+    float weight[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        weight[w] = s_m[w] == LNG_NEG_INF ? 0.0f : expf(s_m[w] - top);
+        total += s_l[w] * weight[w];
+    }
+    T *o = (T *)(a.out + it.out_offset) + (uint64_t)head * dim;
+    for (uint32_t d = threadIdx.x; d < dim; d += 256) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) sum += s_acc[w][d] * weight[w];
+        store_elem<T>(o + d, sum / total);
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void lng_attn_generic_f32(lng_k_attn a) {
+    attn_generic<float>(a);
+}
+
+extern "C" __global__ __launch_bounds__(256) void lng_attn_generic_bf16(lng_k_attn a) {
+    attn_generic<uint16_t>(a);
+}
+
+// =============================================================================================
+// Decode kernel, bf16, head width 64, up to 16 query heads per kv head.
+//
+// Grid: x = chunk of the cache (a.chunk positions), y = row * kv_heads + kv head. A workgroup
+// serves ALL query heads of its kv head at once, so each cached K and V row is read from HBM
+// once per group instead of once per query head. Its four wavefronts take interleaved tiles
+// of 32 positions. Everything is lane-local between the three MFMA stages:
+//
+//   S^T[tok][head] = K[tok][:] . Q[head][:]        2x2 v_mfma_f32_16x16x32_bf16 per tile
+//       lane (n = lane%16, j = lane/16) loads, for token half*16 + n, the 16 bytes at
+//       step*64 + j*16 of the 128-byte K row (global_load_dwordx4): the four lanes of a token
+//       read one contiguous 64-byte half row per instruction, both halves make the 128-byte
+//       run. Q is loaded with the same (step, j) -> bytes rule, so the contraction order is
+//       consistent whatever order the hardware gives the 32 k-slots.
+//       Result: lane holds S^T[half*16 + 4j + i][head n], i = 0..3.
+//   V^T block[dim][tok]: V rows are loaded exactly like K rows (row-major, coalesced) and
+//       transposed on the matrix unit: D = V[tok][k-slots] . E, E a 0/1 selection matrix,
+//       gives lane (n, j) the values V[half*16 + 4j + i][16m + n]: four positions of one
+//       dimension, exact because 1.0 * bf16 accumulates exactly in f32.
+//   O^T[dim][head] += V^T[dim][tok] . P^T[tok][head]: the A operand is the lane's own
+//       transposed V values, the B operand the lane's own exp'd scores, both narrowed to bf16.
+//
+// Online softmax state per lane: running max of its head (log2 domain), its share of the
+// running sum, and 16 accumulators O^T[16m + 4j + i][n]. Wavefronts merge through LDS; with
+// one chunk the workgroup writes the output (sink folded into the normaliser), otherwise it
+// writes (max, sum, O) partials that lng_decode_combine merges.
+// =============================================================================================
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) { return __builtin_bit_cast(bf16x8, x); }
+
+__device__ __forceinline__ bf16x8 narrow8(floatx4 lo, floatx4 hi) {
+    bf16x8 r;
+    r[0] = (__bf16)lo[0];
+    r[1] = (__bf16)lo[1];
+    r[2] = (__bf16)lo[2];
+    r[3] = (__bf16)lo[3];
+    r[4] = (__bf16)hi[0];
+    r[5] = (__bf16)hi[1];
+    r[6] = (__bf16)hi[2];
+    r[7] = (__bf16)hi[3];
+    return r;
+}
+
+struct kv_tile {
+    uint4 k[2][2]; // [position half][k step]
+    uint4 v[2][2];
+};
+
+extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_attn a) {
+    __shared__ float s_m[4][16];
+    __shared__ float s_l[4][16];
+    __shared__ float s_o[4][16][65];
+
+    const uint32_t row = blockIdx.y / a.kv_heads;
+    const uint32_t g = blockIdx.y % a.kv_heads;
+    const lng_k_row it = row_of(a, row);
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+    const uint64_t base = first & ~(uint64_t)31;
+    const uint64_t c0 = base + (uint64_t)blockIdx.x * a.chunk;
+    if (c0 > last) return; // this row has fewer chunks than the longest one
+    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t n = lane & 15u;
+    const uint32_t j = lane >> 4;
+    const uint32_t group = a.heads / a.kv_heads;
+    const bool wraps = it.slots <= last;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
+    const char *kb = a.k + it.k_offset + (uint64_t)g * 128u + j * 16u;
+    const char *vb = a.v + it.v_offset + (uint64_t)g * 128u + j * 16u;
+
+    // Q^T operand: head n of this group, the lane's 8 k-slots of each step.
+    bf16x8 qb[2];
+    {
+        uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
+        if (n < group) {
+            const char *qp = a.q + it.q_offset + ((uint64_t)g * group + n) * 128u + j * 16u;
+            q0 = *(const uint4 *)qp;
+            q1 = *(const uint4 *)(qp + 64);
+        }
+        qb[0] = as_bf16x8(q0);
+        qb[1] = as_bf16x8(q1);
+    }
+    // Selection operands of the transposing product: slot (j, e) of a 32-wide step holds
+    // dimension 8j + e; column n of block parity b wants dimension 16b + n.
+    bf16x8 sel[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sel[b][e] = (8u * j + (uint32_t)e == 16u * (uint32_t)b + n) ? (__bf16)1.0f : (__bf16)0.0f;
+        }
+    }
+
+    auto load_tile = [&](uint64_t tp, kv_tile &t) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            uint64_t p = tp + (uint64_t)(half * 16) + n;
+            p = p < first ? first : p;
+            p = p > last ? last : p;
+            const uint64_t r = wraps ? p % it.slots : p;
+            const uint64_t off = r * row_bytes;
+            t.k[half][0] = *(const uint4 *)(kb + off);
+            t.k[half][1] = *(const uint4 *)(kb + off + 64);
+            t.v[half][0] = *(const uint4 *)(vb + off);
+            t.v[half][1] = *(const uint4 *)(vb + off + 64);
+        }
+    };
+
+    const float sl2 = a.scale * LNG_LOG2E;
+    float m = LNG_NEG_INF; // running max of head n, log2 domain
+    float l = 0.0f;        // this lane's share of the running sum
+    floatx4 ot[4];         // O^T[16mm + 4j + i][head n]
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) ot[mm] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    const floatx4 zero4 = (floatx4){0.f, 0.f, 0.f, 0.f};
+
+    kv_tile cur, nxt;
+    uint64_t tp = c0 + (uint64_t)wave * 32u;
+    if (tp < c1) load_tile(tp, cur);
+    for (; tp < c1; tp += 128u) {
+        const uint64_t tn = tp + 128u;
+        if (tn < c1) load_tile(tn, nxt);
+
+        floatx4 st[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            st[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[half][0]), qb[0], zero4, 0, 0, 0);
+            st[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.k[half][1]), qb[1], st[half], 0, 0, 0);
+        }
+        float tmax = LNG_NEG_INF;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint64_t p = tp + (uint64_t)(half * 16 + i) + 4u * j;
+                const float x = (p >= first && p <= last) ? st[half][i] * sl2 : LNG_NEG_INF;
+                st[half][i] = x;
+                tmax = fmaxf(tmax, x);
+            }
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m, tmax);
+        const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+        float psum = 0.0f;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float pw = __builtin_amdgcn_exp2f(st[half][i] - m_safe);
+                st[half][i] = pw;
+                psum += pw;
+            }
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        const bf16x8 pb = narrow8(st[0], st[1]);
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {
+            const floatx4 t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.v[0][mm >> 1]), sel[mm & 1], zero4, 0, 0, 0);
+            const floatx4 t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.v[1][mm >> 1]), sel[mm & 1], zero4, 0, 0, 0);
+            const bf16x8 va = narrow8(t0, t1);
+            ot[mm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, ot[mm] * alpha, 0, 0, 0);
+        }
+        cur = nxt;
+    }
+
+    // ---- merge the four wavefronts ---------------------------------------------------------
+    {
+        float lt = l + __shfl_xor(l, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (j == 0) {
+            s_m[wave][n] = m;
+            s_l[wave][n] = lt;
+        }
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_o[wave][n][16 * mm + 4 * j + i] = ot[mm][i];
+        }
+    }
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
+        const uint32_t h = idx >> 6;
+        const uint32_t d = idx & 63u;
+        float top = LNG_NEG_INF;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) top = fmaxf(top, s_m[w][h]);
+        float sum = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(s_m[w][h] - top);
+            sum += s_l[w][h] * wt;
+            o += s_o[w][h][d] * wt;
+        }
+        const uint32_t head = g * group + h;
+        if (row_chunks == 1) {
+            const float sink2 = it.sinks_offset != LNG_NO_SINKS
+                                    ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                    : LNG_NEG_INF;
+            const float all = fmaxf(top, sink2);
+            const float keep = __builtin_amdgcn_exp2f(top - all);
+            const float z = sum * keep + (sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - all));
+            uint16_t *op = (uint16_t *)(a.out + it.out_offset) + (uint64_t)head * 64u + d;
+            *op = f32_to_bf16_bits(o * keep / z);
+        } else {
+            const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
+            a.partial_o[slot * 64u + d] = o;
+            if (d == 0) {
+                a.partial_ml[slot * 2u] = top;
+                a.partial_ml[slot * 2u + 1u] = sum;
+            }
+        }
+    }
+}
+
+// Merges the split-K partials of lng_decode_bf16_d64: one wavefront per (row, head), lane =
+// dimension. The sink joins here, once: it adds exp(sink - max) to the normaliser and no value.
+extern "C" __global__ __launch_bounds__(64) void lng_decode_combine(lng_k_attn a) {
+    const uint32_t row = blockIdx.x / a.heads;
+    const uint32_t head = blockIdx.x % a.heads;
+    const lng_k_row it = row_of(a, row);
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+    const uint64_t base = first & ~(uint64_t)31;
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+    if (row_chunks == 1) return; // the decode kernel already wrote this row
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t g = head / group;
+    const uint32_t h = head % group;
+    const uint32_t d = threadIdx.x;
+    const uint64_t slot0 = ((uint64_t)(row * a.kv_heads + g) * a.n_chunks) * group + h;
+    const float sink2 = it.sinks_offset != LNG_NO_SINKS
+                            ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                            : LNG_NEG_INF;
+    float top = sink2;
+    for (uint32_t c = 0; c < row_chunks; ++c) {
+        top = fmaxf(top, a.partial_ml[(slot0 + (uint64_t)c * group) * 2u]);
+    }
+    float z = sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top);
+    float o = 0.0f;
+    for (uint32_t c = 0; c < row_chunks; ++c) {
+        const uint64_t slot = slot0 + (uint64_t)c * group;
+        const float mc = a.partial_ml[slot * 2u];
+        const float wt = mc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(mc - top);
+        z += a.partial_ml[slot * 2u + 1u] * wt;
+        o += a.partial_o[slot * 64u + d] * wt;
+    }
+    uint16_t *op = (uint16_t *)(a.out + it.out_offset) + (uint64_t)head * 64u + d;
+    *op = f32_to_bf16_bits(o / z);
+}
+
+// =============================================================================================
+// Row copy with optional conversion (Batch::copy_rows, apple.rs:1762; kernels.metal:1127-1138):
+// how new K and V rows enter a cache. One thread per element.
+// =============================================================================================
+extern "C" __global__ __launch_bounds__(256) void lng_copy_rows(lng_k_copy a) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (gid >= a.rows * a.width) return;
+    const uint64_t r = gid / a.width;
+    const uint64_t i = gid % a.width;
+    const uint64_t si = r * a.src_stride + i;
+    const uint64_t di = r * a.dst_stride + i;
+    if (a.src_dtype == a.dst_dtype) {
+        if (a.src_dtype == LNG_F32) {
+            ((uint32_t *)a.dst)[di] = ((const uint32_t *)a.src)[si];
+        } else {
+            ((uint16_t *)a.dst)[di] = ((const uint16_t *)a.src)[si];
+        }
+    } else if (a.src_dtype == LNG_F32) {
+        ((uint16_t *)a.dst)[di] = f32_to_bf16_bits(((const float *)a.src)[si]);
+    } else {
+        ((float *)a.dst)[di] = bf16_bits_to_f32(((const uint16_t *)a.src)[si]);
+    }
+}
+
+// Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).
+extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill a) {
+    const uint64_t stride = (uint64_t)gridDim.x * 256u;
+    for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < a.n; i += stride) {
+        const uint64_t e = a.period ? i % a.period : i;
+        uint64_t z = e + a.seed * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        const int s = (int)(z & 0xffff) + (int)((z >> 16) & 0xffff) + (int)((z >> 32) & 0xffff) +
+                      (int)(z >> 48) - 131070;
+        const float x = (float)s * a.factor;
+        if (a.dtype == LNG_F32) {
+            ((float *)a.dst)[i] = x;
+        } else {
+            ((uint16_t *)a.dst)[i] = f32_to_bf16_bits(x);
+        }
+    }
+}

@@ -223,11 +223,12 @@ void lng_oracle_attention_f64(const float *q, const float *k, const float *v,
         double z = 0.0;
         for (uint64_t j = 0; j < count; ++j) z += exp(scores[j] - m);
         z += exp(sink - m);
+        /* exp(x - m) / z does not depend on d: evaluated once per position, same value */
+        for (uint64_t j = 0; j < count; ++j) scores[j] = exp(scores[j] - m) / z;
         for (uint64_t d = 0; d < dim; ++d) {
             double acc = 0.0;
             for (uint64_t p = first; p <= last; ++p) {
-                acc += exp(scores[p - first] - m) / z *
-                       (double)v[((p % slots) * kv_heads + g) * dim + d];
+                acc += scores[p - first] * (double)v[((p % slots) * kv_heads + g) * dim + d];
             }
             out[(i * heads + h) * dim + d] = (float)acc;
         }

@@ -1,0 +1,70 @@
+"""Helpers of the GPU parity tests: everything goes through the C ABI (loadngo_amd.compute)."""
+import numpy as np
+import pytest
+
+from loadngo_amd import compute as C
+from tests.helpers import from_bf16_bits, ring_layout, to_bf16_bits
+
+THREADS = 8  # oracle threads: spreads (query, head) pairs, arithmetic per pair unchanged
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    g = C.Gpu()  # raises without the built library or without a device: no fallback
+    yield g
+    g.close()
+
+
+def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out=True):
+    """One dispatch as the reference's test harness lays it out (attention_grouped.rs:102-158):
+    five buffers (q, k, v, out, sinks), slices over all of each. q is [t][H][D]; for the tiled
+    operator it is zero-padded to t rounded up to 32 rows. Returns out[:t] (f32 or bf16 bits)."""
+    t, heads, dim = q.shape
+    es = 4 if dtype == C.F32 else 2
+    rows = (t + 31) // 32 * 32 if tiled else t
+    qp = np.zeros((rows, heads, dim), dtype=q.dtype)
+    qp[:t] = q
+    out_len = rows * heads * dim * es
+    bufs = [gpu.upload(qp), gpu.upload(k_ring), gpu.upload(v_ring), gpu.buffer(out_len),
+            gpu.upload(sinks if sinks is not None else np.zeros(1, np.float32))]
+    if poison_out:
+        bufs[3].fill(0xFF)  # NaN pattern in both f32 and bf16: unwritten outputs show
+    batch = gpu.batch(bufs)
+    qs, ks, vs, os_ = (C.Slice(0, 0, qp.nbytes), C.Slice(1, 0, k_ring.nbytes), C.Slice(2, 0, v_ring.nbytes),
+                       C.Slice(3, 0, out_len))
+    try:
+        if sinks is None:
+            (batch.attention_grouped_tiled if tiled else batch.attention_grouped)(qs, ks, vs, os_, shape, dtype)
+        else:
+            ss = C.Slice(4, 0, shape.heads * 4)
+            (batch.attention_grouped_tiled_with_sinks if tiled else batch.attention_grouped_with_sinks)(
+                (qs, ks, vs), ss, os_, shape, dtype)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        out = bufs[3].read(np.float32 if dtype == C.F32 else np.uint16)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    return out.reshape(rows, heads, dim)[:t]
+
+
+def reference_case(oracle, case, sharp, tiled, sinks, scale, dtype):
+    """Inputs of one reference test case (attention_grouped.rs:102-135): q = values(1)*sharp,
+    k = values(2), v = values(3) over every absolute position, laid into the ring."""
+    t, start, heads, kv_heads, dim, window, slots = case
+    end = start + t
+    q = (oracle.values(1, t * heads * dim) * np.float32(sharp)).reshape(t, heads, dim)
+    k = oracle.values(2, end * kv_heads * dim).reshape(end, kv_heads, dim)
+    v = oracle.values(3, end * kv_heads * dim).reshape(end, kv_heads, dim)
+    shape = C.GroupedShape(t, start, heads, kv_heads, dim, window, slots, scale)
+    if dtype == C.BF16:
+        q, k, v = (from_bf16_bits(to_bf16_bits(x)) for x in (q, k, v))  # exactly representable
+    kr, vr = ring_layout(k, t, start, slots, tiled), ring_layout(v, t, start, slots, tiled)
+    return q, k, v, kr, vr, shape
+
+
+def max_error(got, want):
+    """attention_grouped.rs:151-157: a NaN counts as infinite error."""
+    e = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    return np.inf if np.isnan(e).any() else float(e.max())

@@ -1,0 +1,286 @@
+"""GPU parity: the HIP operator, called through the C ABI, against the CPU oracle.
+
+Bars: f32 within 1e-5 relative of the CPU reference restatement (and within the reference's
+own 2e-5 / 1e-4 of its float64 definition on its own test shapes); bf16 in/out within 2e-2
+max-abs of the CPU reference run on the same bf16 inputs."""
+import numpy as np
+import pytest
+
+from loadngo_amd import compute as C
+from oracle import oracle
+from tests.gpu_common import THREADS, gpu, max_error, reference_case, run_attention  # noqa: F401
+from tests.helpers import (FULL, REF_GPT_OSS_CASES, REF_PLAIN_CASES, REF_REJECTED, REF_TILED_CASES,
+                           from_bf16_bits, normal_inputs, ring_layout, to_bf16_bits)
+
+pytestmark = pytest.mark.gpu
+
+BF16_TOL = 2e-2  # max-abs, bf16 in/out with f32 accumulation
+F32_RTOL = 1e-5  # relative, f32 configuration
+
+
+def rel_error(got, want):
+    e = np.abs(got.astype(np.float64) - want) / (np.abs(want) + 1.0)
+    return np.inf if np.isnan(e).any() else float(e.max())
+
+
+# ---- the reference's own operator tests, f32 -------------------------------------------------
+@pytest.mark.parametrize("case,sharp", REF_PLAIN_CASES)
+def test_plain_matches_the_float64_definition(gpu, case, sharp):
+    q, k, v, kr, vr, shape = reference_case(oracle, case, sharp, False, None, 1.0, C.F32)
+    got = run_attention(gpu, q, kr, vr, None, shape, False, C.F32)
+    want = oracle.attention_f64(q, k, v, None, shape.start, window=shape.window, scale=1.0, threads=THREADS)
+    assert max_error(got, want) < 2e-5, case  # attention_grouped.rs:201
+
+
+@pytest.mark.parametrize("case,sharp", REF_TILED_CASES)
+def test_tiled_matches_the_float64_definition(gpu, case, sharp):
+    q, k, v, kr, vr, shape = reference_case(oracle, case, sharp, True, None, 1.0, C.F32)
+    got = run_attention(gpu, q, kr, vr, None, shape, True, C.F32)
+    want = oracle.attention_f64(q, k, v, None, shape.start, window=shape.window, scale=1.0, threads=THREADS)
+    assert max_error(got, want) < 1e-4, case  # attention_grouped.rs:224
+
+
+@pytest.mark.parametrize("case,tiled", REF_GPT_OSS_CASES)
+@pytest.mark.parametrize("dtype", [C.F32, C.BF16])
+def test_sinks_take_probability_without_value_on_gpt_oss_shapes(gpu, case, tiled, dtype):
+    t, start, window, slots = case
+    sinks = oracle.values(4, 64) * np.float32(3.0)
+    q, k, v, kr, vr, shape = reference_case(oracle, (t, start, 64, 8, 64, window, slots), 1.0, tiled, sinks,
+                                            0.125, dtype)
+    if dtype == C.F32:
+        got = run_attention(gpu, q, kr, vr, sinks, shape, tiled, C.F32)
+        want = oracle.attention_f64(q, k, v, sinks, start, window=window, scale=0.125, threads=THREADS)
+        assert max_error(got, want) < 1e-4, case  # attention_grouped.rs:251
+        want32 = oracle.attention_f32(q, k, v, sinks, start, window=window, scale=0.125, threads=THREADS)
+        assert rel_error(got, want32) < F32_RTOL
+    else:
+        got = run_attention(gpu, to_bf16_bits(q), to_bf16_bits(kr), to_bf16_bits(vr), sinks, shape, tiled, C.BF16)
+        want = oracle.attention_bf16(to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v), sinks, start,
+                                     window=window, scale=0.125, threads=THREADS)
+        assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL, case
+
+
+def test_rejects_shapes_it_cannot_run(gpu):
+    """attention_grouped.rs:255-275: four 1 MiB buffers, whole-buffer slices, every shape refused."""
+    for case in REF_REJECTED:
+        bufs = [gpu.buffer(1 << 20) for _ in range(4)]
+        batch = gpu.batch(bufs)
+        s = [C.Slice(i, 0, 1 << 20) for i in range(4)]
+        with pytest.raises(C.Dispatch):
+            batch.attention_grouped(s[0], s[1], s[2], s[3], C.GroupedShape(*case, 1.0))
+        assert batch.dispatches() == 0
+        batch.drop()
+        for b in bufs:
+            b.free()
+
+
+# ---- configuration 1: fp32 plumbing ----------------------------------------------------------
+def test_config1_fp32_plumbing_matches_the_cpu_reference(gpu):
+    """H=4, G=1, D=64, T=32 causal with sinks, seed 0: every row of the pass against the CPU
+    reference's f32 arithmetic, 1e-5 relative; both operator forms."""
+    q, k, v, sinks = normal_inputs(0, 32, 32, 4, 1, 64)
+    want = oracle.attention_f32(q, k, v, sinks, 0)
+    shape = C.GroupedShape(32, 0, 4, 1, 64, FULL, 32, 0.125)
+    for tiled in (False, True):
+        got = run_attention(gpu, q, k, v, sinks, shape, tiled, C.F32)
+        assert rel_error(got, want) < F32_RTOL
+    golden = np.load("tests/golden/config1_fp32.npz")
+    assert np.array_equal(golden["q"], q) and np.array_equal(golden["sinks"], sinks)
+    assert rel_error(run_attention(gpu, q, k, v, sinks, shape, False, C.F32), golden["out"]) < F32_RTOL
+
+
+# ---- configuration 2: one decoding query over 4096 cached positions, bf16 ---------------------
+def test_config2_decode_4096_bf16(gpu):
+    q, k, v, sinks = normal_inputs(2, 1, 4096, 64, 8, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    shape = C.GroupedShape(1, 4095, 64, 8, 64, FULL, 4096, 0.125)
+    got = run_attention(gpu, qb, kb, vb, sinks, shape, False, C.BF16)
+    want = oracle.attention_bf16(qb, kb, vb, sinks, 4095, scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+    # and much closer than the bar against the float64 definition
+    exact = oracle.attention_f64(from_bf16_bits(qb), from_bf16_bits(kb), from_bf16_bits(vb), sinks, 4095,
+                                 scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(got), exact) < 4e-3
+
+
+@pytest.mark.parametrize("start,window,slots", [
+    (0, FULL, 64), (1, FULL, 64), (31, FULL, 32), (32, FULL, 33), (127, 128, 640), (128, 128, 640),
+    (700, 128, 640), (3000, 128, 640), (5000, 128, 129), (130, 7, 12), (4095, FULL, 8192), (8191, FULL, 8192),
+    (1000, 1, 5), (999, 1000, 1000), (6001, 4000, 4096),
+])
+def test_decode_bf16_window_ring_and_edges(gpu, start, window, slots):
+    """Decoding at the edges: first token, tile boundaries, windows that wrap the ring, rings not
+    a multiple of the tile, a window of one. Rows the operator must not read hold NaN."""
+    end = start + 1
+    q, k, v, sinks = normal_inputs(start + 17, 1, end, 64, 8, 64, scale=0.5)
+    kr, vr = ring_layout(k, 1, start, slots, False), ring_layout(v, 1, start, slots, False)
+    # rows of the ring older than the window are poisoned too
+    first = 0 if window == FULL else max(0, end - window)
+    for p in range(max(0, end - slots), first):
+        kr[p % slots] = np.nan
+        vr[p % slots] = np.nan
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(kr), to_bf16_bits(vr)
+    shape = C.GroupedShape(1, start, 64, 8, 64, window, slots, 0.125)
+    got = run_attention(gpu, qb, kb, vb, sinks, shape, False, C.BF16)
+    want = oracle.attention_bf16(qb, to_bf16_bits(k), to_bf16_bits(v), sinks, start, window=window, scale=0.125,
+                                 threads=THREADS)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+    none = run_attention(gpu, qb, kb, vb, None, shape, False, C.BF16)
+    want_none = oracle.attention_bf16(qb, to_bf16_bits(k), to_bf16_bits(v), None, start, window=window,
+                                      scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(none), from_bf16_bits(want_none)) < BF16_TOL
+
+
+@pytest.mark.parametrize("heads,kv_heads,dim", [(8, 8, 64), (16, 1, 64), (12, 4, 64), (64, 2, 64), (8, 2, 128),
+                                                (4, 4, 32)])
+def test_decode_bf16_other_groupings(gpu, heads, kv_heads, dim):
+    """Group sizes 1..32 and widths other than 64 (the latter, and groups over 16, take the
+    general kernel)."""
+    start = 777
+    q, k, v, sinks = normal_inputs(5, 3, start + 3, heads, kv_heads, dim, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    shape = C.GroupedShape(3, start, heads, kv_heads, dim, 300, start + 3, 0.125)
+    got = run_attention(gpu, qb, kb, vb, sinks, shape, False, C.BF16)
+    want = oracle.attention_bf16(qb, kb, vb, sinks, start, window=300, scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
+# ---- configuration 3: ragged batch, a full and a sliding layer per sequence -------------------
+def test_config3_batched_ragged_decode(gpu):
+    rng = np.random.default_rng(3)
+    n_seq, heads, kv_heads, dim = 32, 64, 8, 64
+    lens = rng.integers(128, 8193, size=n_seq)
+    row = kv_heads * dim
+    k_all = to_bf16_bits((rng.standard_normal((int(lens.sum()), kv_heads, dim)) * 0.5).astype(np.float32))
+    v_all = to_bf16_bits((rng.standard_normal((int(lens.sum()), kv_heads, dim)) * 0.5).astype(np.float32))
+    q = to_bf16_bits((rng.standard_normal((2 * n_seq, heads, dim)) * 0.5).astype(np.float32))
+    sinks = rng.standard_normal((2, heads)).astype(np.float32)  # one set per layer
+    bufs = [gpu.upload(q), gpu.upload(k_all), gpu.upload(v_all), gpu.buffer(q.nbytes), gpu.upload(sinks)]
+    bufs[3].fill(0xFF)
+    offs = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    items, want = [], np.empty_like(q)
+    for layer, window in enumerate((FULL, 128)):
+        for s in range(n_seq):
+            i = layer * n_seq + s
+            L = int(lens[s])
+            items.append(C.DecodeItem(i * heads * dim * 2, i * heads * dim * 2, int(offs[s]) * row * 2,
+                                      int(offs[s]) * row * 2, layer * heads * 4, L - 1, window, L))
+            sl = slice(int(offs[s]), int(offs[s]) + L)
+            want[i] = oracle.attention_bf16(q[i:i + 1], k_all[sl], v_all[sl], sinks[layer], L - 1, window=window,
+                                            scale=0.125, threads=THREADS)[0]
+    batch = gpu.batch(bufs)
+    batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, 0.125, C.BF16)
+    assert batch.dispatches() == 1
+    done = batch.run()
+    assert not isinstance(done.gpu_time, Exception)
+    got = bufs[3].read(np.uint16).reshape(q.shape)
+    batch.drop()
+    for b in bufs:
+        b.free()
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
+def test_batched_decode_f32_and_errors(gpu):
+    heads, kv_heads, dim = 8, 2, 64
+    q, k, v, sinks = normal_inputs(21, 2, 50, heads, kv_heads, dim)
+    bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.buffer(q.nbytes), gpu.upload(sinks)]
+    batch = gpu.batch(bufs)
+    step = heads * dim * 4
+    items = [C.DecodeItem(0, 0, 0, 0, 0, 39, FULL, 40), C.DecodeItem(step, step, 0, 0, None, 49, 16, 50)]
+    batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, 0.125, C.F32)
+    with pytest.raises(C.Dispatch):  # outputs overlap
+        batch.attention_decode_batched(0, 1, 2, 3, 4, [items[0], items[0]], heads, kv_heads, dim, 0.125, C.F32)
+    with pytest.raises(C.Dispatch):  # cache rows outside the buffer
+        batch.attention_decode_batched(0, 1, 2, 3, 4, [C.DecodeItem(0, 0, 0, 0, 0, 99, FULL, 100)], heads, kv_heads,
+                                       dim, 0.125, C.F32)
+    batch.run()
+    got = bufs[3].read(np.float32).reshape(q.shape)
+    batch.drop()
+    for b in bufs:
+        b.free()
+    want0 = oracle.attention_f32(q[0:1], k[:40], v[:40], sinks, 39, scale=0.125)[0]
+    want1 = oracle.attention_f32(q[1:2], k, v, None, 49, window=16, scale=0.125)[0]
+    assert rel_error(got[0], want0) < F32_RTOL and rel_error(got[1], want1) < F32_RTOL
+
+
+# ---- the glue either side --------------------------------------------------------------------
+def test_copy_rows_writes_new_rows_into_a_ring_and_converts(gpu):
+    """gpt-oss/src/gpu.rs:744-759: position s goes to row s % slots, in at most two runs; here
+    the f32 rows of a projection are rounded into a bf16 cache on the way."""
+    slots, width, n, start = 12, 512, 7, 9
+    rng = np.random.default_rng(4)
+    new = rng.standard_normal((n, width)).astype(np.float32)
+    cache = np.zeros((slots, width), np.uint16)
+    bufs = [gpu.upload(new), gpu.upload(cache)]
+    batch = gpu.batch(bufs)
+    done = 0
+    while done < n:
+        row = (start + done) % slots
+        run = min(n - done, slots - row)
+        batch.copy_rows((C.Slice(0, done * width * 4, run * width * 4), width),
+                        (C.Slice(1, row * width * 2, run * width * 2), width), run, width, C.F32, C.BF16)
+        done += run
+    with pytest.raises(C.Dispatch):
+        batch.copy_rows((C.Slice(0, 0, 4), 1), (C.Slice(1, 0, 2), 1), 0, 1, C.F32, C.BF16)
+    with pytest.raises(C.Dispatch):  # stride narrower than the width
+        batch.copy_rows((C.Slice(0, 0, 2 * width * 4), width - 1), (C.Slice(1, 0, 2 * width * 2), width), 2, width,
+                        C.F32, C.BF16)
+    batch.run()
+    got = bufs[1].read(np.uint16).reshape(slots, width)
+    batch.drop()
+    for i in range(n):
+        cache[(start + i) % slots] = to_bf16_bits(new[i])
+    assert np.array_equal(got, cache)
+    for b in bufs:
+        b.free()
+
+
+def test_buffers_belong_to_their_batch_until_it_finishes(gpu):
+    a, b = gpu.buffer(1024), gpu.buffer(1024)
+    batch = gpu.batch([a, b])
+    with pytest.raises(C.Dispatch):
+        a.write(np.zeros(4, np.float32))
+    with pytest.raises(C.Dispatch):
+        gpu.batch([a])
+    with pytest.raises(C.Dispatch):
+        a.free()
+    batch.drop()  # dropped uncommitted: nothing ran, the buffers are back
+    a.write(np.arange(256, dtype=np.float32))
+    assert np.array_equal(a.read(np.float32), np.arange(256, dtype=np.float32))
+    with pytest.raises(C.Alloc):
+        gpu.buffer(0)
+    res = gpu.resident(np.arange(8, dtype=np.float32))
+    batch = gpu.batch([a, b])
+    whole = batch.attach(res)
+    assert whole == C.Slice(2, 0, 32) and batch.attach(res) == whole
+    with pytest.raises(C.Dispatch):  # output in resident memory
+        batch.copy_rows((C.Slice(0, 0, 32), 8), (whole, 8), 1, 8)
+    with pytest.raises(C.Dispatch):  # output overlaps the input
+        batch.copy_rows((C.Slice(0, 0, 32), 8), (C.Slice(0, 16, 32), 8), 1, 8)
+    batch.copy_rows((whole, 8), (C.Slice(1, 0, 32), 8), 1, 8)
+    seen = []
+    batch.commit(lambda done: seen.append(done.gpu_time))
+    done = batch.wait()
+    assert seen and seen[0] == done.gpu_time and done.gpu_time >= 0.0
+    assert np.array_equal(b.read(np.float32, count=8), np.arange(8, dtype=np.float32))
+    batch.drop()
+    for x in (a, b, res):
+        x.free()
+
+
+def test_synthetic_fill_is_reproducible_on_the_host(gpu):
+    n, seed, scale, period = 5000, 77, 0.5, 1024
+    buf = gpu.buffer(n * 2)
+    f32 = gpu.buffer(n * 4)
+    batch = gpu.batch([buf, f32])
+    batch.fill_synthetic(C.Slice(0, 0, n * 2), C.BF16, seed, scale, period)
+    batch.fill_synthetic(C.Slice(1, 0, n * 4), C.F32, seed, scale, 0)
+    batch.run()
+    got, got32 = buf.read(np.uint16), f32.read(np.float32)
+    batch.drop()
+    buf.free()
+    f32.free()
+    from loadngo_amd.synthetic import synthetic_values
+    assert np.array_equal(got32, synthetic_values(n, seed, scale, 0))
+    assert np.array_equal(got, to_bf16_bits(synthetic_values(n, seed, scale, period)))
+    assert abs(float(got32.std()) - scale) < 0.02 and abs(float(got32.mean())) < 0.03
