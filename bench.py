@@ -1,0 +1,323 @@
+#!/usr/bin/env python3
+"""Benchmark of the gpt-oss attention path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c5|c3|c2] [--no-extras] [--no-cpu]
+
+A step is one pass of the hot path over one batch of synthetic input resident in HBM. The
+headline workload is the long-context decode stack (24 layers alternating 128-token window
+and full-causal, batch 16, context 131072, bf16 KV cache of 96 GiB): one step decodes one
+token for every sequence through all 24 layers' attention. `value` is the KV-cache GB/s of
+the whole step (algorithmic bytes / wall time per step); `roofline` is the decode kernel's
+own bandwidth (algorithmic bytes per launch / its average launch time from HIP events on the
+library's stream). The other configurations (single 4096-token decode, ragged batch of 32,
+8192-token prompt passes) are reported under "extra". The CPU baseline is the oracle (a C
+restatement of the reference's CPU attention) timed on this host on a bounded sample.
+
+Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from loadngo_amd import compute as C  # noqa: E402
+from loadngo_amd.synthetic import bf16_bits, bf16_widen  # noqa: E402
+
+H, G, D = 64, 8, 64
+SCALE = 0.125
+ROW = G * D * 2          # bytes of one cached position of K (or V) in bf16
+QO = H * D * 2           # bytes of one query (or output) row
+HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+METRIC = "decode attn GB/s (% HBM peak) + prefill attn TFLOP/s (% MFMA), gpt-oss shapes"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def decode_bytes(length, window):
+    """Algorithmic bytes of one decoding query over one layer: visible K+V rows, q, out, sinks."""
+    visible = length if window == C.FULL else min(length, window)
+    return visible * 2 * ROW + 2 * QO + H * 4
+
+
+def fill(gpu, buf, seed, scale=0.5, period=0):
+    batch = gpu.batch([buf])
+    batch.fill_synthetic(C.Slice(0, 0, buf.len), C.BF16, seed, scale, period)
+    batch.run()
+    batch.drop()
+
+
+# ------------------------------------------------------------------------------------------------
+def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
+    """Configuration 5: the 24-layer decode stack."""
+    log("allocating %.1f GiB of KV cache" % (layers * 2 * batch_size * ctx * ROW / 2**30))
+    q = gpu.buffer(layers * batch_size * QO)
+    out = gpu.buffer(layers * batch_size * QO)
+    sinks = gpu.upload(np.random.default_rng(5).standard_normal((layers, H)).astype(np.float32))
+    fill(gpu, q, 1000)
+    caches = []
+    for l in range(layers):
+        k, v = gpu.buffer(batch_size * ctx * ROW), gpu.buffer(batch_size * ctx * ROW)
+        fill(gpu, k, 2 * l + 1)
+        fill(gpu, v, 2 * l + 2)
+        caches += [k, v]
+    bufs = [q, out, sinks] + caches
+    tables = []
+    step_bytes = 0
+    for l in range(layers):
+        window = 128 if l % 2 == 0 else C.FULL  # even layers slide (gpt-oss/src/config.rs:99-103)
+        items = [C.DecodeItem((l * batch_size + b) * QO, (l * batch_size + b) * QO, b * ctx * ROW, b * ctx * ROW,
+                              l * H * 4, ctx - 1, window, ctx) for b in range(batch_size)]
+        tables.append(C.decode_items(items))
+        step_bytes += batch_size * decode_bytes(ctx, window)
+
+    def step(timing):
+        batch = gpu.batch(bufs)
+        if timing:
+            batch.set_timing(True)
+        for l in range(layers):
+            batch.attention_decode_batched(0, 3 + 2 * l, 4 + 2 * l, 1, 2, tables[l], H, G, D, SCALE, C.BF16)
+        batch.commit()
+        done = batch.wait()
+        ks = batch.kernel_seconds("lng_decode_bf16_d64") if timing else (0.0, 0)
+        cs = batch.kernel_seconds("lng_decode_combine") if timing else (0.0, 0)
+        batch.drop()
+        return done.gpu_time, ks, cs
+
+    for _ in range(warmup):
+        step(False)
+    t0 = time.perf_counter()
+    gpu_s = kern_s = comb_s = 0.0
+    launches = 0
+    for _ in range(steps):
+        g, (ks, kn), (cs, _) = step(True)
+        gpu_s += g
+        kern_s += ks
+        comb_s += cs
+        launches += kn
+    wall = time.perf_counter() - t0
+    for b in bufs:
+        b.free()
+    per_launch_bytes = step_bytes * steps / launches
+    per_launch_s = kern_s / launches
+    return {
+        "workload": "C5 long-context decode stack: 24 layers (even: 128-token window, odd: full causal), "
+                    "batch %d, context %d, 64 q heads / 8 kv heads / head_dim 64, bf16 KV cache %.1f GiB resident"
+                    % (batch_size, ctx, layers * 2 * batch_size * ctx * ROW / 2**30),
+        "step_bytes": step_bytes,
+        "wall_s_per_step": wall / steps,
+        "gpu_s_per_step": gpu_s / steps,
+        "value_gbs": step_bytes / (wall / steps) / 1e9,
+        "tokens_per_s": batch_size / (wall / steps),
+        "kernel": "lng_decode_bf16_d64",
+        "kernel_launches_per_step": launches // steps,
+        "kernel_bytes_per_launch": per_launch_bytes,
+        "kernel_s_per_launch": per_launch_s,
+        "kernel_gbs": per_launch_bytes / per_launch_s / 1e9,
+        "combine_s_per_step": comb_s / steps,
+    }
+
+
+def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
+    """Configuration 2: one query over 4096 cached positions, full-causal layer. 8.4 MB of
+    traffic is about a microsecond at HBM speed, so one launch is latency-bound: reported as
+    one launch per batch and as `burst` launches back to back in one batch."""
+    q, out = gpu.buffer(QO), gpu.buffer(QO)
+    k, v = gpu.buffer(ctx * ROW), gpu.buffer(ctx * ROW)
+    sinks = gpu.upload(np.random.default_rng(2).standard_normal(H).astype(np.float32))
+    for i, b in enumerate((q, k, v)):
+        fill(gpu, b, 10 + i)
+    bufs = [q, k, v, out, sinks]
+    shape = C.GroupedShape(1, ctx - 1, H, G, D, C.FULL, ctx, SCALE)
+    sl = (C.Slice(0, 0, QO), C.Slice(1, 0, ctx * ROW), C.Slice(2, 0, ctx * ROW))
+
+    def go(n):
+        batch = gpu.batch(bufs)
+        for _ in range(n):
+            batch.attention_grouped_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, QO), shape, C.BF16)
+        t0 = time.perf_counter()
+        done = batch.run()
+        wall = time.perf_counter() - t0
+        batch.drop()
+        return done.gpu_time, wall
+
+    for _ in range(warmup):
+        go(1)
+    one = sorted(go(1) for _ in range(max(steps, 5)))
+    many = sorted(go(burst) for _ in range(max(steps, 5)))
+    for b in bufs:
+        b.free()
+    nbytes = decode_bytes(ctx, C.FULL)
+    g1, w1 = one[len(one) // 2]
+    gb, wb = many[len(many) // 2]
+    return {"workload": "C2 decode, 1 query, 4096 cached positions, full-causal", "bytes": nbytes,
+            "single_launch_gpu_us": g1 * 1e6, "single_launch_wall_us": w1 * 1e6,
+            "single_launch_gbs": nbytes / g1 / 1e9 if g1 > 0 else None,
+            "burst": burst, "burst_gpu_us_per_launch": gb / burst * 1e6,
+            "burst_gbs": nbytes * burst / gb / 1e9,
+            "note": "8 MB working set stays in the 256 MB Infinity Cache across launches: cache-fed, not HBM-fed"}
+
+
+def run_ragged(gpu, steps, warmup, n_seq=32):
+    """Configuration 3: 32 sequences with lengths U{128..8192}; per sequence one full-causal
+    layer and one 128-window layer; both layers of all sequences in one dispatch each."""
+    rng = np.random.default_rng(3)
+    lens = rng.integers(128, 8193, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    total = int(lens.sum())
+    q, out = gpu.buffer(2 * n_seq * QO), gpu.buffer(2 * n_seq * QO)
+    k, v = gpu.buffer(total * ROW), gpu.buffer(total * ROW)
+    sinks = gpu.upload(rng.standard_normal((2, H)).astype(np.float32))
+    for i, b in enumerate((q, k, v)):
+        fill(gpu, b, 20 + i)
+    bufs = [q, k, v, out, sinks]
+    tables, nbytes = [], 0
+    for layer, window in enumerate((C.FULL, 128)):
+        items = []
+        for s in range(n_seq):
+            i = layer * n_seq + s
+            items.append(C.DecodeItem(i * QO, i * QO, int(offs[s]) * ROW, int(offs[s]) * ROW, layer * H * 4,
+                                      int(lens[s]) - 1, window, int(lens[s])))
+            nbytes += decode_bytes(int(lens[s]), window)
+        tables.append(C.decode_items(items))
+
+    def go():
+        batch = gpu.batch(bufs)
+        for tb in tables:
+            batch.attention_decode_batched(0, 1, 2, 3, 4, tb, H, G, D, SCALE, C.BF16)
+        t0 = time.perf_counter()
+        done = batch.run()
+        wall = time.perf_counter() - t0
+        batch.drop()
+        return done.gpu_time, wall
+
+    for _ in range(warmup):
+        go()
+    runs = sorted(go() for _ in range(max(steps, 5)))
+    for b in bufs:
+        b.free()
+    g, w = runs[len(runs) // 2]
+    return {"workload": "C3 batched decode: 32 sequences, lengths U{128..8192} (seed 3), full + 128-window layer each",
+            "bytes": nbytes, "gpu_us": g * 1e6, "wall_us": w * 1e6, "gbs": nbytes / g / 1e9,
+            "tokens_per_s": n_seq / w,
+            "note": "about 280 MB per step: close to the 256 MB Infinity Cache, partly cache-fed"}
+
+
+def run_prefill(gpu, steps, warmup, t=8192):
+    """Configuration 4: one prompt pass of 8192 positions, once full-causal and once with a
+    128-token window. FLOPs = 4 * dim * heads * (unmasked query-key pairs)."""
+    q, out = gpu.buffer(t * QO), gpu.buffer(t * QO)
+    k, v = gpu.buffer(t * ROW), gpu.buffer(t * ROW)
+    sinks = gpu.upload(np.random.default_rng(4).standard_normal(H).astype(np.float32))
+    for i, b in enumerate((q, k, v)):
+        fill(gpu, b, 30 + i)
+    bufs = [q, k, v, out, sinks]
+    sl = (C.Slice(0, 0, t * QO), C.Slice(1, 0, t * ROW), C.Slice(2, 0, t * ROW))
+    res = {}
+    for name, window in (("full", C.FULL), ("window128", 128)):
+        shape = C.GroupedShape(t, 0, H, G, D, window, t, SCALE)
+        w = t if window == C.FULL else window
+        pairs = w * (w + 1) // 2 + (t - w) * w
+        flops = 4 * D * H * pairs
+
+        def go():
+            batch = gpu.batch(bufs)
+            batch.attention_grouped_tiled_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, t * QO), shape, C.BF16)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        for _ in range(warmup):
+            go()
+        runs = sorted(go() for _ in range(max(steps, 5)))
+        g = runs[len(runs) // 2]
+        traffic = 2 * t * QO + 2 * t * ROW
+        res[name] = {"pairs": pairs, "flops": flops, "gpu_ms": g * 1e3, "tflops": flops / g / 1e12,
+                     "mfma_frac": flops / g / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "qkvo_bytes": traffic, "hbm_frac": traffic / g / 1e9 / HBM_PEAK_GBS}
+    for b in bufs:
+        b.free()
+    res["workload"] = "C4 causal prefill, 8192 positions, 64 q / 8 kv heads, head_dim 64, bf16"
+    return res
+
+
+def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
+    """The oracle (port of the reference's CPU attention, f32 on widened bf16 inputs) on a
+    bounded sample of the headline workload: one sequence, one full-causal and one 128-window
+    layer at the full context. GB/s is counted on the same algorithmic bf16 bytes as the GPU."""
+    from oracle import oracle
+    rng = np.random.default_rng(9)
+    q = bf16_widen(bf16_bits(rng.standard_normal((1, H, D), dtype=np.float32) * 0.5))
+    k = bf16_widen(bf16_bits(rng.standard_normal((ctx, G, D), dtype=np.float32) * 0.5))
+    v = bf16_widen(bf16_bits(rng.standard_normal((ctx, G, D), dtype=np.float32) * 0.5))
+    sinks = rng.standard_normal(H).astype(np.float32)
+    cores = min(16, os.cpu_count() or 1)
+    nbytes = decode_bytes(ctx, C.FULL) + decode_bytes(ctx, 128)
+    out = {}
+    for label, threads in (("all", cores), ("one", 1)):
+        t0 = time.perf_counter()
+        oracle.attention_f32(q, k, v, sinks, ctx - 1, window=C.FULL, scale=SCALE, threads=threads)
+        oracle.attention_f32(q, k, v, sinks, ctx - 1, window=128, scale=SCALE, threads=threads)
+        out[label] = time.perf_counter() - t0
+    return {"value": nbytes / out["all"] / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "1 sequence x (1 full-causal + 1 window-128 layer) at context %d, %.0f MB of bf16 KV; "
+                      "the 16 x 12 such pairs of a step scale linearly" % (ctx, nbytes / 1e6),
+            "seconds": out["all"], "value_1thread": nbytes / out["one"] / 1e9, "seconds_1thread": out["one"],
+            "note": "the reference walks heads on one thread (gpt-oss/src/model.rs:439); "
+                    "value uses OpenMP over (query, head) on `cores` threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+    gpu = C.Gpu(0)
+    log("device:", gpu.name())
+    extra = {}
+    if not args.no_extras:
+        extra["c2_single_decode"] = run_single_decode(gpu, args.steps, args.warmup)
+        log("c2", extra["c2_single_decode"])
+        extra["c3_ragged_batch"] = run_ragged(gpu, args.steps, args.warmup)
+        log("c3", extra["c3_ragged_batch"])
+        extra["c4_prefill"] = run_prefill(gpu, args.steps, args.warmup)
+        log("c4", extra["c4_prefill"])
+    r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx)
+    log("c5", r)
+    gpu.close()
+    cpu = None if args.no_cpu else cpu_baseline(0, args.ctx)
+    extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "combine_s_per_step", "step_bytes",
+                                           "kernel_launches_per_step")}
+    line = {
+        "metric": METRIC, "value": r["value_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": r["wall_s_per_step"] * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": r["workload"], "heads": H, "kv_heads": G, "head_dim": D,
+                   "hbm_frac_of_value": r["value_gbs"] / HBM_PEAK_GBS},
+        "roofline": {"bound": "hbm", "kernel": r["kernel"], "achieved": r["kernel_gbs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": r["kernel_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "bytes_per_launch": r["kernel_bytes_per_launch"], "s_per_launch": r["kernel_s_per_launch"]},
+        "cpu_baseline": cpu,
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -133,6 +133,13 @@ int lng_hip_batch_commit(lng_batch *batch, lng_on_done on_done, void *user);
 /* Blocks until a committed batch has finished; gpu_seconds (may be NULL) receives the time
  * between its first and last dispatch on the device (Completed.gpu_time, apple.rs:2219-2221). */
 int lng_hip_batch_wait(lng_batch *batch, double *gpu_seconds);
+/* Per-kernel GPU time, the finer-grained form of the phase accounting in
+ * gpt-oss/src/gpu.rs:247-317 (Profile / PhaseTime). With timing on (set before commit) an
+ * event is recorded after every kernel of the batch; after the batch has finished,
+ * lng_hip_batch_kernel_seconds sums the time and counts the launches of the kernel named
+ * `kernel` (e.g. "lng_decode_bf16_d64"). */
+int lng_hip_batch_set_timing(lng_batch *batch, int enabled);
+int lng_hip_batch_kernel_seconds(lng_batch *batch, const char *kernel, double *seconds, size_t *launches);
 /* Drop of Batch: an uncommitted batch runs nothing (apple.rs:553-561); a committed one is
  * waited for. Its buffers are the caller's again. */
 void lng_hip_batch_drop(lng_batch *batch);

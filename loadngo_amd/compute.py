@@ -95,6 +95,9 @@ SYMBOLS = {
     "lng_hip_batch_commit": (ctypes.c_int, [_P, _ON_DONE, _P]),
     "lng_hip_batch_wait": (ctypes.c_int, [_P, ctypes.POINTER(ctypes.c_double)]),
     "lng_hip_batch_drop": (None, [_P]),
+    "lng_hip_batch_set_timing": (ctypes.c_int, [_P, ctypes.c_int]),
+    "lng_hip_batch_kernel_seconds": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.POINTER(ctypes.c_double),
+                                                    ctypes.POINTER(ctypes.c_size_t)]),
     "lng_hip_check_grouped": (ctypes.c_int, [ctypes.POINTER(_Shape), ctypes.c_int]),
     "lng_hip_attention_grouped": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, ctypes.POINTER(_Slice),
                                                  ctypes.POINTER(_Shape), ctypes.c_int]),
@@ -181,6 +184,14 @@ class DecodeItem:
         self.q_offset, self.out_offset, self.k_offset, self.v_offset = q_offset, out_offset, k_offset, v_offset
         self.sinks_offset = NO_SINKS if sinks_offset is None else sinks_offset
         self.start, self.window, self.slots = start, window, slots
+
+
+def decode_items(items):
+    """A prepared table of ``DecodeItem`` for ``Batch.attention_decode_batched`` (built once,
+    reused every step)."""
+    return (_Item * len(items))(*[
+        _Item(i.q_offset, i.out_offset, i.k_offset, i.v_offset, i.sinks_offset, i.start, i.window, i.slots)
+        for i in items])
 
 
 class Completed:
@@ -341,15 +352,24 @@ class Batch:
 
     def attention_decode_batched(self, q_buffer, k_buffer, v_buffer, out_buffer, sinks_buffer, items, heads,
                                  kv_heads, dim, scale, dtype=BF16):
-        arr = (_Item * len(items))(*[
-            _Item(i.q_offset, i.out_offset, i.k_offset, i.v_offset, i.sinks_offset, i.start, i.window, i.slots)
-            for i in items])
+        arr = items if isinstance(items, ctypes.Array) else decode_items(items)
         _check(library().lng_hip_attention_decode_batched(self._h, q_buffer, k_buffer, v_buffer, out_buffer,
                                                           sinks_buffer, arr, len(items), heads, kv_heads, dim,
                                                           scale, dtype))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))
+
+    def set_timing(self, enabled=True):
+        """Record an event after every kernel so ``kernel_seconds`` can report per-kernel time."""
+        _check(library().lng_hip_batch_set_timing(self._h, int(enabled)))
+
+    def kernel_seconds(self, kernel):
+        """(total seconds, launches) of the kernel named ``kernel`` in this finished batch."""
+        seconds, launches = ctypes.c_double(), ctypes.c_size_t()
+        _check(library().lng_hip_batch_kernel_seconds(self._h, kernel.encode(), ctypes.byref(seconds),
+                                                      ctypes.byref(launches)))
+        return seconds.value, launches.value
 
     def commit(self, on_done=None):
         """apple.rs:2202: submits; ``on_done(Completed)`` runs on a library thread when the GPU

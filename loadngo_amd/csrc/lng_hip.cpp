@@ -65,6 +65,7 @@ struct Table { // one pinned-host / device pair holding row tables of batched di
 
 struct Cmd {
     hipFunction_t fn = nullptr;
+    const char *name = "";
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
     std::vector<char> args;
@@ -120,6 +121,9 @@ struct lng_batch {
     size_t dispatches = 0;
     enum State { Recording, Committed, Done } state = Recording;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool timing = false;
+    std::vector<hipEvent_t> marks; // timing: one event after every command
+    std::vector<double> cmd_seconds;
     lng_on_done on_done = nullptr;
     void *user = nullptr;
     int status = LNG_OK;
@@ -309,6 +313,11 @@ void finish(lng_batch *b) {
         float ms = 0.0f;
         e = hipEventElapsedTime(&ms, b->ev0, b->ev1);
         if (e == hipSuccess) b->seconds = std::max(0.0, (double)ms * 1e-3);
+        b->cmd_seconds.assign(b->marks.size(), 0.0);
+        for (size_t i = 0; e == hipSuccess && i < b->marks.size(); ++i) {
+            e = hipEventElapsedTime(&ms, i ? b->marks[i - 1] : b->ev0, b->marks[i]);
+            if (e == hipSuccess) b->cmd_seconds[i] = std::max(0.0, (double)ms * 1e-3);
+        }
     }
     if (e != hipSuccess) {
         b->status = LNG_ERR_GPU;
@@ -389,6 +398,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     if (!fast) {
         Cmd c;
         c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;
+        c.name = a.dtype == LNG_BF16 ? "lng_attn_generic_bf16" : "lng_attn_generic_f32";
         c.grid[0] = (unsigned)(n_rows * a.heads);
         c.block = 256;
         set_args(c, a);
@@ -411,6 +421,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     }
     Cmd c;
     c.fn = g->decode_bf16_d64;
+    c.name = "lng_decode_bf16_d64";
     c.grid[0] = plan.n_chunks;
     c.grid[1] = (unsigned)(n_rows * a.kv_heads);
     c.block = 256;
@@ -424,6 +435,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     if (plan.n_chunks > 1) {
         Cmd m;
         m.fn = g->decode_combine;
+        m.name = "lng_decode_combine";
         m.grid[0] = (unsigned)(n_rows * a.heads);
         m.block = 64;
         set_args(m, a);
@@ -479,6 +491,7 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         p.scale = s.scale;
         Cmd c;
         c.fn = g->prefill_bf16_d64;
+        c.name = "lng_prefill_bf16_d64";
         c.grid[0] = p.q_tiles;
         c.grid[1] = (unsigned)s.kv_heads;
         c.block = 256;
@@ -746,6 +759,14 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
         void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, c.args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                           HIP_LAUNCH_PARAM_END};
         e = hipModuleLaunchKernel(c.fn, c.grid[0], c.grid[1], c.grid[2], c.block, 1, 1, 0, g->stream, nullptr, config);
+        if (e == hipSuccess && b->timing) {
+            hipEvent_t mark = nullptr;
+            e = hipEventCreate(&mark);
+            if (e == hipSuccess) {
+                b->marks.push_back(mark);
+                e = hipEventRecord(mark, g->stream);
+            }
+        }
     }
     if (e == hipSuccess) e = hipEventRecord(b->ev1, g->stream);
     b->on_done = on_done;
@@ -797,7 +818,31 @@ extern "C" void lng_hip_batch_drop(lng_batch *b) {
     }
     if (b->ev0) hipEventDestroy(b->ev0);
     if (b->ev1) hipEventDestroy(b->ev1);
+    for (hipEvent_t mark : b->marks) hipEventDestroy(mark);
     delete b;
+}
+
+extern "C" int lng_hip_batch_set_timing(lng_batch *b, int enabled) {
+    if (int rc = need_recording(b)) return rc;
+    b->timing = enabled != 0;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_batch_kernel_seconds(lng_batch *b, const char *kernel, double *seconds, size_t *launches) {
+    if (!b || !kernel) return fail(LNG_ERR_DISPATCH, "no batch or no kernel name");
+    if (b->state != lng_batch::Done) return fail(LNG_ERR_DISPATCH, "the batch has not finished");
+    if (!b->timing) return fail(LNG_ERR_DISPATCH, "the batch was not committed with timing on");
+    double total = 0.0;
+    size_t n = 0;
+    for (size_t i = 0; i < b->cmds.size() && i < b->cmd_seconds.size(); ++i) {
+        if (strcmp(b->cmds[i].name, kernel) == 0) {
+            total += b->cmd_seconds[i];
+            n += 1;
+        }
+    }
+    if (seconds) *seconds = total;
+    if (launches) *launches = n;
+    return LNG_OK;
 }
 
 extern "C" int lng_hip_check_grouped(const lng_grouped_shape *shape, int tiled) {
@@ -848,6 +893,7 @@ extern "C" int lng_hip_copy_rows(lng_batch *b, lng_slice src, uint64_t src_strid
     a.dst_dtype = (uint32_t)dst_dtype;
     Cmd c;
     c.fn = b->gpu->copy_rows;
+    c.name = "lng_copy_rows";
     c.grid[0] = (unsigned)((rows * width + 255) / 256);
     c.block = 256;
     set_args(c, a);
@@ -942,6 +988,7 @@ extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, ui
     a.dtype = (uint32_t)dtype;
     Cmd c;
     c.fn = b->gpu->fill_synthetic;
+    c.name = "lng_fill_synthetic";
     c.grid[0] = (unsigned)std::min<uint64_t>((a.n + 255) / 256, 256u * 64u);
     c.block = 256;
     set_args(c, a);

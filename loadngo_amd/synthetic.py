@@ -19,3 +19,15 @@ def synthetic_values(n, seed, scale=1.0, period=0, first=0):
     s = ((z & m) + ((z >> np.uint64(16)) & m) + ((z >> np.uint64(32)) & m) + (z >> np.uint64(48))).astype(np.int64)
     factor = np.float32(scale) / SYNTH_STD
     return (s - 131070).astype(np.float32) * factor
+
+
+def bf16_bits(x):
+    """f32 -> bf16 bit patterns (uint16), round to nearest even."""
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    bias = np.uint32(0x7FFF) + ((b >> np.uint32(16)) & np.uint32(1))
+    return ((b + bias) >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_widen(bits):
+    """bf16 bit patterns -> f32 (exact)."""
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
