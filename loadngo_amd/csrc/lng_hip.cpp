@@ -473,7 +473,7 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     lng_gpu *g = b->gpu;
     const bool aligned16 = ((q.offset | k.offset | v.offset | out.offset) & 15u) == 0;
 
-    if (tiled && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 16 && aligned16 && g->prefill_bf16_d64) {
+    if (tiled && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16) {
         lng_k_prefill p{};
         p.q = (const char *)oq.buf->ptr + q.offset;
         p.k = (const char *)ok.buf->ptr + k.offset;
@@ -482,19 +482,18 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         p.sinks = sinks ? (const float *)((const char *)os.buf->ptr + sinks->offset) : nullptr;
         p.t = s.t;
         p.start = s.start;
-        p.window = s.window;
+        p.window = s.window >= end ? LNG_WINDOW_FULL : s.window; // a window over everything is no window
         p.slots = s.slots;
         p.heads = (uint32_t)s.heads;
         p.kv_heads = (uint32_t)s.kv_heads;
         p.dim = (uint32_t)s.dim;
-        p.q_tiles = (uint32_t)((s.t + 127) / 128);
+        p.q_tiles = (uint32_t)((s.t + 63) / 64); // PF_BM query rows per workgroup
         p.scale = s.scale;
         Cmd c;
         c.fn = g->prefill_bf16_d64;
         c.name = "lng_prefill_bf16_d64";
-        c.grid[0] = p.q_tiles;
-        c.grid[1] = (unsigned)s.kv_heads;
-        c.block = 256;
+        c.grid[0] = p.q_tiles * (unsigned)s.kv_heads; // kv head fastest: one XCD's L2 per kv head
+        c.block = 512;
         set_args(c, p);
         b->cmds.push_back(std::move(c));
         b->dispatches += 1;
@@ -563,7 +562,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_attn_generic_bf16", &g->generic_bf16, true},
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
         {"lng_decode_combine", &g->decode_combine, true},
-        {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, false},
+        {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
     };

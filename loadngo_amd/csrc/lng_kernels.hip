@@ -461,3 +461,242 @@ extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill 
         }
     }
 }
+
+// =============================================================================================
+// Prompt-pass kernel, bf16, head width 64, up to 8 query heads per kv head.
+//
+// A workgroup (8 wavefronts) takes 64 consecutive query positions and ALL query heads of one
+// kv head: wavefront w handles query block w&1 (32 positions) and head pair w>>1, so every
+// K/V tile staged in LDS is used by every head of the group. Workgroup ids put the kv head
+// fastest (id % kv_heads): consecutive ids go to different XCDs, so each XCD's L2 keeps one kv
+// head's K and V; the longest (latest) query tiles are issued first.
+//
+// Per 64-key tile, everything per query is lane-local: the products are computed transposed,
+//   S^T[key][query] = K . Q^T   (v_mfma_f32_32x32x16_bf16; A = K rows read from LDS with
+//                                ds_read_b128, B = Q^T held in registers for the whole pass)
+// so lane l owns query l%32 and 16 of each 32 keys; the row maximum and sum need one exchange
+// with lane l^32 only. exp'd scores narrowed to bf16 are directly the B operand of
+//   O^T[dim][query] += V^T . P^T (A = V^T read from the row-major V tile with the transposing
+//                                LDS read ds_read_b64_tr_b16: a 16-lane block reads 4 keys x 16
+//                                dims and each lane receives 4 keys of one dim)
+// and the accumulator column, like the softmax state, belongs to the lane's query. The sink
+// initialises the running maximum and contributes 1 to the running sum (it is one more logit
+// with no value); tiles wholly outside the causal/window band are never visited.
+// =============================================================================================
+#define PF_BM 64
+#define PF_BN 64
+#define PF_THREADS 512
+#define PF_KSTRIDE 72 // bf16 elements per LDS row (144 bytes): conflict-free 16-byte row reads
+#define PF_VSTRIDE 72
+
+typedef short short4v __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8 lds_read_tr8(const uint16_t *p0, const uint16_t *p1) {
+    // two transposing reads: slots 0..3 and 4..7 of the lane's k-group
+    const short4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p0);
+    const short4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v *)p1);
+    typedef short short8v __attribute__((ext_vector_type(8)));
+    const short8v both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+}
+
+extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(lng_k_prefill a) {
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
+
+    const uint32_t g = blockIdx.x % a.kv_heads;
+    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = tid >> 6;
+    const uint32_t n = lane & 31u;  // query within the wave's block
+    const uint32_t hh = lane >> 5;  // which half of the k-slots / of each 8 accumulator rows
+    const uint32_t qb = wave & 1u;
+    const uint32_t hp = wave >> 1;
+
+    const uint64_t q0 = (uint64_t)qtile * PF_BM;              // first query row of the workgroup
+    const uint64_t rows_here = a.t - q0 < PF_BM ? a.t - q0 : PF_BM;
+    const uint64_t end = a.start + a.t;                        // positions in the cache
+    const uint64_t pos_first = a.start + q0;                   // position of the first query row
+    const uint64_t pos_last = pos_first + rows_here - 1;       // of the last real one
+    const uint64_t kfirst = first_visible(pos_first, a.window);
+    const uint64_t tile0 = kfirst & ~(uint64_t)(PF_BN - 1);
+    const uint32_t n_tiles = (uint32_t)((pos_last - tile0) / PF_BN + 1);
+    const bool ring = a.slots < end;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
+
+    // ---- this wavefront's queries -----------------------------------------------------------
+    const uint64_t my_row = q0 + 32u * qb + n;      // query row of this lane
+    const uint64_t my_pos = a.start + my_row;       // its absolute position
+    const bool row_ok = my_row < a.t;
+    bool head_ok[2];
+    uint32_t head[2];
+    bf16x8 qreg[2][4];
+    float m[2], l[2];
+    floatx16 ot[2][2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const uint32_t slot = hp * 2u + h;
+        head_ok[h] = slot < group;
+        head[h] = g * group + (head_ok[h] ? slot : 0u);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (row_ok && head_ok[h]) {
+                raw = *(const uint4 *)(a.q + ((my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
+            }
+            qreg[h][ks] = as_bf16x8(raw);
+        }
+        const float sink2 = (a.sinks && head_ok[h]) ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+        m[h] = sink2;
+        l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
+        }
+    }
+    const bool wave_active = head_ok[0]; // head slots fill from 0: slot 2hp missing => nothing to do
+    const float sl2 = a.scale * LNG_LOG2E;
+
+    // ---- tile loader: one 16-byte chunk of K and of V per thread --------------------------------
+    const uint32_t ld_key = tid >> 3;  // 0..63
+    const uint32_t ld_chunk = tid & 7u;
+    const char *kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
+    const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
+    auto fetch = [&](uint32_t tile, uint4 &kr, uint4 &vr) {
+        uint64_t p = tile0 + (uint64_t)tile * PF_BN + ld_key;
+        p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway
+        const uint64_t r = ring ? (uint32_t)p % (uint32_t)a.slots : p;
+        kr = *(const uint4 *)(kbase + r * row_bytes);
+        vr = *(const uint4 *)(vbase + r * row_bytes);
+    };
+    auto stash = [&](uint32_t buf, const uint4 &kr, const uint4 &vr) {
+        *(uint4 *)(&s_k[buf][ld_key * PF_KSTRIDE + ld_chunk * 8u]) = kr;
+        *(uint4 *)(&s_v[buf][ld_key * PF_VSTRIDE + ld_chunk * 8u]) = vr;
+    };
+
+    uint4 kr, vr;
+    fetch(0, kr, vr);
+    stash(0, kr, vr);
+    __syncthreads();
+
+    // per-lane constant parts of the LDS addresses
+    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
+    const uint32_t L = lane & 15u;
+    const uint32_t blk16 = lane >> 4;                                     // 16-lane block 0..3
+    // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
+    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+
+    for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+        const uint32_t buf = tile & 1u;
+        if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
+        if (wave_active) {
+            const uint64_t kt0 = tile0 + (uint64_t)tile * PF_BN; // position of the tile's first key
+            // interior tiles need no mask: every key visible to every query of the workgroup
+            const bool need_mask = kt0 + (PF_BN - 1) > pos_first ||
+                                   (a.window != LNG_WINDOW_FULL && kt0 + a.window < pos_first + PF_BM);
+            // ---- S^T = K . Q^T for both heads ---------------------------------------------------
+            floatx16 st[2][2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) st[h][kb][i] = 0.0f;
+                }
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    const bf16x8 ka = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
+                    st[0][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][ks], st[0][kb], 0, 0, 0);
+                    if (head_ok[1]) st[1][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][ks], st[1][kb], 0, 0, 0);
+                }
+            }
+            // ---- online softmax, one query per lane ---------------------------------------------
+            bf16x8 pb[2][4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (h == 1 && !head_ok[1]) break;
+                float tmax = LNG_NEG_INF;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        float x = st[h][kb][i] * sl2;
+                        if (need_mask) {
+                            const uint64_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
+                            const bool vis = kp <= my_pos && (a.window == LNG_WINDOW_FULL || kp + a.window > my_pos);
+                            x = vis ? x : LNG_NEG_INF;
+                        }
+                        st[h][kb][i] = x;
+                        tmax = fmaxf(tmax, x);
+                    }
+                }
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                const float m_new = fmaxf(m[h], tmax);
+                const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+                float psum = 0.0f;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float pw = __builtin_amdgcn_exp2f(st[h][kb][i] - m_safe);
+                        st[h][kb][i] = pw;
+                        psum += pw;
+                    }
+                }
+                l[h] = l[h] * alpha + psum;
+                m[h] = m_new;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int kb = j >> 1, o = 8 * (j & 1);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pb[h][j][e] = (__bf16)st[h][kb][o + e];
+                }
+            }
+            // ---- O^T += V^T . P^T -------------------------------------------------------------------
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+                    const uint16_t *vp = &s_v[buf][v_lane_off + (16 * j) * PF_VSTRIDE + 32 * db];
+                    const bf16x8 va = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                    ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][j], ot[0][db], 0, 0, 0);
+                    if (head_ok[1]) ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][j], ot[1][db], 0, 0, 0);
+                }
+            }
+        }
+        if (tile + 1 < n_tiles) stash(buf ^ 1u, kr, vr);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------
+    if (wave_active && row_ok) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (!head_ok[h]) continue;
+            const float total = l[h] + __shfl_xor(l[h], 32, 64);
+            const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+            uint16_t *op = (uint16_t *)a.out + (my_row * a.heads + head[h]) * 64u;
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                for (int blk = 0; blk < 4; ++blk) {
+                    ushort4 w;
+                    w.x = f32_to_bf16_bits(ot[h][db][4 * blk + 0] * inv);
+                    w.y = f32_to_bf16_bits(ot[h][db][4 * blk + 1] * inv);
+                    w.z = f32_to_bf16_bits(ot[h][db][4 * blk + 2] * inv);
+                    w.w = f32_to_bf16_bits(ot[h][db][4 * blk + 3] * inv);
+                    *(ushort4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
+                }
+            }
+        }
+    }
+}

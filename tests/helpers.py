@@ -70,6 +70,8 @@ def ring_layout(all_rows, t, start, slots, tiled, fill=None):
         rows = (end + 31) // 32 * 32
     if fill is None:
         fill = 0.0 if tiled else np.nan
+    if all_rows.dtype == np.uint16 and isinstance(fill, float):
+        fill = 0x7FC0 if np.isnan(fill) else 0  # bf16 bit patterns: quiet NaN or zero
     out = np.full((rows,) + all_rows.shape[1:], fill, dtype=all_rows.dtype)
     for p in range(max(0, end - slots), end):
         out[p % slots] = all_rows[p]

@@ -284,3 +284,47 @@ def test_synthetic_fill_is_reproducible_on_the_host(gpu):
     assert np.array_equal(got32, synthetic_values(n, seed, scale, 0))
     assert np.array_equal(got, to_bf16_bits(synthetic_values(n, seed, scale, period)))
     assert abs(float(got32.std()) - scale) < 0.02 and abs(float(got32.mean())) < 0.03
+
+
+# ---- prompt passes in bf16 (MFMA kernel) -----------------------------------------------------
+@pytest.mark.parametrize("t,start,window,slots,heads,kv_heads", [
+    (64, 0, FULL, 64, 64, 8), (33, 5, FULL, 64, 64, 8), (100, 37, FULL, 160, 64, 8), (65, 0, 1, 96, 64, 8),
+    (128, 64, 64, 192, 64, 8), (200, 1400, 1024, 1536, 16, 2), (512, 2600, 128, 640, 8, 8), (97, 31, 40, 128, 16, 4),
+    (130, 1000, 128, 320, 6, 2), (77, 700, FULL, 4096, 10, 2), (40, 97, 7, 64, 4, 1), (256, 0, 100, 256, 32, 8),
+])
+def test_prefill_bf16_matches_the_cpu_reference(gpu, t, start, window, slots, heads, kv_heads):
+    end = start + t
+    q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    kr, vr = ring_layout(kb, t, start, slots, True), ring_layout(vb, t, start, slots, True)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    want = oracle.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS)
+    got = run_attention(gpu, qb, kr, vr, sinks, shape, True, C.BF16)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+    want_none = oracle.attention_bf16(qb, kb, vb, None, start, window=window, scale=0.125, threads=THREADS)
+    none = run_attention(gpu, qb, kr, vr, None, shape, True, C.BF16)
+    assert max_error(from_bf16_bits(none), from_bf16_bits(want_none)) < BF16_TOL
+    # the row-by-row operator gives the same pass (decode == prefill, row for row)
+    krp, vrp = ring_layout(kb, t, start, slots, False), ring_layout(vb, t, start, slots, False)
+    plain = run_attention(gpu, qb, krp, vrp, sinks, shape, False, C.BF16)
+    assert max_error(from_bf16_bits(plain), from_bf16_bits(want)) < BF16_TOL
+
+
+@pytest.mark.parametrize("window", [FULL, 128])
+def test_config4_prefill_8192_sampled_rows(gpu, window):
+    """The 8192-position prompt pass at its real size; a sample of query rows (first, last,
+    tile edges, random) is checked against the CPU reference, every head of each."""
+    t, heads, kv_heads = 8192, 64, 8
+    rng = np.random.default_rng(44)
+    qb = to_bf16_bits((rng.standard_normal((t, heads, 64), dtype=np.float32) * 0.5))
+    kb = to_bf16_bits((rng.standard_normal((t, kv_heads, 64), dtype=np.float32) * 0.5))
+    vb = to_bf16_bits((rng.standard_normal((t, kv_heads, 64), dtype=np.float32) * 0.5))
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    shape = C.GroupedShape(t, 0, heads, kv_heads, 64, window, t, 0.125)
+    got = run_attention(gpu, qb, kb, vb, sinks, shape, True, C.BF16)
+    assert not np.isnan(from_bf16_bits(got)).any()
+    rows = sorted(set([0, 1, 31, 32, 63, 64, 127, 128, 129, 4095, 4096, 8190, 8191] +
+                      [int(x) for x in rng.integers(0, t, 40)]))
+    want = oracle.attention_rows_f32(from_bf16_bits(qb[rows]), from_bf16_bits(kb), from_bf16_bits(vb), sinks, rows,
+                                     window=window, scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(got[rows]), want) < BF16_TOL
