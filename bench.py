@@ -283,6 +283,8 @@ def main():
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4: run just these and print their results "
+                    "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -291,6 +293,12 @@ def main():
     gpu = C.Gpu(0)
     log("device:", gpu.name())
     extra = {}
+    if args.only:
+        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill}
+        for name in args.only.split(","):
+            print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
+        gpu.close()
+        return
     if not args.no_extras:
         extra["c2_single_decode"] = run_single_decode(gpu, args.steps, args.warmup)
         log("c2", extra["c2_single_decode"])

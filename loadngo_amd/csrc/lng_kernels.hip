@@ -12,6 +12,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "lng_kernel_args.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -489,7 +491,16 @@ extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill 
 #define PF_KSTRIDE 72 // bf16 elements per LDS row (144 bytes): conflict-free 16-byte row reads
 #define PF_VSTRIDE 72
 
+#define PF_TAU 8.0f
 typedef short short4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// max of x over lanes l and l^32, without LDS: swap the upper half of one copy with the
+// lower half of another, then both copies hold one half's value in every lane.
+__device__ __forceinline__ float other_half_max(float x) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
 
 __device__ __forceinline__ bf16x8 lds_read_tr8(const uint16_t *p0, const uint16_t *p1) {
     // two transposing reads: slots 0..3 and 4..7 of the lane's k-group
@@ -509,47 +520,53 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     const uint32_t group = a.heads / a.kv_heads;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
-    const uint32_t wave = tid >> 6;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6); // scalar: branches on it are uniform
     const uint32_t n = lane & 31u;  // query within the wave's block
     const uint32_t hh = lane >> 5;  // which half of the k-slots / of each 8 accumulator rows
     const uint32_t qb = wave & 1u;
     const uint32_t hp = wave >> 1;
 
-    const uint64_t q0 = (uint64_t)qtile * PF_BM;              // first query row of the workgroup
-    const uint64_t rows_here = a.t - q0 < PF_BM ? a.t - q0 : PF_BM;
-    const uint64_t end = a.start + a.t;                        // positions in the cache
-    const uint64_t pos_first = a.start + q0;                   // position of the first query row
-    const uint64_t pos_last = pos_first + rows_here - 1;       // of the last real one
-    const uint64_t kfirst = first_visible(pos_first, a.window);
-    const uint64_t tile0 = kfirst & ~(uint64_t)(PF_BN - 1);
-    const uint32_t n_tiles = (uint32_t)((pos_last - tile0) / PF_BN + 1);
+    // Positions fit 32 bits (the host refuses shapes whose counts do not).
+    const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
+    const uint32_t q0 = qtile * PF_BM;                         // first query row of the workgroup
+    const uint32_t rows_here = t - q0 < PF_BM ? t - q0 : PF_BM;
+    const uint32_t end = start + t;                            // positions in the cache
+    const uint32_t pos_first = start + q0;                     // position of the first query row
+    const uint32_t pos_last = pos_first + rows_here - 1;       // of the last real one
+    const bool windowed = a.window != LNG_WINDOW_FULL;         // the host maps window >= end to FULL
+    const uint32_t window = windowed ? (uint32_t)a.window : 0u;
+    const uint32_t kfirst = (windowed && pos_first + 1 > window) ? pos_first + 1 - window : 0u;
+    const uint32_t tile0 = kfirst & ~(uint32_t)(PF_BN - 1);
+    const uint32_t n_tiles = (pos_last - tile0) / PF_BN + 1;
     const bool ring = a.slots < end;
+    const uint32_t slots = (uint32_t)a.slots;
     const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
 
-    // ---- this wavefront's queries -----------------------------------------------------------
-    const uint64_t my_row = q0 + 32u * qb + n;      // query row of this lane
-    const uint64_t my_pos = a.start + my_row;       // its absolute position
-    const bool row_ok = my_row < a.t;
-    bool head_ok[2];
+    // ---- this wavefront's queries and its two heads -------------------------------------------
+    // A wavefront whose second head slot is past the group computes its first head twice and
+    // stores it once; one whose first slot is past the group only helps loading tiles.
+    const uint32_t my_row = q0 + 32u * qb + n;      // query row of this lane
+    const uint32_t my_pos = start + my_row;         // its absolute position
+    const bool row_ok = my_row < t;
+    const bool wave_active = hp * 2u < group;
+    const bool second_ok = hp * 2u + 1u < group;
     uint32_t head[2];
+    head[0] = g * group + (wave_active ? hp * 2u : 0u);
+    head[1] = second_ok ? head[0] + 1u : head[0];
     bf16x8 qreg[2][4];
     float m[2], l[2];
     floatx16 ot[2][2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-        const uint32_t slot = hp * 2u + h;
-        head_ok[h] = slot < group;
-        head[h] = g * group + (head_ok[h] ? slot : 0u);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             uint4 raw = make_uint4(0, 0, 0, 0);
-            if (row_ok && head_ok[h]) {
-                raw = *(const uint4 *)(a.q + ((my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
+            if (row_ok) {
+                raw = *(const uint4 *)(a.q + (((uint64_t)my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
             }
             qreg[h][ks] = as_bf16x8(raw);
         }
-        const float sink2 = (a.sinks && head_ok[h]) ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
-        m[h] = sink2;
+        m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
         l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
@@ -557,8 +574,10 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
             for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
         }
     }
-    const bool wave_active = head_ok[0]; // head slots fill from 0: slot 2hp missing => nothing to do
     const float sl2 = a.scale * LNG_LOG2E;
+    bf16x2 ones2;
+    ones2[0] = (__bf16)1.0f;
+    ones2[1] = (__bf16)1.0f;
 
     // ---- tile loader: one 16-byte chunk of K and of V per thread --------------------------------
     const uint32_t ld_key = tid >> 3;  // 0..63
@@ -566,11 +585,11 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     const char *kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
     const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
     auto fetch = [&](uint32_t tile, uint4 &kr, uint4 &vr) {
-        uint64_t p = tile0 + (uint64_t)tile * PF_BN + ld_key;
+        uint32_t p = tile0 + tile * PF_BN + ld_key;
         p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway
-        const uint64_t r = ring ? (uint32_t)p % (uint32_t)a.slots : p;
-        kr = *(const uint4 *)(kbase + r * row_bytes);
-        vr = *(const uint4 *)(vbase + r * row_bytes);
+        const uint32_t r = ring ? p % slots : p;
+        kr = *(const uint4 *)(kbase + (uint64_t)r * row_bytes);
+        vr = *(const uint4 *)(vbase + (uint64_t)r * row_bytes);
     };
     auto stash = [&](uint32_t buf, const uint4 &kr, const uint4 &vr) {
         *(uint4 *)(&s_k[buf][ld_key * PF_KSTRIDE + ld_chunk * 8u]) = kr;
@@ -589,102 +608,127 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
     const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
 
-    for (uint32_t tile = 0; tile < n_tiles; ++tile) {
+    // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
+    // carries no position arithmetic at all.
+    auto step = [&](auto mask_tag, uint32_t tile) {
+        constexpr bool MASK = decltype(mask_tag)::value;
         const uint32_t buf = tile & 1u;
         if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
         if (wave_active) {
-            const uint64_t kt0 = tile0 + (uint64_t)tile * PF_BN; // position of the tile's first key
-            // interior tiles need no mask: every key visible to every query of the workgroup
-            const bool need_mask = kt0 + (PF_BN - 1) > pos_first ||
-                                   (a.window != LNG_WINDOW_FULL && kt0 + a.window < pos_first + PF_BM);
-            // ---- S^T = K . Q^T for both heads ---------------------------------------------------
-            floatx16 st[2][2];
+            const uint32_t kt0 = tile0 + tile * PF_BN; // position of the tile's first key
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < 2; ++kb) { // the tile's two blocks of 32 keys
+                // ---- S^T = K . Q^T, both heads ------------------------------------------------------
+                bf16x8 ka[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
+                }
+                floatx16 st[2];
 #pragma unroll
                 for (int h = 0; h < 2; ++h) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) st[h][kb][i] = 0.0f;
+                    for (int i = 0; i < 16; ++i) st[h][i] = 0.0f;
                 }
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
-                    const bf16x8 ka = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
-                    st[0][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[0][ks], st[0][kb], 0, 0, 0);
-                    if (head_ok[1]) st[1][kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qreg[1][ks], st[1][kb], 0, 0, 0);
+                    st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[0][ks], st[0], 0, 0, 0);
+                    st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[1][ks], st[1], 0, 0, 0);
                 }
-            }
-            // ---- online softmax, one query per lane ---------------------------------------------
-            bf16x8 pb[2][4];
+                // V^T operands of this block: two groups of 16 keys x two halves of the head width;
+                // issued now, their LDS latency hides behind the softmax arithmetic
+                bf16x8 va[2][2];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                if (h == 1 && !head_ok[1]) break;
-                float tmax = LNG_NEG_INF;
+                for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
+                    for (int db = 0; db < 2; ++db) {
+                        const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                        va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                    }
+                }
+                // ---- online softmax, one query per lane -----------------------------------------------
+                // The running maximum only moves when the block's maximum exceeds it by PF_TAU (log2
+                // domain): weights then stay below 2^PF_TAU, and the accumulators are rescaled only
+                // on the rare blocks where some lane's maximum moved. The normaliser uses the same
+                // maximum, so the result is the same softmax.
+                bf16x8 pb[2][2];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        float x = st[h][kb][i] * sl2;
-                        if (need_mask) {
-                            const uint64_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
-                            const bool vis = kp <= my_pos && (a.window == LNG_WINDOW_FULL || kp + a.window > my_pos);
-                            x = vis ? x : LNG_NEG_INF;
+                for (int h = 0; h < 2; ++h) {
+                    if constexpr (MASK) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const uint32_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
+                            const bool vis = kp <= my_pos && (!windowed || kp + window > my_pos);
+                            st[h][i] = vis ? st[h][i] : LNG_NEG_INF;
                         }
-                        st[h][kb][i] = x;
-                        tmax = fmaxf(tmax, x);
                     }
-                }
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-                const float m_new = fmaxf(m[h], tmax);
-                const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
-                const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
-                float psum = 0.0f;
+                    float tmax = LNG_NEG_INF;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
+                    for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
+                    tmax = other_half_max(tmax) * sl2; // scale > 0: max commutes with it
+                    const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
+                    const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                    if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
+                        const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+                        l[h] *= alpha;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const float pw = __builtin_amdgcn_exp2f(st[h][kb][i] - m_safe);
-                        st[h][kb][i] = pw;
-                        psum += pw;
+                        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
+                        }
+                        m[h] = m_new;
                     }
+                    float psum = 0.0f;
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                        for (int e = 0; e < 8; e += 2) {
+                            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[h][8 * jj + e], sl2, -m_safe));
+                            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[h][8 * jj + e + 1], sl2, -m_safe));
+                            bf16x2 pr;
+                            pr[0] = (__bf16)p0;
+                            pr[1] = (__bf16)p1;
+                            pb[h][jj][e] = pr[0];
+                            pb[h][jj][e + 1] = pr[1];
+                            // the normaliser sums the same rounded weights the product uses
+                            psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum, false);
+                        }
+                    }
+                    l[h] += psum;
                 }
-                l[h] = l[h] * alpha + psum;
-                m[h] = m_new;
+                // ---- O^T += V^T . P^T ---------------------------------------------------------------------
 #pragma unroll
-                for (int db = 0; db < 2; ++db) {
+                for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
-                }
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int kb = j >> 1, o = 8 * (j & 1);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) pb[h][j][e] = (__bf16)st[h][kb][o + e];
-                }
-            }
-            // ---- O^T += V^T . P^T -------------------------------------------------------------------
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-#pragma unroll
-                for (int db = 0; db < 2; ++db) {
-                    const uint16_t *vp = &s_v[buf][v_lane_off + (16 * j) * PF_VSTRIDE + 32 * db];
-                    const bf16x8 va = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
-                    ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[0][j], ot[0][db], 0, 0, 0);
-                    if (head_ok[1]) ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, pb[1][j], ot[1][db], 0, 0, 0);
+                    for (int db = 0; db < 2; ++db) {
+                        ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[0][jj], ot[0][db], 0, 0, 0);
+                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
+                    }
                 }
             }
         }
         if (tile + 1 < n_tiles) stash(buf ^ 1u, kr, vr);
         __syncthreads();
-    }
+    };
+    // interior tiles need no mask: every key visible to every query of the workgroup
+    auto edge = [&](uint32_t tile) {
+        const uint32_t kt0 = tile0 + tile * PF_BN;
+        return kt0 + (PF_BN - 1) > pos_first || (windowed && kt0 + window < pos_first + PF_BM);
+    };
+    uint32_t tile = 0;
+    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tile);   // window edge
+    for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tile); // interior
+    for (; tile < n_tiles; ++tile) step(std::true_type{}, tile);                 // diagonal
+
 
     // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------
     if (wave_active && row_ok) {
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-            if (!head_ok[h]) continue;
+            if (h == 1 && !second_ok) continue;
             const float total = l[h] + __shfl_xor(l[h], 32, 64);
             const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-            uint16_t *op = (uint16_t *)a.out + (my_row * a.heads + head[h]) * 64u;
+            uint16_t *op = (uint16_t *)a.out + ((uint64_t)my_row * a.heads + head[h]) * 64u;
 #pragma unroll
             for (int db = 0; db < 2; ++db) {
 #pragma unroll
