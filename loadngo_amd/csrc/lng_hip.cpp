@@ -551,7 +551,13 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         g->name = prop.gcnArchName;
         g->cus = (unsigned)prop.multiProcessorCount;
     }
-    hipError_t e = hipModuleLoadData(&g->module, lng_hsaco_begin);
+    // LNG_HSACO names a code object file to load instead of the embedded one (kernel development).
+    hipError_t e;
+    if (const char *path = getenv("LNG_HSACO")) {
+        e = hipModuleLoad(&g->module, path);
+    } else {
+        e = hipModuleLoadData(&g->module, lng_hsaco_begin);
+    }
     if (e != hipSuccess) {
         const int rc = fail(LNG_ERR_COMPILE, "the gfx950 code object does not load on %s: %s", g->name.c_str(), hip_text(e));
         delete g;
