@@ -88,20 +88,18 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
         batch.commit()
         done = batch.wait()
         ks = batch.kernel_seconds("lng_decode_bf16_d64") if timing else (0.0, 0)
-        cs = batch.kernel_seconds("lng_decode_combine") if timing else (0.0, 0)
         batch.drop()
-        return done.gpu_time, ks, cs
+        return done.gpu_time, ks
 
     for _ in range(warmup):
         step(False)
     t0 = time.perf_counter()
-    gpu_s = kern_s = comb_s = 0.0
+    gpu_s = kern_s = 0.0
     launches = 0
     for _ in range(steps):
-        g, (ks, kn), (cs, _) = step(True)
+        g, (ks, kn) = step(True)
         gpu_s += g
         kern_s += ks
-        comb_s += cs
         launches += kn
     wall = time.perf_counter() - t0
     for b in bufs:
@@ -122,7 +120,6 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
         "kernel_bytes_per_launch": per_launch_bytes,
         "kernel_s_per_launch": per_launch_s,
         "kernel_gbs": per_launch_bytes / per_launch_s / 1e9,
-        "combine_s_per_step": comb_s / steps,
     }
 
 
@@ -310,8 +307,7 @@ def main():
     log("c5", r)
     gpu.close()
     cpu = None if args.no_cpu else cpu_baseline(0, args.ctx)
-    extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "combine_s_per_step", "step_bytes",
-                                           "kernel_launches_per_step")}
+    extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "step_bytes", "kernel_launches_per_step")}
     line = {
         "metric": METRIC, "value": r["value_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["wall_s_per_step"] * 1e3, "higher_is_better": True,

@@ -90,8 +90,7 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_combine = nullptr, prefill_bf16_d64 = nullptr, copy_rows = nullptr,
-                  fill_synthetic = nullptr;
+                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -99,7 +98,8 @@ struct lng_gpu {
     std::vector<Table> free_tables;
     float *scratch_o = nullptr;  // split-K partial outputs, grown on demand
     float *scratch_ml = nullptr; // split-K partial (max, sum)
-    size_t scratch_o_len = 0, scratch_ml_len = 0;
+    uint32_t *tickets = nullptr; // split-K arrival counters, zero whenever no dispatch is running
+    size_t scratch_o_len = 0, scratch_ml_len = 0, tickets_len = 0;
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
     std::atomic<long> live_buffers{0};
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
@@ -240,8 +240,22 @@ template <typename A> void set_args(Cmd &c, const A &a) {
 
 // Device scratch for split-K partials, shared by every dispatch of the gpu: dispatches run
 // in order on one stream, so the next one starts after the previous combine has read it.
-int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats) {
+int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats, size_t n_tickets) {
     std::lock_guard<std::mutex> lock(g->mu);
+    if (n_tickets > g->tickets_len) {
+        void *p = nullptr;
+        const size_t want = std::max(n_tickets, g->tickets_len * 2);
+        if (hipMalloc(&p, want * sizeof(uint32_t)) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte scratch buffer", want * sizeof(uint32_t));
+        // Zeroed on the dispatch stream: later dispatches are ordered after it, earlier ones keep
+        // the retired counters they were recorded with.
+        if (hipMemsetAsync(p, 0, want * sizeof(uint32_t), g->stream) != hipSuccess) {
+            hipFree(p);
+            return fail(LNG_ERR_GPU, "could not clear the scratch counters");
+        }
+        if (g->tickets) g->retired.push_back(g->tickets);
+        g->tickets = (uint32_t *)p;
+        g->tickets_len = want;
+    }
     if (o_floats > g->scratch_o_len) {
         void *p = nullptr;
         const size_t want = std::max(o_floats, g->scratch_o_len * 2);
@@ -383,7 +397,8 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     const uint64_t per_wg = (total * kv_heads + g->decode_wgs - 1) / g->decode_wgs;
     uint64_t chunk = (per_wg + 127) / 128 * 128;
     chunk = std::max<uint64_t>(chunk, 128);
-    chunk = std::min<uint64_t>(chunk, 1u << 20);
+    // no row may have more than LNG_MAX_CHUNKS chunks (the merge keeps one weight per chunk in LDS)
+    chunk = std::max<uint64_t>(chunk, ((longest + LNG_MAX_CHUNKS - 1) / LNG_MAX_CHUNKS + 127) / 128 * 128);
     p.chunk = (uint32_t)chunk;
     p.n_chunks = (uint32_t)((longest + chunk - 1) / chunk);
     return p;
@@ -415,9 +430,12 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     a.n_chunks = plan.n_chunks;
     if (plan.n_chunks > 1) {
         const size_t slots = n_rows * a.kv_heads * (size_t)plan.n_chunks * group;
-        if (int rc = reserve_scratch(g, slots * 64, slots * 2)) return rc;
+        if (int rc = reserve_scratch(g, slots * 64, slots * 2, n_rows * (size_t)a.kv_heads)) return rc;
         a.partial_o = g->scratch_o;
         a.partial_ml = g->scratch_ml;
+        a.tickets = g->tickets;
+        // Small grids merge inside the kernel; large ones with a second dispatch.
+        a.fused = (uint64_t)plan.n_chunks * n_rows * a.kv_heads <= 4ull * g->cus ? 1u : 0u;
     }
     Cmd c;
     c.fn = g->decode_bf16_d64;
@@ -432,12 +450,12 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         c.copy_len = n_rows * sizeof(lng_k_row);
     }
     b->cmds.push_back(std::move(c));
-    if (plan.n_chunks > 1) {
+    if (plan.n_chunks > 1 && !a.fused) {
         Cmd m;
-        m.fn = g->decode_combine;
-        m.name = "lng_decode_combine";
-        m.grid[0] = (unsigned)(n_rows * a.heads);
-        m.block = 64;
+        m.fn = g->decode_merge;
+        m.name = "lng_decode_merge";
+        m.grid[1] = (unsigned)(n_rows * a.kv_heads);
+        m.block = 256;
         set_args(m, a);
         b->cmds.push_back(std::move(m));
     }
@@ -567,7 +585,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_attn_generic_f32", &g->generic_f32, true},
         {"lng_attn_generic_bf16", &g->generic_bf16, true},
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
-        {"lng_decode_combine", &g->decode_combine, true},
+        {"lng_decode_merge", &g->decode_merge, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
@@ -613,6 +631,7 @@ extern "C" void lng_hip_close(lng_gpu *g) {
     for (void *p : g->retired) hipFree(p);
     if (g->scratch_o) hipFree(g->scratch_o);
     if (g->scratch_ml) hipFree(g->scratch_ml);
+    if (g->tickets) hipFree(g->tickets);
     hipStreamDestroy(g->stream);
     hipModuleUnload(g->module);
     delete g;

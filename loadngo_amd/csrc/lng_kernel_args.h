@@ -23,6 +23,7 @@ typedef struct lng_k_attn {
     const lng_k_row *rows;    /* device table of n_rows rows, or NULL: derive row i from `first` */
     float *partial_o;         /* split-K scratch: [row][kv_head][chunk][group][dim] f32 */
     float *partial_ml;        /* split-K scratch: [row][kv_head][chunk][group][2] f32 (max, sum) */
+    uint32_t *tickets;        /* split-K scratch: [row][kv_head] arrival counters, zero between dispatches */
     lng_k_row first;          /* row 0 when rows == NULL; row i: q/out advance by one row, start by i */
     uint32_t n_rows;
     uint32_t heads;
@@ -31,8 +32,12 @@ typedef struct lng_k_attn {
     uint32_t chunk;           /* positions per workgroup along the cache (multiple of 128) */
     uint32_t n_chunks;        /* workgroups along the cache = ceil(longest visible run / chunk) */
     uint32_t dtype;           /* lng_dtype of q, k, v, out */
+    uint32_t fused;           /* split-K: 1 = the last workgroup of a row merges, 0 = lng_decode_merge follows */
     float scale;
 } lng_k_attn;
+
+/* Most chunks one row may be split into: bounds the merge's LDS weight table. */
+#define LNG_MAX_CHUNKS 256
 
 /* Prompt pass: t query rows from `start`, one cache. */
 typedef struct lng_k_prefill {

@@ -189,7 +189,9 @@ extern "C" __global__ __launch_bounds__(256) void lng_attn_generic_bf16(lng_k_at
 // Online softmax state per lane: running max of its head (log2 domain), its share of the
 // running sum, and 16 accumulators O^T[16m + 4j + i][n]. Wavefronts merge through LDS; with
 // one chunk the workgroup writes the output (sink folded into the normaliser), otherwise it
-// writes (max, sum, O) partials that lng_decode_combine merges.
+// writes (max, sum, O) partials; these are merged by the workgroup that finishes last (small
+// grids, where a second dispatch would cost more than the chunks themselves) or by
+// lng_decode_merge as the next dispatch (large grids).
 // =============================================================================================
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 x) { return __builtin_bit_cast(bf16x8, x); }
 
@@ -204,6 +206,74 @@ __device__ __forceinline__ bf16x8 narrow8(floatx4 lo, floatx4 hi) {
     r[6] = (__bf16)hi[2];
     r[7] = (__bf16)hi[3];
     return r;
+}
+
+// Merges the split-K partials of one (row, kv head): 16 threads per head first turn the chunks'
+// (max, sum) pairs into weights in LDS and the head's normaliser; then each thread owns outputs
+// (head, dim) and streams the chunks' partial rows with independent loads. The sink joins here,
+// once: exp(sink - max) in the normaliser and no value. COHERENT: the partials were written by
+// other workgroups of the same dispatch and are read with device-coherent loads.
+template <bool COHERENT> __device__ __forceinline__ float load_partial(const float *p) {
+    if (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+
+template <bool COHERENT>
+__device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_row &it, uint32_t g, uint32_t group,
+                                             uint32_t row_chunks) {
+    __shared__ float s_w[16][LNG_MAX_CHUNKS];
+    __shared__ float s_z[16];
+    {
+        const uint32_t h = threadIdx.x >> 4, t16 = threadIdx.x & 15u;
+        if (h < group) {
+            const uint32_t head = g * group + h;
+            const uint64_t slot0 = ((uint64_t)blockIdx.y * a.n_chunks) * group + h;
+            const float sink2 = it.sinks_offset != LNG_NO_SINKS
+                                    ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                    : LNG_NEG_INF;
+            float top = sink2;
+            for (uint32_t c = t16; c < row_chunks; c += 16u) {
+                const float mc = load_partial<COHERENT>(&a.partial_ml[(slot0 + (uint64_t)c * group) * 2u]);
+                s_w[h][c] = mc;
+                top = fmaxf(top, mc);
+            }
+#pragma unroll
+            for (int s = 8; s >= 1; s >>= 1) top = fmaxf(top, __shfl_xor(top, s, 64));
+            float z = 0.0f;
+            for (uint32_t c = t16; c < row_chunks; c += 16u) {
+                const float lc = load_partial<COHERENT>(&a.partial_ml[(slot0 + (uint64_t)c * group) * 2u + 1u]);
+                const float mc = s_w[h][c];
+                const float wt = mc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(mc - top);
+                s_w[h][c] = wt;
+                z += lc * wt;
+            }
+#pragma unroll
+            for (int s = 8; s >= 1; s >>= 1) z += __shfl_xor(z, s, 64);
+            if (t16 == 0) s_z[h] = z + (sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top));
+        }
+    }
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
+        const uint32_t h = idx >> 6;
+        const uint32_t d = idx & 63u;
+        const float *po = a.partial_o + (((uint64_t)blockIdx.y * a.n_chunks) * group + h) * 64u + d;
+        const uint64_t step = (uint64_t)group * 64u;
+        float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+        uint32_t c = 0;
+        for (; c + 4 <= row_chunks; c += 4) {
+            const float x0 = load_partial<COHERENT>(po + (c + 0) * step);
+            const float x1 = load_partial<COHERENT>(po + (c + 1) * step);
+            const float x2 = load_partial<COHERENT>(po + (c + 2) * step);
+            const float x3 = load_partial<COHERENT>(po + (c + 3) * step);
+            o0 += x0 * s_w[h][c];
+            o1 += x1 * s_w[h][c + 1];
+            o2 += x2 * s_w[h][c + 2];
+            o3 += x3 * s_w[h][c + 3];
+        }
+        for (; c < row_chunks; ++c) o0 += load_partial<COHERENT>(po + c * step) * s_w[h][c];
+        uint16_t *op = (uint16_t *)(a.out + it.out_offset) + ((uint64_t)g * group + h) * 64u + d;
+        *op = f32_to_bf16_bits(((o0 + o1) + (o2 + o3)) / s_z[h]);
+    }
 }
 
 struct kv_tile {
@@ -363,8 +433,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
             sum += s_l[w][h] * wt;
             o += s_o[w][h][d] * wt;
         }
-        const uint32_t head = g * group + h;
         if (row_chunks == 1) {
+            const uint32_t head = g * group + h;
             const float sink2 = it.sinks_offset != LNG_NO_SINKS
                                     ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
                                     : LNG_NEG_INF;
@@ -375,49 +445,51 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
             *op = f32_to_bf16_bits(o * keep / z);
         } else {
             const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
-            a.partial_o[slot * 64u + d] = o;
-            if (d == 0) {
-                a.partial_ml[slot * 2u] = top;
-                a.partial_ml[slot * 2u + 1u] = sum;
+            if (a.fused) {
+                // device-coherent stores: visible to every XCD once acknowledged, no cache write-back
+                __hip_atomic_store(&a.partial_o[slot * 64u + d], o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (d == 0) {
+                    __hip_atomic_store(&a.partial_ml[slot * 2u], top, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(&a.partial_ml[slot * 2u + 1u], sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            } else { // lng_decode_merge runs as the next dispatch and sees ordinary stores
+                a.partial_o[slot * 64u + d] = o;
+                if (d == 0) {
+                    a.partial_ml[slot * 2u] = top;
+                    a.partial_ml[slot * 2u + 1u] = sum;
+                }
             }
         }
     }
+    if (row_chunks == 1 || !a.fused) return;
+
+    // ---- split-K: the workgroup that finishes last for this (row, kv head) merges the partials ----
+    // Every thread waits for its own coherent stores to be acknowledged, the workgroup meets, and
+    // one thread takes a ticket; whoever draws the last ticket reads the partials back with
+    // coherent loads. No cache-wide write-back or invalidate is involved. The ticket counter
+    // returns to zero for the next dispatch (dispatches run in stream order).
+    __shared__ uint32_t s_ticket;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) s_ticket = atomicAdd(&a.tickets[blockIdx.y], 1u);
+    __syncthreads();
+    if (s_ticket != row_chunks - 1u) return;
+    if (threadIdx.x == 0) __hip_atomic_store(&a.tickets[blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+    merge_chunks<true>(a, it, g, group, row_chunks);
 }
 
-// Merges the split-K partials of lng_decode_bf16_d64: one wavefront per (row, head), lane =
-// dimension. The sink joins here, once: it adds exp(sink - max) to the normaliser and no value.
-extern "C" __global__ __launch_bounds__(64) void lng_decode_combine(lng_k_attn a) {
-    const uint32_t row = blockIdx.x / a.heads;
-    const uint32_t head = blockIdx.x % a.heads;
+// The same merge as its own dispatch, for large grids: there a workgroup that waits for its
+// coherent stores and its ticket holds a compute unit's slot that another chunk could use.
+extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a) {
+    const uint32_t row = blockIdx.y / a.kv_heads;
+    const uint32_t g = blockIdx.y % a.kv_heads;
     const lng_k_row it = row_of(a, row);
     const uint64_t last = it.start;
-    const uint64_t first = first_visible(last, it.window);
-    const uint64_t base = first & ~(uint64_t)31;
+    const uint64_t base = first_visible(last, it.window) & ~(uint64_t)31;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
     if (row_chunks == 1) return; // the decode kernel already wrote this row
-    const uint32_t group = a.heads / a.kv_heads;
-    const uint32_t g = head / group;
-    const uint32_t h = head % group;
-    const uint32_t d = threadIdx.x;
-    const uint64_t slot0 = ((uint64_t)(row * a.kv_heads + g) * a.n_chunks) * group + h;
-    const float sink2 = it.sinks_offset != LNG_NO_SINKS
-                            ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
-                            : LNG_NEG_INF;
-    float top = sink2;
-    for (uint32_t c = 0; c < row_chunks; ++c) {
-        top = fmaxf(top, a.partial_ml[(slot0 + (uint64_t)c * group) * 2u]);
-    }
-    float z = sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top);
-    float o = 0.0f;
-    for (uint32_t c = 0; c < row_chunks; ++c) {
-        const uint64_t slot = slot0 + (uint64_t)c * group;
-        const float mc = a.partial_ml[slot * 2u];
-        const float wt = mc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(mc - top);
-        z += a.partial_ml[slot * 2u + 1u] * wt;
-        o += a.partial_o[slot * 64u + d] * wt;
-    }
-    uint16_t *op = (uint16_t *)(a.out + it.out_offset) + (uint64_t)head * 64u + d;
-    *op = f32_to_bf16_bits(o / z);
+    merge_chunks<false>(a, it, g, a.heads / a.kv_heads, row_chunks);
 }
 
 // =============================================================================================
