@@ -35,6 +35,9 @@ ROW = G * D * 2          # bytes of one cached position of K (or V) in bf16
 QO = H * D * 2           # bytes of one query (or output) row
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+# HBM bytes per launch of the decode kernel on the default stack workload, from rocprofv3 FETCH_SIZE
+# and WRITE_SIZE scaled by a 1 GiB copy (profiles/decode_stack_c5_hbm_traffic.md).
+STACK_TRAFFIC_PER_LAUNCH = 2155619789
 METRIC = "decode attn GB/s (% HBM peak) + prefill attn TFLOP/s (% MFMA), gpt-oss shapes"
 
 
@@ -246,6 +249,31 @@ def run_prefill(gpu, steps, warmup, t=8192):
     return res
 
 
+def run_copy(gpu, steps, warmup, nbytes=1 << 30):
+    """A plain copy of known size through lng_copy_rows: the yardstick that the FETCH_SIZE and
+    WRITE_SIZE counters of a profile are scaled by (it reads nbytes and writes nbytes)."""
+    src, dst = gpu.buffer(nbytes), gpu.buffer(nbytes)
+    fill(gpu, src, 99)
+    width = 1 << 16
+    rows = nbytes // 4 // width
+
+    def go():
+        batch = gpu.batch([src, dst])
+        batch.copy_rows((C.Slice(0, 0, nbytes), width), (C.Slice(1, 0, nbytes), width), rows, width, C.F32, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(warmup):
+        go()
+    runs = sorted(go() for _ in range(max(steps, 3)))
+    src.free()
+    dst.free()
+    g = runs[len(runs) // 2]
+    return {"workload": "copy of %d bytes (lng_copy_rows, f32)" % nbytes, "read_bytes": nbytes, "write_bytes": nbytes,
+            "gpu_ms": g * 1e3, "gbs": 2 * nbytes / g / 1e9}
+
+
 def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
     """The oracle (port of the reference's CPU attention, f32 on widened bf16 inputs) on a
     bounded sample of the headline workload: one sequence, one full-causal and one 128-window
@@ -280,7 +308,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,copy: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -291,7 +319,7 @@ def main():
     log("device:", gpu.name())
     extra = {}
     if args.only:
-        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill}
+        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -315,7 +343,8 @@ def main():
         "config": {"workload": r["workload"], "heads": H, "kv_heads": G, "head_dim": D,
                    "hbm_frac_of_value": r["value_gbs"] / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": r["kernel"], "achieved": r["kernel_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": r["kernel_gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "unit": "GB/s", "frac": r["kernel_gbs"] / HBM_PEAK_GBS,
+                     "traffic": STACK_TRAFFIC_PER_LAUNCH if (args.ctx, args.batch) == (131072, 16) else None,
                      "bytes_per_launch": r["kernel_bytes_per_launch"], "s_per_launch": r["kernel_s_per_launch"]},
         "cpu_baseline": cpu,
         "extra": extra,

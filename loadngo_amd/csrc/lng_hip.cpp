@@ -69,10 +69,6 @@ struct Cmd {
     unsigned grid[3] = {1, 1, 1};
     unsigned block = 256;
     std::vector<char> args;
-    // optional host->device copy enqueued before the launch (row tables)
-    const void *copy_src = nullptr;
-    void *copy_dst = nullptr;
-    size_t copy_len = 0;
 };
 
 } // namespace
@@ -417,11 +413,6 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         c.grid[0] = (unsigned)(n_rows * a.heads);
         c.block = 256;
         set_args(c, a);
-        if (a.rows) { // table upload rides on the first command
-            c.copy_src = host_rows;
-            c.copy_dst = (void *)a.rows;
-            c.copy_len = n_rows * sizeof(lng_k_row);
-        }
         b->cmds.push_back(std::move(c));
         return LNG_OK;
     }
@@ -444,11 +435,6 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     c.grid[1] = (unsigned)(n_rows * a.kv_heads);
     c.block = 256;
     set_args(c, a);
-    if (a.rows) {
-        c.copy_src = host_rows;
-        c.copy_dst = (void *)a.rows;
-        c.copy_len = n_rows * sizeof(lng_k_row);
-    }
     b->cmds.push_back(std::move(c));
     if (plan.n_chunks > 1 && !a.fused) {
         Cmd m;
@@ -773,12 +759,13 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
     hipError_t e = hipEventCreate(&b->ev0);
     if (e == hipSuccess) e = hipEventCreate(&b->ev1);
     if (e == hipSuccess) e = hipEventRecord(b->ev0, g->stream);
+    // the row tables of every batched dispatch, one copy per table block, ahead of the kernels
+    for (size_t i = 0; e == hipSuccess && i < b->tables.size(); ++i) {
+        const Table &t = b->tables[i];
+        if (t.used) e = hipMemcpyAsync(t.dev, t.host, t.used, hipMemcpyHostToDevice, g->stream);
+    }
     for (size_t i = 0; e == hipSuccess && i < b->cmds.size(); ++i) {
         Cmd &c = b->cmds[i];
-        if (c.copy_len) {
-            e = hipMemcpyAsync(c.copy_dst, c.copy_src, c.copy_len, hipMemcpyHostToDevice, g->stream);
-            if (e != hipSuccess) break;
-        }
         size_t size = c.args.size();
         void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, c.args.data(), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                           HIP_LAUNCH_PARAM_END};
