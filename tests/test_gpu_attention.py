@@ -328,3 +328,50 @@ def test_config4_prefill_8192_sampled_rows(gpu, window):
     want = oracle.attention_rows_f32(from_bf16_bits(qb[rows]), from_bf16_bits(kb), from_bf16_bits(vb), sinks, rows,
                                      window=window, scale=0.125, threads=THREADS)
     assert max_error(from_bf16_bits(got[rows]), want) < BF16_TOL
+
+
+# ---- configuration 5 at its real per-layer size, through a size-independent identity -----------
+def test_config5_layer_at_full_size_periodic_identity(gpu):
+    """One layer of the long-context stack at its real shape (batch 16, context 131072, 2 GiB of K
+    and of V). The cache is filled on the device with a stream that repeats every 1024 positions,
+    so every weight of the full-causal layer appears 128 times: the exact result is attention over
+    one period with the sink lowered by ln(128) (pinned on the oracle in test_oracle_pinning). The
+    128-window layer sees the last 128 positions of a period. Every sequence and head is checked."""
+    from loadngo_amd.synthetic import synthetic_values
+    batch_size, ctx, heads, kv_heads, dim, period = 16, 131072, 64, 8, 64, 1024
+    row = kv_heads * dim
+    kbuf, vbuf = gpu.buffer(batch_size * ctx * row * 2), gpu.buffer(batch_size * ctx * row * 2)
+    rng = np.random.default_rng(55)
+    q = to_bf16_bits((rng.standard_normal((2 * batch_size, heads, dim), dtype=np.float32) * 0.5))
+    sinks = rng.standard_normal((2, heads)).astype(np.float32)
+    qbuf, obuf, sbuf = gpu.upload(q), gpu.buffer(q.nbytes), gpu.upload(sinks)
+    obuf.fill(0xFF)
+    bufs = [qbuf, kbuf, vbuf, obuf, sbuf]
+    batch = gpu.batch(bufs)
+    batch.fill_synthetic(C.Slice(1, 0, kbuf.len), C.BF16, 7, 0.5, period * row)
+    batch.fill_synthetic(C.Slice(2, 0, vbuf.len), C.BF16, 8, 0.5, period * row)
+    step = heads * dim * 2
+    items = []
+    for layer, window in enumerate((FULL, 128)):
+        for b in range(batch_size):
+            i = layer * batch_size + b
+            items.append(C.DecodeItem(i * step, i * step, b * ctx * row * 2, b * ctx * row * 2, layer * heads * 4,
+                                      ctx - 1, window, ctx))
+    batch.attention_decode_batched(0, 1, 2, 3, 4, items[:batch_size], heads, kv_heads, dim, 0.125, C.BF16)
+    batch.attention_decode_batched(0, 1, 2, 3, 4, items[batch_size:], heads, kv_heads, dim, 0.125, C.BF16)
+    done = batch.run()
+    assert not isinstance(done.gpu_time, Exception)
+    got = from_bf16_bits(obuf.read(np.uint16).reshape(q.shape))
+    batch.drop()
+    for b in bufs:
+        b.free()
+    k1 = to_bf16_bits(synthetic_values(period * row, 7, 0.5).reshape(period, kv_heads, dim))
+    v1 = to_bf16_bits(synthetic_values(period * row, 8, 0.5).reshape(period, kv_heads, dim))
+    repeats = ctx // period
+    lowered = sinks[0] - np.float32(np.log(repeats))
+    for b in range(batch_size):
+        full = oracle.attention_bf16(q[b:b + 1], k1, v1, lowered, period - 1, scale=0.125, threads=THREADS)
+        assert max_error(got[b], from_bf16_bits(full[0])) < BF16_TOL, ("full", b)
+        win = oracle.attention_bf16(q[batch_size + b:batch_size + b + 1], k1, v1, sinks[1], period - 1, window=128,
+                                    scale=0.125, threads=THREADS)
+        assert max_error(got[batch_size + b], from_bf16_bits(win[0])) < BF16_TOL, ("window", b)
