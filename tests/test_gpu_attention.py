@@ -375,3 +375,22 @@ def test_config5_layer_at_full_size_periodic_identity(gpu):
         win = oracle.attention_bf16(q[batch_size + b:batch_size + b + 1], k1, v1, sinks[1], period - 1, window=128,
                                     scale=0.125, threads=THREADS)
         assert max_error(got[batch_size + b], from_bf16_bits(win[0])) < BF16_TOL, ("window", b)
+
+
+@pytest.mark.parametrize("start,window,slots", [(131148, FULL, 131149), (200000, 100000, 150016), (70000, FULL, 70001)])
+def test_decode_bf16_one_long_row(gpu, start, window, slots):
+    """A single query over a very long cache: the run is cut into the largest allowed number of
+    chunks (the chunk length grows to respect it) and merged by a second dispatch; with a ring that
+    has wrapped and a window that does not start on a tile boundary."""
+    heads, kv_heads, dim = 64, 8, 64
+    rows = min(slots, start + 1)
+    rng = np.random.default_rng(start)
+    q = to_bf16_bits(rng.standard_normal((1, heads, dim), dtype=np.float32) * 0.5)
+    kr = to_bf16_bits(rng.standard_normal((rows, kv_heads, dim), dtype=np.float32) * 0.5)
+    vr = to_bf16_bits(rng.standard_normal((rows, kv_heads, dim), dtype=np.float32) * 0.5)
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    shape = C.GroupedShape(1, start, heads, kv_heads, dim, window, slots, 0.125)
+    got = run_attention(gpu, q, kr, vr, sinks, shape, False, C.BF16)
+    # the oracle reads position p from row p % slots of the same ring
+    want = oracle.attention_bf16(q, kr, vr, sinks, start, window=window, slots=slots, scale=0.125, threads=THREADS)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
