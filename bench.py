@@ -7,9 +7,11 @@ A step is one pass of the hot path over one batch of synthetic input resident in
 headline workload is the long-context decode stack (24 layers alternating 128-token window
 and full-causal, batch 16, context 131072, bf16 KV cache of 96 GiB): one step decodes one
 token for every sequence through all 24 layers' attention. `value` is the KV-cache GB/s of
-the whole step (algorithmic bytes / wall time per step); `roofline` is the decode kernel's
-own bandwidth (algorithmic bytes per launch / its average launch time from HIP events on the
-library's stream). The other configurations (single 4096-token decode, ragged batch of 32,
+the whole step (algorithmic bytes / wall time per step, K steps with nothing recorded between
+the kernels); `roofline` is the decode kernel's own bandwidth (algorithmic bytes per launch /
+its average launch time, from HIP events recorded after every kernel on the library's stream
+during K further steps: those events cost a few microseconds of gap each, so the throughput is
+not taken from the instrumented steps). The other configurations (single 4096-token decode, ragged batch of 32,
 8192-token prompt passes) are reported under "extra". The CPU baseline is the oracle (a C
 restatement of the reference's CPU attention) timed on this host on a bounded sample.
 
@@ -96,15 +98,21 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
 
     for _ in range(warmup):
         step(False)
+    # timed region: K steps, nothing recorded between the kernels
     t0 = time.perf_counter()
-    gpu_s = kern_s = 0.0
+    gpu_s = 0.0
+    for _ in range(steps):
+        g, _ = step(False)
+        gpu_s += g
+    wall = time.perf_counter() - t0
+    # the same K steps again with an event after every kernel (each event costs a ~5 us gap, which
+    # is why the throughput above is not taken from these): per-launch time of the decode kernel
+    kern_s = 0.0
     launches = 0
     for _ in range(steps):
-        g, (ks, kn) = step(True)
-        gpu_s += g
+        _, (ks, kn) = step(True)
         kern_s += ks
         launches += kn
-    wall = time.perf_counter() - t0
     for b in bufs:
         b.free()
     per_launch_bytes = step_bytes * steps / launches
