@@ -86,7 +86,7 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr;
+                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -491,11 +491,16 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         p.heads = (uint32_t)s.heads;
         p.kv_heads = (uint32_t)s.kv_heads;
         p.dim = (uint32_t)s.dim;
-        p.q_tiles = (uint32_t)((s.t + 63) / 64); // PF_BM query rows per workgroup
+        // Two heads per wavefront (64 query rows per workgroup) for long causal runs; one head
+        // per wavefront (32 rows, two workgroups per compute unit) when each query sees few keys
+        // and the pass is bound by latency, not by the matrix pipe.
+        const bool narrow = p.window != LNG_WINDOW_FULL && p.window <= 1024;
+        const unsigned rows_per_wg = narrow ? 32 : 64;
+        p.q_tiles = (uint32_t)((s.t + rows_per_wg - 1) / rows_per_wg);
         p.scale = s.scale;
         Cmd c;
-        c.fn = g->prefill_bf16_d64;
-        c.name = "lng_prefill_bf16_d64";
+        c.fn = narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
+        c.name = narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
         c.grid[0] = p.q_tiles * (unsigned)s.kv_heads; // kv head fastest: one XCD's L2 per kv head
         c.block = 512;
         set_args(c, p);
@@ -573,6 +578,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
         {"lng_decode_merge", &g->decode_merge, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
+        {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
     };

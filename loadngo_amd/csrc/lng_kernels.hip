@@ -557,7 +557,8 @@ extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill 
 // initialises the running maximum and contributes 1 to the running sum (it is one more logit
 // with no value); tiles wholly outside the causal/window band are never visited.
 // =============================================================================================
-#define PF_BM 64
+// PF_BM query rows per workgroup = 32 * (8 wavefronts / (8 / NH) head slots): 64 with two heads per
+// wavefront, 32 with one.
 #define PF_BN 64
 #define PF_THREADS 512
 #define PF_KSTRIDE 72 // bf16 elements per LDS row (144 bytes): conflict-free 16-byte row reads
@@ -583,7 +584,12 @@ __device__ __forceinline__ bf16x8 lds_read_tr8(const uint16_t *p0, const uint16_
     return __builtin_bit_cast(bf16x8, both);
 }
 
-extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(lng_k_prefill a) {
+// NH = heads per wavefront. NH = 2: 64 query rows per workgroup, wavefront = (32-row block, head pair);
+// every K/V operand read from LDS feeds two products, which is what a long causal pass needs.
+// NH = 1: 32 query rows per workgroup, wavefront = head; half the registers, so two workgroups share a
+// compute unit (4 wavefronts per SIMD) and short, latency-bound passes (a 128-token window) overlap.
+template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefill &a) {
+    constexpr uint32_t PF_BM = NH == 2 ? 64u : 32u;
     __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
 
@@ -595,8 +601,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6); // scalar: branches on it are uniform
     const uint32_t n = lane & 31u;  // query within the wave's block
     const uint32_t hh = lane >> 5;  // which half of the k-slots / of each 8 accumulator rows
-    const uint32_t qb = wave & 1u;
-    const uint32_t hp = wave >> 1;
+    const uint32_t qb = NH == 2 ? (wave & 1u) : 0u;
+    const uint32_t hp = NH == 2 ? (wave >> 1) : wave; // first head slot of the wavefront is hp * NH
 
     // Positions fit 32 bits (the host refuses shapes whose counts do not).
     const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
@@ -620,16 +626,16 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     const uint32_t my_row = q0 + 32u * qb + n;      // query row of this lane
     const uint32_t my_pos = start + my_row;         // its absolute position
     const bool row_ok = my_row < t;
-    const bool wave_active = hp * 2u < group;
-    const bool second_ok = hp * 2u + 1u < group;
-    uint32_t head[2];
-    head[0] = g * group + (wave_active ? hp * 2u : 0u);
-    head[1] = second_ok ? head[0] + 1u : head[0];
-    bf16x8 qreg[2][4];
-    float m[2], l[2];
-    floatx16 ot[2][2];
+    const bool wave_active = hp * NH < group;
+    const bool second_ok = NH == 2 && hp * 2u + 1u < group;
+    uint32_t head[NH];
+    head[0] = g * group + (wave_active ? hp * NH : 0u);
+    if constexpr (NH == 2) head[1] = second_ok ? head[0] + 1u : head[0];
+    bf16x8 qreg[NH][4];
+    float m[NH], l[NH];
+    floatx16 ot[NH][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < NH; ++h) {
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             uint4 raw = make_uint4(0, 0, 0, 0);
@@ -696,16 +702,16 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
                 for (int ks = 0; ks < 4; ++ks) {
                     ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
                 }
-                floatx16 st[2];
+                floatx16 st[NH];
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
+                for (int h = 0; h < NH; ++h) {
 #pragma unroll
                     for (int i = 0; i < 16; ++i) st[h][i] = 0.0f;
                 }
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[0][ks], st[0], 0, 0, 0);
-                    st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[1][ks], st[1], 0, 0, 0);
+                    if constexpr (NH == 2) st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[1][ks], st[1], 0, 0, 0);
                 }
                 // V^T operands of this block: two groups of 16 keys x two halves of the head width;
                 // issued now, their LDS latency hides behind the softmax arithmetic
@@ -723,9 +729,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
                 // domain): weights then stay below 2^PF_TAU, and the accumulators are rescaled only
                 // on the rare blocks where some lane's maximum moved. The normaliser uses the same
                 // maximum, so the result is the same softmax.
-                bf16x8 pb[2][2];
+                bf16x8 pb[NH][2];
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
+                for (int h = 0; h < NH; ++h) {
                     if constexpr (MASK) {
 #pragma unroll
                         for (int i = 0; i < 16; ++i) {
@@ -774,7 +780,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
 #pragma unroll
                     for (int db = 0; db < 2; ++db) {
                         ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[0][jj], ot[0][db], 0, 0, 0);
-                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
+                        if constexpr (NH == 2) ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
                     }
                 }
             }
@@ -796,7 +802,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
     // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------
     if (wave_active && row_ok) {
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < NH; ++h) {
             if (h == 1 && !second_ok) continue;
             const float total = l[h] + __shfl_xor(l[h], 32, 64);
             const float inv = total > 0.0f ? 1.0f / total : 0.0f;
@@ -815,4 +821,12 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
             }
         }
     }
+}
+
+extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(lng_k_prefill a) {
+    prefill_body<2>(a);
+}
+
+extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1(lng_k_prefill a) {
+    prefill_body<1>(a);
 }
