@@ -194,6 +194,59 @@ int lng_hip_attention_decode_batched(lng_batch *batch, uint64_t q_buffer, uint64
                                      const lng_decode_item *items, size_t n_items, uint64_t heads,
                                      uint64_t kv_heads, uint64_t dim, float scale, int dtype);
 
+/* ---- The step before attention (gpt-oss/src/gpu.rs:733-759) -------------------------------- */
+
+/* apple.rs:1886-1911 Batch::add_rows(dst, (src, src_stride), rows, width), f32:
+ * dst[r][i] += src[r * src_stride + i]; src_stride == 0 adds one row (a bias) to every row.
+ * Refused like the reference: rows == 0, width == 0, 0 < src_stride < width. */
+int lng_hip_add_rows(lng_batch *batch, lng_slice dst, lng_slice src, uint64_t src_stride,
+                     uint64_t rows, uint64_t width);
+
+/* apple.rs:1916-1955 Batch::rotate_halves / rotate_halves_partial(x, table, rows, (heads, dim,
+ * rotary)), f32, in place: x is [rows][heads][dim]; table holds per row rotary / 2 pairs
+ * (cos, sin); element i of the first half of a head's first `rotary` dimensions turns with
+ * element i of their second half: (a, b) -> (a cos - b sin, b cos + a sin), every product
+ * rounded on its own. Refused: rows, heads or rotary == 0, rotary > dim, rotary odd. */
+int lng_hip_rotate_halves(lng_batch *batch, lng_slice x, lng_slice table, uint64_t rows,
+                          uint64_t heads, uint64_t dim, uint64_t rotary);
+
+/* The whole step in one dispatch. No counterpart in the reference, which records three
+ * add_rows, two rotate_halves and two to four copy_rows per layer (gpu.rs:733-759); this
+ * computes exactly what those compute, in the same f32 operations, and narrows the results
+ * to `out_dtype` as it stores them.
+ *
+ * An item is one sequence: its `n` new positions start, start + 1, ... Its projections q
+ * [n][heads*dim], k and v [n][kv_heads*dim] are f32; the prepared queries go to q_out
+ * [n][heads*dim]; the prepared k and v rows of position p go to row p % slots of caches
+ * [slots][kv_heads*dim]. One item with n rows is a prompt pass; many items with n = 1 are one
+ * decoding step of many sequences. Offsets are bytes into the buffers named by
+ * lng_prepare_buffers. Refused: n == 0, n > slots (two new rows would land on one cache row),
+ * outputs that overlap an input or one another, outputs in resident memory. */
+typedef struct lng_prepare_item {
+    uint64_t q_offset, k_offset, v_offset; /* f32 projections of the item's n rows */
+    uint64_t table_offset;                 /* [n][rotary/2] (cos, sin) f32 pairs */
+    uint64_t q_out_offset;                 /* [n][heads*dim] of out_dtype */
+    uint64_t k_cache_offset;               /* row 0 of [slots][kv_heads*dim] of out_dtype */
+    uint64_t v_cache_offset;
+    uint64_t n;
+    uint64_t start;
+    uint64_t slots;
+} lng_prepare_item;
+
+typedef struct lng_prepare_buffers {
+    uint64_t q, k, v;          /* indices (as in lng_slice.buffer) of the projection buffers */
+    uint64_t table;
+    uint64_t q_out;
+    uint64_t k_cache, v_cache;
+    const lng_slice *q_bias;   /* [heads*dim] f32, or NULL */
+    const lng_slice *k_bias;   /* [kv_heads*dim] f32, or NULL */
+    const lng_slice *v_bias;
+} lng_prepare_buffers;
+
+int lng_hip_prepare_attention(lng_batch *batch, const lng_prepare_buffers *buffers,
+                              const lng_prepare_item *items, size_t n_items, uint64_t heads,
+                              uint64_t kv_heads, uint64_t dim, uint64_t rotary, int out_dtype);
+
 /* Deterministic synthetic data written on the device (benchmarks and full-size tests):
  * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
  * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The

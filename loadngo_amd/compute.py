@@ -66,6 +66,19 @@ class _Item(ctypes.Structure):
                 ("q_offset", "out_offset", "k_offset", "v_offset", "sinks_offset", "start", "window", "slots")]
 
 
+_PREPARE_FIELDS = ("q_offset", "k_offset", "v_offset", "table_offset", "q_out_offset", "k_cache_offset",
+                   "v_cache_offset", "n", "start", "slots")
+
+
+class _PrepareItem(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in _PREPARE_FIELDS]
+
+
+class _PrepareBuffers(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_uint64) for n in ("q", "k", "v", "table", "q_out", "k_cache", "v_cache")] + \
+               [(n, ctypes.POINTER(_Slice)) for n in ("q_bias", "k_bias", "v_bias")]
+
+
 class _Completed(ctypes.Structure):
     _fields_ = [("status", ctypes.c_int), ("gpu_seconds", ctypes.c_double), ("message", ctypes.c_char_p)]
 
@@ -108,6 +121,10 @@ SYMBOLS = {
                                                         ctypes.c_size_t, _U64, _U64, _U64, ctypes.c_float,
                                                         ctypes.c_int]),
     "lng_hip_fill_synthetic": (ctypes.c_int, [_P, _Slice, ctypes.c_int, _U64, ctypes.c_float, _U64]),
+    "lng_hip_add_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64]),
+    "lng_hip_rotate_halves": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, _U64]),
+    "lng_hip_prepare_attention": (ctypes.c_int, [_P, ctypes.POINTER(_PrepareBuffers), ctypes.POINTER(_PrepareItem),
+                                                 ctypes.c_size_t, _U64, _U64, _U64, _U64, ctypes.c_int]),
 }
 
 _lib = None
@@ -192,6 +209,32 @@ def decode_items(items):
     return (_Item * len(items))(*[
         _Item(i.q_offset, i.out_offset, i.k_offset, i.v_offset, i.sinks_offset, i.start, i.window, i.slots)
         for i in items])
+
+
+class PrepareItem:
+    """One sequence of ``Batch.prepare_attention``: byte offsets of its ``n`` projection rows, of its
+    rotary table rows, of its prepared queries and of row 0 of its caches; its first new position
+    and the rows its caches hold."""
+
+    __slots__ = _PREPARE_FIELDS
+
+    def __init__(self, **fields):
+        for name in _PREPARE_FIELDS:
+            setattr(self, name, fields.pop(name, 0))
+        if fields:
+            raise TypeError("unknown fields: %s" % sorted(fields))
+
+
+def prepare_items(items):
+    """A prepared table of ``PrepareItem`` (built once, reused while the offsets hold)."""
+    return (_PrepareItem * len(items))(*[_PrepareItem(*[getattr(i, n) for n in _PREPARE_FIELDS]) for i in items])
+
+
+def rope_table(inv_freq, scale, start, n):
+    """``[n][len(inv_freq)][2]`` f32 pairs ``(cos, sin) * scale`` of ``position * inv_freq`` for positions
+    ``start..start+n``, computed in f64 as the reference's host does every pass (gpt-oss/src/gpu.rs:690-697)."""
+    angle = (start + np.arange(n, dtype=np.float64))[:, None] * np.asarray(inv_freq, dtype=np.float64)[None, :]
+    return np.stack([(np.cos(angle) * scale).astype(np.float32), (np.sin(angle) * scale).astype(np.float32)], axis=-1)
 
 
 class Completed:
@@ -356,6 +399,33 @@ class Batch:
         _check(library().lng_hip_attention_decode_batched(self._h, q_buffer, k_buffer, v_buffer, out_buffer,
                                                           sinks_buffer, arr, len(items), heads, kv_heads, dim,
                                                           scale, dtype))
+
+    def add_rows(self, dst, src, rows, width):
+        """``add_rows(dst, (src, src_stride), rows, width)`` (apple.rs:1886), f32."""
+        s, s_stride = src
+        _check(library().lng_hip_add_rows(self._h, dst._c(), s._c(), s_stride, rows, width))
+
+    def rotate_halves(self, x, table, rows, heads_dim):
+        """``rotate_halves(x, table, rows, (heads, dim))`` (apple.rs:1916), f32, in place."""
+        heads, dim = heads_dim
+        _check(library().lng_hip_rotate_halves(self._h, x._c(), table._c(), rows, heads, dim, dim))
+
+    def rotate_halves_partial(self, x, table, rows, heads_dim_rotary):
+        """``rotate_halves_partial(x, table, rows, (heads, dim, rotary))`` (apple.rs:1929)."""
+        heads, dim, rotary = heads_dim_rotary
+        _check(library().lng_hip_rotate_halves(self._h, x._c(), table._c(), rows, heads, dim, rotary))
+
+    def prepare_attention(self, buffers, items, heads, kv_heads, dim, rotary=None, out_dtype=BF16,
+                          q_bias=None, k_bias=None, v_bias=None):
+        """Biases, rotation, narrowing and cache append of gpt-oss/src/gpu.rs:733-759 in one dispatch.
+        ``buffers`` maps q, k, v, table, q_out, k_cache, v_cache to buffer numbers of this batch;
+        the biases are slices (or None)."""
+        held = [None if b is None else b._c() for b in (q_bias, k_bias, v_bias)]
+        pb = _PrepareBuffers(*[buffers[n] for n in ("q", "k", "v", "table", "q_out", "k_cache", "v_cache")],
+                             *[None if h is None else ctypes.pointer(h) for h in held])
+        arr = items if isinstance(items, ctypes.Array) else prepare_items(items)
+        _check(library().lng_hip_prepare_attention(self._h, ctypes.byref(pb), arr, len(arr), heads, kv_heads, dim,
+                                                   dim if rotary is None else rotary, out_dtype))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))

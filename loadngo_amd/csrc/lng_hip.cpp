@@ -86,7 +86,8 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr;
+                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
+                  add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -581,6 +582,10 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
+        {"lng_add_rows", &g->add_rows, true},
+        {"lng_rotate_halves", &g->rotate_halves, true},
+        {"lng_prepare_v4", &g->prepare_v4, true},
+        {"lng_prepare_v1", &g->prepare_v1, true},
     };
     for (auto &w : wanted) {
         e = hipModuleGetFunction(w.fn, g->module, w.name);
@@ -983,6 +988,207 @@ extern "C" int lng_hip_attention_decode_batched(lng_batch *b, uint64_t q_buffer,
     a.dtype = (uint32_t)dtype;
     a.scale = scale;
     if (int rc = record_rows(b, a, (const lng_k_row *)host, n_items, 0, aligned16)) return rc;
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_add_rows(lng_batch *b, lng_slice dst, lng_slice src, uint64_t src_stride, uint64_t rows,
+                                uint64_t width) {
+    if (int rc = need_recording(b)) return rc;
+    // apple.rs:1893-1897
+    if (rows == 0 || width == 0 || (src_stride != 0 && src_stride < width)) {
+        return fail(LNG_ERR_DISPATCH, "unsupported add: %llu x %llu, source stride %llu", (unsigned long long)rows,
+                    (unsigned long long)width, (unsigned long long)src_stride);
+    }
+    for (uint64_t n : {rows, width, src_stride}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (!fits_u32(rows * width)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)(rows * width));
+    Operand od, os;
+    if (int rc = check_slice(b, "dst", dst, rows * width * 4, 4, &od)) return rc;
+    if (int rc = check_slice(b, "src", src, ((rows - 1) * src_stride + width) * 4, 4, &os)) return rc;
+    if (int rc = check_output(b, od, {&os})) return rc;
+    lng_k_add a{};
+    a.dst = (float *)((char *)od.buf->ptr + dst.offset);
+    a.src = (const float *)((const char *)os.buf->ptr + src.offset);
+    a.rows = rows;
+    a.width = width;
+    a.src_stride = src_stride;
+    Cmd c;
+    c.fn = b->gpu->add_rows;
+    c.name = "lng_add_rows";
+    c.grid[0] = (unsigned)((rows * width + 255) / 256);
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_rotate_halves(lng_batch *b, lng_slice x, lng_slice table, uint64_t rows, uint64_t heads,
+                                     uint64_t dim, uint64_t rotary) {
+    if (int rc = need_recording(b)) return rc;
+    // apple.rs:1936-1940
+    if (rows == 0 || heads == 0 || rotary == 0 || rotary > dim || rotary % 2 != 0) {
+        return fail(LNG_ERR_DISPATCH, "unsupported rotation: %llu rows of %llu x %llu, %llu rotated",
+                    (unsigned long long)rows, (unsigned long long)heads, (unsigned long long)dim,
+                    (unsigned long long)rotary);
+    }
+    for (uint64_t n : {rows, heads, dim, rotary}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (!fits_u32(rows * heads) || !fits_u32(rows * heads * dim)) {
+        return fail(LNG_ERR_DISPATCH, "%llu rows of %llu x %llu do not fit in u32", (unsigned long long)rows,
+                    (unsigned long long)heads, (unsigned long long)dim);
+    }
+    Operand ox, ot;
+    if (int rc = check_slice(b, "x", x, rows * heads * dim * 4, 4, &ox)) return rc;
+    if (int rc = check_slice(b, "table", table, rows * rotary * 4, 8, &ot)) return rc;
+    if (int rc = check_output(b, ox, {&ot})) return rc;
+    lng_k_rotate a{};
+    a.x = (float *)((char *)ox.buf->ptr + x.offset);
+    a.table = (const float *)((const char *)ot.buf->ptr + table.offset);
+    a.rows = rows;
+    a.heads = (uint32_t)heads;
+    a.dim = (uint32_t)dim;
+    a.rotary = (uint32_t)rotary;
+    Cmd c;
+    c.fn = b->gpu->rotate_halves;
+    c.name = "lng_rotate_halves";
+    c.grid[0] = (unsigned)((rows * heads * (rotary / 2) + 255) / 256);
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+namespace {
+struct Span {
+    uint64_t buffer, lo, hi;
+    bool operator<(const Span &o) const { return buffer != o.buffer ? buffer < o.buffer : lo < o.lo; }
+};
+// True when two spans of one buffer share a byte (sorts `spans`).
+bool any_overlap(std::vector<Span> &spans) {
+    std::sort(spans.begin(), spans.end());
+    for (size_t i = 1; i < spans.size(); ++i) {
+        if (spans[i].buffer == spans[i - 1].buffer && spans[i].lo < spans[i - 1].hi) return true;
+    }
+    return false;
+}
+} // namespace
+
+extern "C" int lng_hip_prepare_attention(lng_batch *b, const lng_prepare_buffers *pb, const lng_prepare_item *items,
+                                         size_t n_items, uint64_t heads, uint64_t kv_heads, uint64_t dim,
+                                         uint64_t rotary, int out_dtype) {
+    if (int rc = need_recording(b)) return rc;
+    if (out_dtype != LNG_F32 && out_dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", out_dtype);
+    if (!pb || !items || n_items == 0) return fail(LNG_ERR_DISPATCH, "no items");
+    if (n_items > 65535) return fail(LNG_ERR_DISPATCH, "%zu items are more than one dispatch takes (65535)", n_items);
+    if (heads == 0 || kv_heads == 0 || dim == 0 || rotary == 0 || rotary > dim || rotary % 2 != 0) {
+        return fail(LNG_ERR_DISPATCH, "unsupported preparation: %llu + %llu heads of %llu, %llu rotated",
+                    (unsigned long long)heads, (unsigned long long)kv_heads, (unsigned long long)dim,
+                    (unsigned long long)rotary);
+    }
+    for (uint64_t n : {heads, kv_heads, dim, (uint64_t)n_items}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (!fits_u32((heads + 2 * kv_heads) * dim)) return fail(LNG_ERR_DISPATCH, "rows of %llu elements do not fit in u32", (unsigned long long)((heads + 2 * kv_heads) * dim));
+    const uint64_t es = elem_size(out_dtype), qw = heads * dim, kw = kv_heads * dim, half = rotary / 2;
+    for (uint64_t out : {pb->q_out, pb->k_cache, pb->v_cache}) {
+        if (!buffer_at(b, out)) return fail(LNG_ERR_DISPATCH, "no buffer %llu (batch has %zu)", (unsigned long long)out, b->buffers.size() + b->residents.size());
+        if (out >= b->buffers.size()) return fail(LNG_ERR_DISPATCH, "output is in read-only resident memory");
+    }
+    Operand oqb{}, okb{}, ovb{};
+    if (pb->q_bias) if (int rc = check_slice(b, "q_bias", *pb->q_bias, qw * 4, 4, &oqb)) return rc;
+    if (pb->k_bias) if (int rc = check_slice(b, "k_bias", *pb->k_bias, kw * 4, 4, &okb)) return rc;
+    if (pb->v_bias) if (int rc = check_slice(b, "v_bias", *pb->v_bias, kw * 4, 4, &ovb)) return rc;
+    std::vector<Span> outs, ins;
+    uint64_t most = 0;
+    uint64_t align = 0;
+    for (const Operand *o : {&oqb, &okb, &ovb}) {
+        if (o->buf) {
+            ins.push_back(Span{o->index, o->offset, o->offset + o->len});
+            align |= o->offset;
+        }
+    }
+    for (size_t i = 0; i < n_items; ++i) {
+        const lng_prepare_item &it = items[i];
+        if (it.n == 0 || it.slots == 0 || it.n > it.slots || it.start + it.n < it.start) {
+            return fail(LNG_ERR_DISPATCH, "item %zu: unsupported preparation of %llu rows from %llu into %llu slots", i,
+                        (unsigned long long)it.n, (unsigned long long)it.start, (unsigned long long)it.slots);
+        }
+        if (!fits_u32(it.n) || !fits_u32(it.slots)) return fail(LNG_ERR_DISPATCH, "item %zu: %llu does not fit in u32", i, (unsigned long long)std::max(it.n, it.slots));
+        struct { const char *what; uint64_t buffer, offset, len, align; bool out; } parts[] = {
+            {"q", pb->q, it.q_offset, it.n * qw * 4, 4, false},
+            {"k", pb->k, it.k_offset, it.n * kw * 4, 4, false},
+            {"v", pb->v, it.v_offset, it.n * kw * 4, 4, false},
+            {"table", pb->table, it.table_offset, it.n * rotary * 4, 8, false},
+            {"q_out", pb->q_out, it.q_out_offset, it.n * qw * es, es, true},
+            {"k_cache", pb->k_cache, it.k_cache_offset, it.slots * kw * es, es, true},
+            {"v_cache", pb->v_cache, it.v_cache_offset, it.slots * kw * es, es, true},
+        };
+        for (const auto &p : parts) {
+            Operand o;
+            const lng_slice sl{p.buffer, p.offset, p.len};
+            if (int rc = check_slice(b, p.what, sl, p.len, p.align, &o)) return fail(rc, "item %zu: %s", i, std::string(g_error).c_str());
+            (p.out ? outs : ins).push_back(Span{p.buffer, p.offset, p.offset + p.len});
+            align |= p.offset;
+        }
+        most = std::max(most, it.n);
+    }
+    // An output may share bytes neither with another output nor with an input.
+    if (any_overlap(outs)) return fail(LNG_ERR_DISPATCH, "outputs of the preparation overlap");
+    {
+        std::sort(ins.begin(), ins.end());
+        for (const Span &o : outs) {
+            // inputs are sorted by (buffer, lo) but may overlap one another: scan this buffer's run
+            auto at = std::lower_bound(ins.begin(), ins.end(), Span{o.buffer, 0, 0});
+            for (; at != ins.end() && at->buffer == o.buffer && at->lo < o.hi; ++at) {
+                if (at->hi > o.lo) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+            }
+        }
+    }
+    const bool vec4 = half % 4 == 0 && (dim - rotary) % 4 == 0 && (align & 15u) == 0;
+    const uint64_t w = vec4 ? 4 : 1;
+    const uint64_t units = (heads + kv_heads) * (half / w + (dim - rotary) / w) + kw / w;
+    if (!fits_u32(most * units + 256)) return fail(LNG_ERR_DISPATCH, "%llu rows do not fit in one dispatch", (unsigned long long)most);
+    lng_k_prepare a{};
+    a.q = (const char *)buffer_at(b, pb->q)->ptr;
+    a.k = (const char *)buffer_at(b, pb->k)->ptr;
+    a.v = (const char *)buffer_at(b, pb->v)->ptr;
+    a.q_bias = oqb.buf ? (const float *)((const char *)oqb.buf->ptr + oqb.offset) : nullptr;
+    a.k_bias = okb.buf ? (const float *)((const char *)okb.buf->ptr + okb.offset) : nullptr;
+    a.v_bias = ovb.buf ? (const float *)((const char *)ovb.buf->ptr + ovb.offset) : nullptr;
+    a.table = (const char *)buffer_at(b, pb->table)->ptr;
+    a.q_out = (char *)buffer_at(b, pb->q_out)->ptr;
+    a.k_cache = (char *)buffer_at(b, pb->k_cache)->ptr;
+    a.v_cache = (char *)buffer_at(b, pb->v_cache)->ptr;
+    if (n_items == 1) {
+        a.items = nullptr;
+        a.first = items[0];
+    } else {
+        char *host = nullptr, *dev = nullptr;
+        if (int rc = reserve_table(b, n_items * sizeof(lng_prepare_item), &host, &dev)) return rc;
+        memcpy(host, items, n_items * sizeof(lng_prepare_item));
+        a.items = (const lng_prepare_item *)dev;
+    }
+    a.n_items = (uint32_t)n_items;
+    a.heads = (uint32_t)heads;
+    a.kv_heads = (uint32_t)kv_heads;
+    a.dim = (uint32_t)dim;
+    a.rotary = (uint32_t)rotary;
+    a.out_dtype = (uint32_t)out_dtype;
+    a.units_per_row = (uint32_t)units;
+    a.vec = (uint32_t)w;
+    Cmd c;
+    c.fn = vec4 ? b->gpu->prepare_v4 : b->gpu->prepare_v1;
+    c.name = vec4 ? "lng_prepare_v4" : "lng_prepare_v1";
+    c.grid[0] = (unsigned)((most * units + 255) / 256);
+    c.grid[1] = (unsigned)n_items;
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
     b->dispatches += 1;
     return LNG_OK;
 }

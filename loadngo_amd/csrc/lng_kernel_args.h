@@ -78,6 +78,44 @@ typedef struct lng_k_fill {
     uint32_t dtype;
 } lng_k_fill;
 
+/* dst[r][i] += src[r * src_stride + i], f32. */
+typedef struct lng_k_add {
+    float *dst;
+    const float *src;
+    uint64_t rows;
+    uint64_t width;
+    uint64_t src_stride;
+} lng_k_add;
+
+/* In-place rotation by halves of x[rows][heads][dim], f32. */
+typedef struct lng_k_rotate {
+    float *x;
+    const float *table; /* [rows][rotary/2][2] */
+    uint64_t rows;
+    uint32_t heads;
+    uint32_t dim;
+    uint32_t rotary;
+    uint32_t pad;
+} lng_k_rotate;
+
+/* Bias + rotation + narrowing + cache append for a table of items (or the one item `first`). */
+typedef struct lng_k_prepare {
+    const char *q, *k, *v;   /* bases of the projection buffers */
+    const float *q_bias, *k_bias, *v_bias; /* NULL when absent */
+    const char *table;
+    char *q_out, *k_cache, *v_cache;
+    const lng_prepare_item *items; /* device table of n_items, or NULL: the one item is `first` */
+    lng_prepare_item first;
+    uint32_t n_items;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t dim;
+    uint32_t rotary;
+    uint32_t out_dtype;
+    uint32_t units_per_row;  /* work units of `vec` elements (pairs, for rotated parts) per row */
+    uint32_t vec;            /* 1 or 4 */
+} lng_k_prepare;
+
 /* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with
  * i' = period ? i % period : i; s = sum of the four 16-bit fields of z; value =
  * (float)(s - 131070) * factor, one f32 multiply, then narrowed if the dtype is bf16.

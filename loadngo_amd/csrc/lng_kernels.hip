@@ -516,6 +516,158 @@ extern "C" __global__ __launch_bounds__(256) void lng_copy_rows(lng_k_copy a) {
     }
 }
 
+// =============================================================================================
+// The step before attention (gpt-oss/src/gpu.rs:733-759): biases, rotation by halves, append.
+// The arithmetic is the CPU model's (model.rs:282-286, 389-404): one f32 add for the bias, then
+// four products, one difference and one sum, each rounded on its own, so fused multiply-add
+// is switched off in these functions.
+// =============================================================================================
+
+// Batch::add_rows (apple.rs:1886-1911; kernels.metal:1648-1660). One thread per element.
+extern "C" __global__ __launch_bounds__(256) void lng_add_rows(lng_k_add a) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (gid >= a.rows * a.width) return;
+    const uint64_t r = gid / a.width;
+    const uint64_t i = gid % a.width;
+    a.dst[gid] += a.src[r * a.src_stride + i];
+}
+
+// Batch::rotate_halves_partial (apple.rs:1929-1955; kernels.metal:1673-1690), in place.
+// One thread per rotated pair.
+extern "C" __global__ __launch_bounds__(256) void lng_rotate_halves(lng_k_rotate a) {
+#pragma clang fp contract(off)
+    const uint32_t half = a.rotary / 2;
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (gid >= a.rows * a.heads * half) return;
+    const uint32_t i = (uint32_t)(gid % half);
+    const uint64_t row_head = gid / half;
+    const uint64_t row = row_head / a.heads;
+    float *h = a.x + row_head * a.dim;
+    const float c = a.table[(row * half + i) * 2], s = a.table[(row * half + i) * 2 + 1];
+    const float x0 = h[i], x1 = h[i + half];
+    h[i] = x0 * c - x1 * s;
+    h[i + half] = x1 * c + x0 * s;
+}
+
+template <int W> struct prep_vec;
+template <> struct prep_vec<1> {
+    static __device__ void load(const float *p, float (&x)[1]) { x[0] = *p; }
+    static __device__ void store_f32(float *p, const float (&x)[1]) { *p = x[0]; }
+    static __device__ void store_bf16(uint16_t *p, const float (&x)[1]) { *p = f32_to_bf16_bits(x[0]); }
+};
+template <> struct prep_vec<4> {
+    static __device__ void load(const float *p, float (&x)[4]) {
+        const float4 t = *(const float4 *)p;
+        x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+    }
+    static __device__ void store_f32(float *p, const float (&x)[4]) {
+        *(float4 *)p = make_float4(x[0], x[1], x[2], x[3]);
+    }
+    static __device__ void store_bf16(uint16_t *p, const float (&x)[4]) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16_bits(x[0]) | ((uint32_t)f32_to_bf16_bits(x[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16_bits(x[2]) | ((uint32_t)f32_to_bf16_bits(x[3]) << 16);
+        *(uint2 *)p = t;
+    }
+};
+
+// One work unit = W consecutive pairs of a head's rotated part (reads and writes W elements
+// in each half), or W consecutive elements of a head's unrotated tail or of a v row.
+// Grid: x over (row, unit) of the longest item, y = item.
+template <int W> static __device__ __forceinline__ void prepare_body(const lng_k_prepare &a) {
+#pragma clang fp contract(off)
+    const lng_prepare_item it = a.items ? a.items[blockIdx.y] : a.first;
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    const uint32_t r = idx / a.units_per_row;
+    if (r >= it.n) return;
+    uint32_t u = idx % a.units_per_row;
+    const uint32_t half = a.rotary / 2, ru = half / W, uph = ru + (a.dim - a.rotary) / W;
+    const uint32_t qw = a.heads * a.dim, kw = a.kv_heads * a.dim;
+    const uint64_t slot = (it.start + r) % it.slots;
+    const bool bf16 = a.out_dtype == LNG_BF16;
+    const uint32_t es = bf16 ? 2u : 4u;
+
+    const float *src, *bias;
+    char *dst;
+    if (u < (a.heads + a.kv_heads) * uph) {
+        const bool is_q = u < a.heads * uph;
+        if (!is_q) u -= a.heads * uph;
+        const uint32_t head = u / uph, w = u % uph;
+        if (is_q) {
+            src = (const float *)(a.q + it.q_offset) + (uint64_t)r * qw + head * a.dim;
+            bias = a.q_bias ? a.q_bias + head * a.dim : nullptr;
+            dst = a.q_out + it.q_out_offset + ((uint64_t)r * qw + head * a.dim) * es;
+        } else {
+            src = (const float *)(a.k + it.k_offset) + (uint64_t)r * kw + head * a.dim;
+            bias = a.k_bias ? a.k_bias + head * a.dim : nullptr;
+            dst = a.k_cache + it.k_cache_offset + (slot * kw + head * a.dim) * es;
+        }
+        if (w < ru) {
+            const uint32_t i = w * W;
+            float x0[W], x1[W], cs[2][W], y0[W], y1[W];
+            prep_vec<W>::load(src + i, x0);
+            prep_vec<W>::load(src + i + half, x1);
+            if (bias) {
+                float b0[W], b1[W];
+                prep_vec<W>::load(bias + i, b0);
+                prep_vec<W>::load(bias + i + half, b1);
+#pragma unroll
+                for (int e = 0; e < W; ++e) {
+                    x0[e] += b0[e];
+                    x1[e] += b1[e];
+                }
+            }
+            const float *t = (const float *)(a.table + it.table_offset) + ((uint64_t)r * half + i) * 2;
+            if constexpr (W == 4) {
+                float lo[4], hi[4];
+                prep_vec<4>::load(t, lo);
+                prep_vec<4>::load(t + 4, hi);
+                cs[0][0] = lo[0]; cs[1][0] = lo[1]; cs[0][1] = lo[2]; cs[1][1] = lo[3];
+                cs[0][2] = hi[0]; cs[1][2] = hi[1]; cs[0][3] = hi[2]; cs[1][3] = hi[3];
+            } else {
+                cs[0][0] = t[0];
+                cs[1][0] = t[1];
+            }
+#pragma unroll
+            for (int e = 0; e < W; ++e) {
+                y0[e] = x0[e] * cs[0][e] - x1[e] * cs[1][e];
+                y1[e] = x1[e] * cs[0][e] + x0[e] * cs[1][e];
+            }
+            if (bf16) {
+                prep_vec<W>::store_bf16((uint16_t *)dst + i, y0);
+                prep_vec<W>::store_bf16((uint16_t *)dst + i + half, y1);
+            } else {
+                prep_vec<W>::store_f32((float *)dst + i, y0);
+                prep_vec<W>::store_f32((float *)dst + i + half, y1);
+            }
+            return;
+        }
+        const uint32_t j = a.rotary + (w - ru) * W;
+        src += j;
+        if (bias) bias += j;
+        dst += (uint64_t)j * es;
+    } else {
+        u -= (a.heads + a.kv_heads) * uph;
+        const uint32_t j = u * W;
+        src = (const float *)(a.v + it.v_offset) + (uint64_t)r * kw + j;
+        bias = a.v_bias ? a.v_bias + j : nullptr;
+        dst = a.v_cache + it.v_cache_offset + (slot * kw + j) * es;
+    }
+    float x[W];
+    prep_vec<W>::load(src, x);
+    if (bias) {
+        float b[W];
+        prep_vec<W>::load(bias, b);
+#pragma unroll
+        for (int e = 0; e < W; ++e) x[e] += b[e];
+    }
+    if (bf16) prep_vec<W>::store_bf16((uint16_t *)dst, x);
+    else prep_vec<W>::store_f32((float *)dst, x);
+}
+
+extern "C" __global__ __launch_bounds__(256) void lng_prepare_v4(lng_k_prepare a) { prepare_body<4>(a); }
+extern "C" __global__ __launch_bounds__(256) void lng_prepare_v1(lng_k_prepare a) { prepare_body<1>(a); }
+
 // Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).
 extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill a) {
     const uint64_t stride = (uint64_t)gridDim.x * 256u;

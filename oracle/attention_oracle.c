@@ -15,13 +15,18 @@
  *   metal-compute/tests/attention_grouped.rs:47-63    ring layout of a cache (`ring`)
  *   metal-compute/src/apple.rs:1243-1256,1356-1369    accepted / rejected shapes
  *   weights/src/dtype.rs:95-116             bf16 widen / round-to-nearest-even narrow
+ *   gpt-oss/src/model.rs:282-286,389-404,427-433      bias add, rotation by halves, cache append
+ *   gpt-oss/src/gpu.rs:690-697,733-759      rotary table; the same step as GPU dispatches
  *
  * What pins each function (tests/test_oracle_*.py): the three literal bf16 vectors and the
  * round trip over all codes from dtype.rs:183-202; the integer generator reproduced
  * independently in Python; the f32 restatement against the f64 definition; the f64
  * definition against torch's scaled_dot_product_attention with an explicit mask and with
  * the sink written as one extra key of value zero; closed forms (zero queries, constant
- * values, window of one); ring independence; NaN poisoning of rows outside the window.
+ * values, window of one); ring independence; NaN poisoning of rows outside the window;
+ * the rotation against complex multiplication in float64, its composition law and norm; and,
+ * end to end, the reference's tiny-model fixture (transformers' logits within 2e-3) with this
+ * file's attention and pre-attention step inside a numpy restatement of the rest of the model.
  *
  * Build: make -C oracle   (gcc -O2 -fno-fast-math -ffp-contract=off -fopenmp)
  */
@@ -283,4 +288,82 @@ void lng_oracle_attention_rows_f32(const float *q, const float *k, const float *
                    out + (i * heads + head) * dim, positions[i], head / group, kv_heads, dim,
                    window, slots, scale);
     }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * The step before attention (gpt-oss/src/gpu.rs:733-759; CPU form gpt-oss/src/model.rs:427-433):
+ * biases on the projections, rotary position embedding by halves on q and k, new k/v rows
+ * appended to the cache at row position % slots.
+ * ------------------------------------------------------------------------------------------ */
+
+/* metal-compute/src/kernels.metal:1648-1660, apple.rs:1886-1911 (model.rs:282-286 `add`):
+ * dst[r][i] += src[r * src_stride + i]; a stride of 0 adds one row, a bias, to every row. */
+void lng_oracle_add_rows(float *dst, const float *src, uint64_t rows, uint64_t width,
+                         uint64_t src_stride) {
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t i = 0; i < width; ++i) dst[r * width + i] += src[r * src_stride + i];
+}
+
+/* gpt-oss/src/gpu.rs:690-697 (same numbers as model.rs:393-398): per position dim/2 pairs
+ * (cos, sin) of position * inv_freq[i], computed in f64, times the YaRN factor, rounded to f32. */
+void lng_oracle_rope_table(float *table, const double *inv_freq, uint64_t half, double scale,
+                           uint64_t start, uint64_t n) {
+    for (uint64_t p = 0; p < n; ++p)
+        for (uint64_t i = 0; i < half; ++i) {
+            const double angle = (double)(start + p) * inv_freq[i];
+            table[(p * half + i) * 2] = (float)(cos(angle) * scale);
+            table[(p * half + i) * 2 + 1] = (float)(sin(angle) * scale);
+        }
+}
+
+/* model.rs:389-404 on rows, with the partial form of kernels.metal:1673-1690 / apple.rs:1929-1955:
+ * x is [rows][heads][dim]; element i of the first half of a head's first `rotary` dimensions
+ * turns with element i of their second half by the row's pair i; dimensions from `rotary` on
+ * stay. Four products, one difference, one sum, each rounded to f32 (no fused multiply-add:
+ * this file is compiled with -ffp-contract=off). */
+void lng_oracle_rotate_halves(float *x, const float *table, uint64_t rows, uint64_t heads,
+                              uint64_t dim, uint64_t rotary) {
+    const uint64_t half = rotary / 2;
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t h = 0; h < heads; ++h) {
+            float *head = x + (r * heads + h) * dim;
+            for (uint64_t i = 0; i < half; ++i) {
+                const float c = table[(r * half + i) * 2], s = table[(r * half + i) * 2 + 1];
+                const float a = head[i], b = head[i + half];
+                head[i] = a * c - b * s;
+                head[i + half] = b * c + a * s;
+            }
+        }
+}
+
+/* gpu.rs:733-759 as one function: q, k, v are the projections of n positions from `start`
+ * ([n][heads*dim], [n][kv_heads*dim]); biases may be NULL. Writes the prepared queries to
+ * q_out[n][heads*dim] and the prepared k/v rows of position start + r to cache row
+ * (start + r) % slots. bf16 != 0: outputs are bf16 (weights/src/dtype.rs:103-116 rounding of the
+ * f32 results), else f32. */
+void lng_oracle_prepare(const float *q, const float *k, const float *v, const float *q_bias,
+                        const float *k_bias, const float *v_bias, const float *table, void *q_out,
+                        void *k_cache, void *v_cache, uint64_t n, uint64_t start, uint64_t slots,
+                        uint64_t heads, uint64_t kv_heads, uint64_t dim, uint64_t rotary, int bf16) {
+    const uint64_t qw = heads * dim, kw = kv_heads * dim;
+    float *row = (float *)malloc((qw > kw ? qw : kw) * sizeof(float));
+    for (uint64_t r = 0; r < n; ++r) {
+        const uint64_t slot = (start + r) % slots;
+        const float *pair = table + r * (rotary / 2) * 2;
+        memcpy(row, q + r * qw, qw * sizeof(float));
+        if (q_bias) lng_oracle_add_rows(row, q_bias, 1, qw, 0);
+        lng_oracle_rotate_halves(row, pair, 1, heads, dim, rotary);
+        if (bf16) lng_oracle_narrow(row, (uint16_t *)q_out + r * qw, qw);
+        else memcpy((float *)q_out + r * qw, row, qw * sizeof(float));
+        memcpy(row, k + r * kw, kw * sizeof(float));
+        if (k_bias) lng_oracle_add_rows(row, k_bias, 1, kw, 0);
+        lng_oracle_rotate_halves(row, pair, 1, kv_heads, dim, rotary);
+        if (bf16) lng_oracle_narrow(row, (uint16_t *)k_cache + slot * kw, kw);
+        else memcpy((float *)k_cache + slot * kw, row, kw * sizeof(float));
+        memcpy(row, v + r * kw, kw * sizeof(float));
+        if (v_bias) lng_oracle_add_rows(row, v_bias, 1, kw, 0);
+        if (bf16) lng_oracle_narrow(row, (uint16_t *)v_cache + slot * kw, kw);
+        else memcpy((float *)v_cache + slot * kw, row, kw * sizeof(float));
+    }
+    free(row);
 }

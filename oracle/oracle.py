@@ -50,6 +50,11 @@ def _load():
     lib.lng_oracle_attention_rows_f32.argtypes = (
         [_fp, _fp, _fp, _fp, _fp, ctypes.POINTER(_u64)] + [_u64] * 6 + [ctypes.c_float, ctypes.c_int]
     )
+    _dp = ctypes.POINTER(ctypes.c_double)
+    lib.lng_oracle_add_rows.argtypes = [_fp, _fp, _u64, _u64, _u64]
+    lib.lng_oracle_rope_table.argtypes = [_fp, _dp, _u64, ctypes.c_double, _u64, _u64]
+    lib.lng_oracle_rotate_halves.argtypes = [_fp, _fp, _u64, _u64, _u64, _u64]
+    lib.lng_oracle_prepare.argtypes = [_fp] * 7 + [ctypes.c_void_p] * 3 + [_u64] * 7 + [ctypes.c_int]
     return lib
 
 
@@ -168,3 +173,47 @@ def attention_rows_f32(q, k, v, sinks, positions, window=FULL, slots=None, scale
                                        pos.ctypes.data_as(ctypes.POINTER(_u64)), n, heads, kv_heads,
                                        dim, window, slots, float(scale), threads)
     return out
+
+
+def add_rows(dst, src, src_stride):
+    """dst[r] + src[r * src_stride:][:width] (a stride of 0 adds one row to every row)."""
+    out = np.ascontiguousarray(dst, dtype=np.float32).copy()
+    src = np.ascontiguousarray(src, dtype=np.float32)
+    rows, width = out.shape
+    _lib.lng_oracle_add_rows(_f(out), _f(src), rows, width, src_stride)
+    return out
+
+
+def rope_table(inv_freq, scale, start, n):
+    """[n][half][2] f32: (cos, sin) of position * inv_freq, times scale."""
+    inv = np.ascontiguousarray(inv_freq, dtype=np.float64)
+    table = np.empty((n, len(inv), 2), dtype=np.float32)
+    _lib.lng_oracle_rope_table(_f(table), inv.ctypes.data_as(ctypes.POINTER(ctypes.c_double)), len(inv),
+                               float(scale), start, n)
+    return table
+
+
+def rotate_halves(x, table, heads, dim, rotary=None):
+    """x [rows][heads*dim] rotated by table [rows][rotary/2][2]."""
+    out = np.ascontiguousarray(x, dtype=np.float32).copy()
+    table = np.ascontiguousarray(table, dtype=np.float32)
+    _lib.lng_oracle_rotate_halves(_f(out), _f(table), out.shape[0], heads, dim, rotary or dim)
+    return out
+
+
+def prepare(q, k, v, q_bias, k_bias, v_bias, table, k_cache, v_cache, start, heads, kv_heads, dim,
+            rotary=None, bf16=False):
+    """The step before attention on n rows; writes rows (start + r) % slots of k_cache / v_cache
+    in place (f32 arrays, or uint16 bf16 bit arrays when bf16) and returns the prepared queries."""
+    q, k, v = (np.ascontiguousarray(a, dtype=np.float32) for a in (q, k, v))
+    table = np.ascontiguousarray(table, dtype=np.float32)
+    n, slots = q.shape[0], k_cache.shape[0]
+    want = np.uint16 if bf16 else np.float32
+    assert k_cache.dtype == want and v_cache.dtype == want
+    assert k_cache.flags.c_contiguous and v_cache.flags.c_contiguous
+    q_out = np.empty((n, heads * dim), dtype=want)
+    bias = [None if b is None else np.ascontiguousarray(b, dtype=np.float32) for b in (q_bias, k_bias, v_bias)]
+    _lib.lng_oracle_prepare(_f(q), _f(k), _f(v), *[None if b is None else _f(b) for b in bias], _f(table),
+                            q_out.ctypes.data, k_cache.ctypes.data, v_cache.ctypes.data, n, start, slots,
+                            heads, kv_heads, dim, rotary or dim, int(bf16))
+    return q_out

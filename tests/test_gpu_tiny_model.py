@@ -1,0 +1,149 @@
+"""The reference's end-to-end golden (gpt-oss/tests/tiny_oracle.rs:10-40: transformers' logits of a
+4-layer gpt-oss over 40 positions, within 2e-3) with the HIP library doing the step before attention
+and attention itself, through the C ABI, the way gpt-oss/src/gpu.rs:703-806 records them: caches on
+the device, sliding layers in rings of window + chunk rows, one token at a time and in prompt chunks.
+Everything else of the model is the numpy restatement in oracle/tiny_model.py."""
+import os
+
+import numpy as np
+import pytest
+
+from loadngo_amd import compute as C
+from oracle import oracle as orc
+from oracle import tiny_model as tm
+from tests.gpu_common import gpu  # noqa: F401
+from tests.helpers import from_bf16_bits
+
+pytestmark = pytest.mark.gpu
+FIXTURE = os.path.join(os.path.dirname(__file__), "golden", "tiny")
+TOLERANCE = 2e-3  # tiny_oracle.rs:10
+
+
+class DeviceSession:
+    def __init__(self, gpu, model, chunk, dtype, tiled):
+        m = self.m = model
+        self.gpu, self.chunk, self.dtype, self.tiled = gpu, chunk, dtype, tiled
+        self.es = 4 if dtype == C.F32 else 2
+        self.qw, self.kw = m.heads * m.dim, m.kv_heads * m.dim
+        pad = (chunk + 31) // 32 * 32
+        # gpu.rs:567-578: sliding layers hold (window + chunk) rounded up to 32 rows, full layers the context
+        self.slots = [((m.window + chunk + 31) // 32 * 32) if m.is_sliding(l) else 64 for l in range(m.layers_n)]
+        self.q = gpu.buffer(pad * self.qw * 4)
+        self.k = gpu.buffer(chunk * self.kw * 4)
+        self.v = gpu.buffer(chunk * self.kw * 4)
+        self.table = gpu.buffer(chunk * m.dim * 4)
+        self.q_out = gpu.buffer(pad * self.qw * self.es)
+        self.att = gpu.buffer(pad * self.qw * self.es)
+        self.q_out.fill(0)  # rows past n of a padded prompt pass must be finite (apple.rs:1386-1395)
+        self.caches = []
+        for l in range(m.layers_n):
+            pair = (gpu.buffer(self.slots[l] * self.kw * self.es), gpu.buffer(self.slots[l] * self.kw * self.es))
+            for b in pair:
+                b.fill(0 if tiled else 0xFF)  # NaN where the plain operator must never read
+            self.caches.append(pair)
+        self.weights = [[gpu.resident(model.layers[l][n]) for n in ("q_bias", "k_bias", "v_bias", "sinks")]
+                        for l in range(m.layers_n)]
+        self.n = 0
+
+    def prepare(self, l, q, k, v, start):
+        m, n = self.m, q.shape[0]
+        self.n = n
+        self.q.write(q)
+        self.k.write(k)
+        self.v.write(v)
+        self.table.write(C.rope_table(m.inv_freq, m.rope_scale, start, n))
+        kc, vc = self.caches[l]
+        batch = self.gpu.batch([self.q, self.k, self.v, self.table, self.q_out, kc, vc, self.att])
+        qb, kb, vb, sinks = (batch.attach(r) for r in self.weights[l])
+        item = C.PrepareItem(n=n, start=start, slots=self.slots[l])
+        batch.prepare_attention(dict(q=0, k=1, v=2, table=3, q_out=4, k_cache=5, v_cache=6), [item], m.heads,
+                                m.kv_heads, m.dim, m.dim, self.dtype, qb, kb, vb)
+        window = m.window if m.is_sliding(l) else C.FULL
+        shape = C.GroupedShape(n, start, m.heads, m.kv_heads, m.dim, window, self.slots[l], 1.0 / np.sqrt(np.float32(m.dim)))
+        end, slots = start + n, self.slots[l]
+        if self.tiled and n >= 32:  # gpu.rs:777-793
+            pad = (n + 31) // 32 * 32
+            rows = slots if slots < end else (end + 31) // 32 * 32
+            batch.attention_grouped_tiled_with_sinks(
+                (C.Slice(4, 0, pad * self.qw * self.es), C.Slice(5, 0, rows * self.kw * self.es),
+                 C.Slice(6, 0, rows * self.kw * self.es)), sinks, C.Slice(7, 0, pad * self.qw * self.es), shape,
+                self.dtype)
+        else:                       # gpu.rs:794-805
+            rows = min(slots, end)
+            batch.attention_grouped_with_sinks(
+                (C.Slice(4, 0, n * self.qw * self.es), C.Slice(5, 0, rows * self.kw * self.es),
+                 C.Slice(6, 0, rows * self.kw * self.es)), sinks, C.Slice(7, 0, n * self.qw * self.es), shape,
+                self.dtype)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        batch.drop()
+
+    def attention(self, l, start, n, window):
+        if self.dtype == C.F32:
+            return self.att.read(np.float32, count=n * self.qw).reshape(n, self.qw)
+        return from_bf16_bits(self.att.read(np.uint16, count=n * self.qw)).reshape(n, self.qw)
+
+    def close(self):
+        for b in [self.q, self.k, self.v, self.table, self.q_out, self.att] + [b for p in self.caches for b in p] + \
+                [r for w in self.weights for r in w]:
+            b.free()
+
+
+@pytest.fixture(scope="module")
+def model():
+    return tm.TinyModel(os.path.join(FIXTURE, "model.gguf"))
+
+
+@pytest.mark.parametrize("chunk,tiled", [(1, False), (7, False), (40, False), (40, True), (32, True)])
+def test_every_position_matches_transformers_in_f32(gpu, model, chunk, tiled):
+    ids, want = tm.load_fixture(FIXTURE)
+    s = DeviceSession(gpu, model, chunk, C.F32, tiled)
+    try:
+        got = model.forward(ids, s.prepare, s.attention, chunk=chunk)
+    finally:
+        s.close()
+    worst = np.abs(got - want).max(axis=1)
+    assert worst.max() < TOLERANCE, f"position {worst.argmax()}: max error {worst.max()}"
+
+
+class Bf16Shadow:
+    """The CPU oracle with bf16 q, k, v and output decides what the model sees; the device session is
+    fed the same projections layer by layer and each of its attention outputs is held against the
+    oracle's. (End to end in bf16 the logits of this random model are not a usable yardstick: a
+    rounding difference can flip a near-tie in the expert router and move a logit by 0.9.)"""
+
+    def __init__(self, device):
+        self.dev, m = device, device.m
+        self.k = [np.zeros((s, m.kv_heads * m.dim), np.uint16) for s in device.slots]
+        self.v = [np.zeros((s, m.kv_heads * m.dim), np.uint16) for s in device.slots]
+        self.worst = 0.0
+
+    def prepare(self, l, q, k, v, start):
+        m, layer = self.dev.m, self.dev.m.layers[l]
+        self.dev.prepare(l, q, k, v, start)
+        table = orc.rope_table(m.inv_freq, m.rope_scale, start, q.shape[0])
+        self.q = orc.prepare(q, k, v, layer["q_bias"], layer["k_bias"], layer["v_bias"], table, self.k[l], self.v[l],
+                             start, m.heads, m.kv_heads, m.dim, bf16=True)
+
+    def attention(self, l, start, n, window):
+        m, slots = self.dev.m, self.dev.slots[l]
+        want = from_bf16_bits(orc.attention_bf16(self.q.reshape(n, m.heads, m.dim),
+                                                 self.k[l].reshape(slots, m.kv_heads, m.dim),
+                                                 self.v[l].reshape(slots, m.kv_heads, m.dim), m.layers[l]["sinks"],
+                                                 start, window=window, slots=slots)).reshape(n, -1)
+        got = self.dev.attention(l, start, n, window)
+        self.worst = max(self.worst, float(np.abs(got - want).max()))
+        assert not np.isnan(got).any()
+        return want
+
+
+@pytest.mark.parametrize("chunk,tiled", [(1, False), (40, False), (40, True)])
+def test_bf16_session_follows_the_bf16_oracle_layer_by_layer(gpu, model, chunk, tiled):
+    ids, _ = tm.load_fixture(FIXTURE)
+    s = DeviceSession(gpu, model, chunk, C.BF16, tiled)
+    shadow = Bf16Shadow(s)
+    try:
+        model.forward(ids, shadow.prepare, shadow.attention, chunk=chunk)
+    finally:
+        s.close()
+    assert shadow.worst <= 2e-2, shadow.worst

@@ -28,14 +28,9 @@ class OracleSession:
 
     def prepare(self, l, q, k, v, start):
         m, layer = self.m, self.m.layers[l]
-        table = m.rope_table(start, q.shape[0])
-        self.q = tm.rotate_halves(q + layer["q_bias"], table, m.heads, m.dim)
-        k = tm.rotate_halves(k + layer["k_bias"], table, m.kv_heads, m.dim)
-        v = v + layer["v_bias"]
-        rows = self.k[l].shape[0]
-        for i in range(q.shape[0]):
-            self.k[l][(start + i) % rows] = k[i]
-            self.v[l][(start + i) % rows] = v[i]
+        table = orc.rope_table(m.inv_freq, m.rope_scale, start, q.shape[0])
+        self.q = orc.prepare(q, k, v, layer["q_bias"], layer["k_bias"], layer["v_bias"], table,
+                             self.k[l], self.v[l], start, m.heads, m.kv_heads, m.dim)
 
     def attention(self, l, start, n, window):
         m = self.m
