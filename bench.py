@@ -282,6 +282,52 @@ def run_copy(gpu, steps, warmup, nbytes=1 << 30):
             "gpu_ms": g * 1e3, "gbs": 2 * nbytes / g / 1e9}
 
 
+def run_prepare(gpu, steps, warmup):
+    """The step before attention (biases, rotation by halves, bf16 narrowing, ring append) at gpt-oss
+    shapes: a prompt pass of 8192 rows into a flat cache, and one decoding step of 16 sequences (one
+    dispatch each). Bytes: per row 80 heads x 64 f32 in, 64 (cos, sin) f32, 80 x 64 bf16 out; biases once."""
+    qw, kw = H * D, G * D
+    row_bytes = (qw + 2 * kw) * 4 + D * 4 + (qw + 2 * kw) * 2
+    out = {}
+    for label, seqs, n, slots in (("prompt_8192", 1, 8192, 8192), ("decode_16_sequences", 16, 1, 640)):
+        rows = seqs * n
+        bufs = [gpu.buffer(rows * qw * 4), gpu.buffer(rows * kw * 4), gpu.buffer(rows * kw * 4),
+                gpu.buffer(rows * D * 4), gpu.buffer(rows * qw * 2), gpu.buffer(seqs * slots * kw * 2),
+                gpu.buffer(seqs * slots * kw * 2), gpu.buffer((qw + 2 * kw) * 4)]
+        for i in (0, 1, 2, 7):
+            b = gpu.batch([bufs[i]])
+            b.fill_synthetic(C.Slice(0, 0, bufs[i].len), C.F32, 40 + i, 0.5, 0)
+            b.run()
+            b.drop()
+        inv = 150000.0 ** (-np.arange(D // 2, dtype=np.float64) / (D // 2))
+        bufs[3].write(np.concatenate([C.rope_table(inv, 1.3465736, 5000 + 37 * s, n) for s in range(seqs)]))
+        items = C.prepare_items([C.PrepareItem(q_offset=s * n * qw * 4, k_offset=s * n * kw * 4, v_offset=s * n * kw * 4,
+                                               table_offset=s * n * D * 4, q_out_offset=s * n * qw * 2,
+                                               k_cache_offset=s * slots * kw * 2, v_cache_offset=s * slots * kw * 2,
+                                               n=n, start=5000 + 37 * s, slots=slots) for s in range(seqs)])
+        names = dict(q=0, k=1, v=2, table=3, q_out=4, k_cache=5, v_cache=6)
+        bias = [C.Slice(7, 0, qw * 4), C.Slice(7, qw * 4, kw * 4), C.Slice(7, (qw + kw) * 4, kw * 4)]
+
+        def go():
+            batch = gpu.batch(bufs)
+            batch.prepare_attention(names, items, H, G, D, D, C.BF16, *bias)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        for _ in range(warmup):
+            go()
+        runs = sorted(go() for _ in range(max(steps, 5)))
+        g = runs[len(runs) // 2]
+        nbytes = rows * row_bytes + (qw + 2 * kw) * 4
+        out[label] = {"rows": rows, "bytes": nbytes, "gpu_us": g * 1e6, "gbs": nbytes / g / 1e9,
+                      "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS}
+        for b in bufs:
+            b.free()
+    out["kernel"] = "lng_prepare_v4"
+    return out
+
+
 def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
     """The oracle (port of the reference's CPU attention, f32 on widened bf16 inputs) on a
     bounded sample of the headline workload: one sequence, one full-causal and one 128-window
@@ -316,7 +362,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,copy: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,copy,prep: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -327,7 +373,7 @@ def main():
     log("device:", gpu.name())
     extra = {}
     if args.only:
-        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy}
+        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -339,6 +385,8 @@ def main():
         log("c3", extra["c3_ragged_batch"])
         extra["c4_prefill"] = run_prefill(gpu, args.steps, args.warmup)
         log("c4", extra["c4_prefill"])
+        extra["pre_attention_step"] = run_prepare(gpu, args.steps, args.warmup)
+        log("prep", extra["pre_attention_step"])
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx)
     log("c5", r)
     gpu.close()
