@@ -236,24 +236,61 @@ def run_prefill(gpu, steps, warmup, t=8192):
         pairs = w * (w + 1) // 2 + (t - w) * w
         flops = 4 * D * H * pairs
 
-        def go():
+        def go(n=1):
             batch = gpu.batch(bufs)
-            batch.attention_grouped_tiled_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, t * QO), shape, C.BF16)
+            for _ in range(n):
+                batch.attention_grouped_tiled_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, t * QO), shape,
+                                                         C.BF16)
             done = batch.run()
             batch.drop()
-            return done.gpu_time
+            return done.gpu_time / n
 
         for _ in range(warmup):
             go()
         runs = sorted(go() for _ in range(max(steps, 5)))
         g = runs[len(runs) // 2]
+        sustained = go(20)  # 20 launches back to back: no gap before each kernel, steady clocks
         traffic = 2 * t * QO + 2 * t * ROW
         res[name] = {"pairs": pairs, "flops": flops, "gpu_ms": g * 1e3, "tflops": flops / g / 1e12,
                      "mfma_frac": flops / g / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "back_to_back_ms": sustained * 1e3, "back_to_back_tflops": flops / sustained / 1e12,
                      "qkvo_bytes": traffic, "hbm_frac": traffic / g / 1e9 / HBM_PEAK_GBS}
     for b in bufs:
         b.free()
     res["workload"] = "C4 causal prefill, 8192 positions, 64 q / 8 kv heads, head_dim 64, bf16"
+    return res
+
+
+def run_prefill_activity(gpu, steps, warmup, t=8192):
+    """The full-causal prompt pass of configuration 4 on all-zero inputs and on random inputs of two
+    magnitudes, one launch at a time and 50 launches back to back in one batch. Same instructions, same
+    memory traffic: a difference in time is the clock following the switching activity of the data."""
+    res = {}
+    for label, scale in (("zeros", 0.0), ("random_0.5", 0.5), ("random_2.0", 2.0)):
+        q, out = gpu.buffer(t * QO), gpu.buffer(t * QO)
+        k, v = gpu.buffer(t * ROW), gpu.buffer(t * ROW)
+        sinks = gpu.upload(np.zeros(H, np.float32))
+        for i, b in enumerate((q, k, v)):
+            fill(gpu, b, 30 + i, scale=scale)
+        bufs = [q, k, v, out, sinks]
+        sl = (C.Slice(0, 0, t * QO), C.Slice(1, 0, t * ROW), C.Slice(2, 0, t * ROW))
+        shape = C.GroupedShape(t, 0, H, G, D, C.FULL, t, SCALE)
+
+        def go(n):
+            batch = gpu.batch(bufs)
+            for _ in range(n):
+                batch.attention_grouped_tiled_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, t * QO), shape, C.BF16)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time / n
+
+        for _ in range(warmup):
+            go(1)
+        single = sorted(go(1) for _ in range(max(steps, 5)))
+        res[label] = {"single_ms": single[len(single) // 2] * 1e3, "back_to_back_ms": go(50) * 1e3}
+        for b in bufs:
+            b.free()
+    res["workload"] = "C4 full-causal prefill, 8192 positions, inputs of different switching activity"
     return res
 
 
@@ -362,7 +399,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,copy,prep: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -373,7 +410,8 @@ def main():
     log("device:", gpu.name())
     extra = {}
     if args.only:
-        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare}
+        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare,
+                "c4act": run_prefill_activity}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
