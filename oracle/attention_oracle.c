@@ -367,3 +367,80 @@ void lng_oracle_prepare(const float *q, const float *k, const float *v, const fl
     }
     free(row);
 }
+
+/* ------------------------------------------------------------------------------------------
+ * Q8_0 projections (the products either side of attention: gpt-oss/src/gpu.rs:99-138,724-732,
+ * 807-817; CPU form weights/src/q8_0.rs).
+ * ------------------------------------------------------------------------------------------ */
+
+/* weights/src/dtype.rs:123-145: IEEE binary16 bits to f32, exact (subnormals renormalised). */
+float lng_oracle_f16_to_f32(uint16_t bits) {
+    const uint32_t sign = (uint32_t)(bits >> 15) << 31;
+    const uint32_t exponent = (bits >> 10) & 0x1f;
+    uint32_t mantissa = bits & 0x3ff;
+    uint32_t out;
+    if (exponent == 0 && mantissa == 0) {
+        out = sign;
+    } else if (exponent == 0) {
+        int unbiased = -14;
+        while ((mantissa & 0x400) == 0) {
+            mantissa <<= 1;
+            unbiased -= 1;
+        }
+        out = sign | ((uint32_t)(unbiased + 127) << 23) | ((mantissa & 0x3ff) << 13);
+    } else if (exponent == 0x1f) {
+        out = sign | 0x7f800000u | (mantissa << 13);
+    } else {
+        out = sign | ((exponent + 127 - 15) << 23) | (mantissa << 13);
+    }
+    float f;
+    memcpy(&f, &out, 4);
+    return f;
+}
+
+/* weights/src/q8_0.rs:17-31 split_blocks: ggml blocks (2-byte binary16 scale + 32 signed bytes)
+ * into the codes, in order, and the scales, in order: the layout the GPU kernels take. */
+void lng_oracle_q8_split_blocks(const uint8_t *blocks, size_t n_blocks, int8_t *codes, uint16_t *scales) {
+    for (size_t b = 0; b < n_blocks; ++b) {
+        scales[b] = (uint16_t)(blocks[34 * b] | (blocks[34 * b + 1] << 8));
+        memcpy(codes + 32 * b, blocks + 34 * b + 2, 32);
+    }
+}
+
+/* weights/src/q8_0.rs:103-123 mul_rows on the split layout, for n positions (the CPU model calls
+ * it once per position): per block the 32 products code * x are summed in f32 in order, the
+ * block sum is scaled once by d and added to the row's f32 accumulator.
+ * x: n rows x_stride apart, y: n rows y_stride apart (metal-compute/src/apple.rs:987-1013). */
+void lng_oracle_q8_mul(const int8_t *codes, const uint16_t *scales, const float *x, float *y,
+                       uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride) {
+    const uint64_t blocks = cols / 32;
+#pragma omp parallel for schedule(static)
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t p = 0; p < n; ++p) {
+            float acc = 0.0f;
+            for (uint64_t b = 0; b < blocks; ++b) {
+                const float d = lng_oracle_f16_to_f32(scales[r * blocks + b]);
+                float sum = 0.0f;
+                for (int i = 0; i < 32; ++i)
+                    sum += (float)codes[r * cols + 32 * b + i] * x[p * x_stride + 32 * b + i];
+                acc += d * sum;
+            }
+            y[p * y_stride + r] = acc;
+        }
+}
+
+/* The float64 definition the reference's GPU tests hold the products to
+ * (metal-compute/tests/q8_0_and_gpt_oss_glue.rs:139-149): element = scale * code, y = sum in f64. */
+void lng_oracle_q8_mul_f64(const int8_t *codes, const uint16_t *scales, const float *x, double *y,
+                           uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride) {
+    const uint64_t blocks = cols / 32;
+#pragma omp parallel for schedule(static)
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t p = 0; p < n; ++p) {
+            double acc = 0.0;
+            for (uint64_t c = 0; c < cols; ++c)
+                acc += (double)lng_oracle_f16_to_f32(scales[r * blocks + c / 32]) * (double)codes[r * cols + c] *
+                       (double)x[p * x_stride + c];
+            y[p * y_stride + r] = acc;
+        }
+}

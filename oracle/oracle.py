@@ -55,6 +55,12 @@ def _load():
     lib.lng_oracle_rope_table.argtypes = [_fp, _dp, _u64, ctypes.c_double, _u64, _u64]
     lib.lng_oracle_rotate_halves.argtypes = [_fp, _fp, _u64, _u64, _u64, _u64]
     lib.lng_oracle_prepare.argtypes = [_fp] * 7 + [ctypes.c_void_p] * 3 + [_u64] * 7 + [ctypes.c_int]
+    _bp = ctypes.POINTER(ctypes.c_int8)
+    lib.lng_oracle_f16_to_f32.restype = ctypes.c_float
+    lib.lng_oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
+    lib.lng_oracle_q8_split_blocks.argtypes = [ctypes.POINTER(ctypes.c_uint8), ctypes.c_size_t, _bp, _hp]
+    lib.lng_oracle_q8_mul.argtypes = [_bp, _hp, _fp, _fp] + [_u64] * 5
+    lib.lng_oracle_q8_mul_f64.argtypes = [_bp, _hp, _fp, ctypes.POINTER(ctypes.c_double)] + [_u64] * 5
     return lib
 
 
@@ -217,3 +223,46 @@ def prepare(q, k, v, q_bias, k_bias, v_bias, table, k_cache, v_cache, start, hea
                             q_out.ctypes.data, k_cache.ctypes.data, v_cache.ctypes.data, n, start, slots,
                             heads, kv_heads, dim, rotary or dim, int(bf16))
     return q_out
+
+
+def f16_to_f32(bits):
+    """binary16 bit patterns (uint16 array) widened to f32."""
+    b = np.ascontiguousarray(bits, dtype=np.uint16)
+    return np.array([_lib.lng_oracle_f16_to_f32(int(v)) for v in b.reshape(-1)], dtype=np.float32).reshape(b.shape)
+
+
+def q8_split_blocks(raw):
+    """ggml Q8_0 blocks (bytes) -> (codes int8 [32 * blocks], scales uint16 [blocks])."""
+    raw = np.ascontiguousarray(np.frombuffer(raw, dtype=np.uint8) if isinstance(raw, (bytes, bytearray, memoryview)) else raw,
+                               dtype=np.uint8)
+    assert raw.size % 34 == 0, "whole Q8_0 blocks"
+    n = raw.size // 34
+    codes, scales = np.empty(32 * n, np.int8), np.empty(n, np.uint16)
+    _lib.lng_oracle_q8_split_blocks(raw.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)), n,
+                                    codes.ctypes.data_as(ctypes.POINTER(ctypes.c_int8)), _h(scales))
+    return codes, scales
+
+
+def _q8(fn, kind, codes, scales, x, rows, cols, y_stride):
+    codes = np.ascontiguousarray(codes, dtype=np.int8)
+    scales = np.ascontiguousarray(scales, dtype=np.uint16)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert codes.size == rows * cols and scales.size == rows * cols // 32 and cols % 32 == 0
+    n, x_stride = x.shape
+    assert x_stride >= cols
+    y_stride = rows if y_stride is None else y_stride
+    y = np.zeros((n, y_stride), dtype=kind)
+    fn(codes.ctypes.data_as(ctypes.POINTER(ctypes.c_int8)), _h(scales), _f(x),
+       y.ctypes.data_as(ctypes.POINTER(ctypes.c_double if kind == np.float64 else ctypes.c_float)),
+       rows, cols, n, x_stride, y_stride)
+    return y
+
+
+def q8_mul(codes, scales, x, rows, cols, y_stride=None):
+    """y[p] = W x[p], f32 as the reference's CPU product: x is [n][x_stride >= cols]."""
+    return _q8(_lib.lng_oracle_q8_mul, np.float32, codes, scales, x, rows, cols, y_stride)
+
+
+def q8_mul_f64(codes, scales, x, rows, cols, y_stride=None):
+    """The same product by its float64 definition."""
+    return _q8(_lib.lng_oracle_q8_mul_f64, np.float64, codes, scales, x, rows, cols, y_stride)

@@ -162,9 +162,13 @@ class TinyModel:
             assert kind == F32 and int(np.prod(dims)) == n, name
             return np.frombuffer(raw, dtype="<f4").copy()
 
+        self.q8_raw = {}  # tensor name -> (ggml Q8_0 block bytes, rows, cols), for tests of Q8_0 products
+
         def matrix(name, rows, cols):
             dims, kind, raw = t[name]
             assert dims == [cols, rows], (name, dims)
+            if kind == Q8_0:
+                self.q8_raw[name] = (raw, rows, cols)
             return _matrix(kind, raw, rows, cols)
 
         def experts(name, rows, cols):
@@ -242,7 +246,7 @@ class TinyModel:
             out += weight * y
         return out
 
-    def forward(self, ids, prepare, attention, chunk=1):
+    def forward(self, ids, prepare, attention, chunk=1, project=None):
         """Logits [len(ids)][vocab]. Positions are fed `chunk` at a time (1 = `Model::step`,
         model.rs:408-478; more = a prompt pass, gpu.rs:703-827).
 
@@ -251,7 +255,16 @@ class TinyModel:
             q and k, and append k and v to layer l's cache, keeping q for `attention`.
         attention(l, start, n, window) -> [n][heads*dim] f32: layer l's attention output for the
             rows `prepare` was just given.
+        project(name, x) -> [n][rows] f32, optional: the product with the Q8_0 tensor `name`
+            (blk.{l}.attn_{q,k,v,output}.weight; its blocks are in self.q8_raw) instead of this
+            file's dequantise-and-multiply.
         """
+        def mul(l, part, x):
+            name = f"blk.{l}.attn_{part}.weight"
+            if project is not None and name in self.q8_raw:
+                return np.asarray(project(name, np.ascontiguousarray(x, dtype=np.float32)), dtype=np.float32)
+            return _mul(self.layers[l][{"output": "o"}.get(part, part)], x)
+
         logits = np.zeros((len(ids), self.vocab), dtype=np.float32)
         for start in range(0, len(ids), chunk):
             tokens = ids[start:start + chunk]
@@ -259,10 +272,10 @@ class TinyModel:
             h = self.embedding[tokens].copy()
             for l, layer in enumerate(self.layers):
                 x = rms_norm(h, layer["attn_norm"], self.eps)
-                prepare(l, _mul(layer["q"], x), _mul(layer["k"], x), _mul(layer["v"], x), start)
+                prepare(l, mul(l, "q", x), mul(l, "k", x), mul(l, "v", x), start)
                 window = self.window if self.is_sliding(l) else FULL
                 attended = np.asarray(attention(l, start, n, window), dtype=np.float32).reshape(n, -1)
-                h = h + (_mul(layer["o"], attended) + layer["o_bias"])
+                h = h + (mul(l, "output", attended) + layer["o_bias"])
                 x = rms_norm(h, layer["ffn_norm"], self.eps)
                 h = h + np.stack([self.experts_out(layer, x[i]) for i in range(n)])
             logits[start:start + n] = _mul(self.output, rms_norm(h, self.output_norm, self.eps))

@@ -100,3 +100,23 @@ def normal_inputs(seed, t, end, heads, kv_heads, dim, scale=1.0):
     v = (rng.standard_normal((end, kv_heads, dim)) * scale).astype(np.float32)
     sinks = rng.standard_normal(heads).astype(np.float32)
     return q, k, v, sinks
+
+
+# metal-compute/tests/q8_0_and_gpt_oss_glue.rs:58-65: exact binary16 scales of either sign
+Q8_TEST_SCALES = [(0x3800, 0.5), (0x2000, 0.0078125), (0xB600, -0.375), (0x3C00, 1.0), (0x1400, 0.0009765625),
+                  (0x4100, 2.5)]
+# q8_0_and_gpt_oss_glue.rs:160-168: (rows, cols, positions, kind)
+REF_Q8_CASES = [(4096, 2880, 1, "gemv"), (512, 2880, 1, "gemv"), (37, 96, 1, "gemv"), (512, 2880, 5, "gemm"),
+                (37, 96, 13, "gemm"), (2880, 4096, 32, "tiled"), (512, 2880, 96, "tiled")]
+
+
+def q8_test_matrix(rows, cols, seed):
+    """q8_0_and_gpt_oss_glue.rs:56-84 `q8_matrix`: (codes int8, scale bits uint16, elements f64 [rows][cols])."""
+    v = xorshift_values(seed, rows * cols)
+    codes = (v * np.float32(127.9)).astype(np.int32).astype(np.int8)  # `as i8` truncates toward zero
+    sv = xorshift_values(seed + 1, rows * cols // 32)
+    pick = ((((sv + np.float32(1.0)) * np.float32(3.0)).astype(np.int64)) + np.arange(len(sv))) % 6
+    bits = np.array([Q8_TEST_SCALES[i][0] for i in pick], dtype=np.uint16)
+    scale = np.array([Q8_TEST_SCALES[i][1] for i in pick], dtype=np.float64)
+    elements = codes.astype(np.float64).reshape(rows, cols // 32, 32) * scale.reshape(rows, cols // 32, 1)
+    return codes, bits, elements.reshape(rows, cols)
