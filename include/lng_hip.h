@@ -247,6 +247,29 @@ int lng_hip_prepare_attention(lng_batch *batch, const lng_prepare_buffers *buffe
                               const lng_prepare_item *items, size_t n_items, uint64_t heads,
                               uint64_t kv_heads, uint64_t dim, uint64_t rotary, int out_dtype);
 
+/* ---- Q8_0 products: the projections either side of attention (gpt-oss/src/gpu.rs:99-138) ----
+ * `codes` holds each row's signed bytes in order (rows * cols), `scales` one little-endian
+ * binary16 per 32 of them (weights/src/q8_0.rs:17-31 split_blocks makes both from ggml blocks);
+ * element c of row r is scales[(r * cols + c) / 32] * codes[r * cols + c]. x and y are f32.
+ * Refused like the reference: rows or cols == 0 or past u32, cols % 32 != 0, codes or x off a
+ * 16-byte boundary, slices of the wrong length, y overlapping an input or in resident memory. */
+
+/* apple.rs:1812-1830 Batch::gemv_q8_0((codes, scales), x, y, rows, cols): y = W x. */
+int lng_hip_gemv_q8_0(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                      uint64_t rows, uint64_t cols);
+
+/* apple.rs:1833-1854 Batch::gemm_q8_0(..., n, (x_stride, y_stride)): y[p] = W x[p] for n
+ * positions; x holds n rows of cols floats x_stride floats apart (a multiple of 4, >= cols), y n
+ * rows of `rows` floats y_stride apart (apple.rs:987-1013 gemm_args). */
+int lng_hip_gemm_q8_0(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                      uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride);
+
+/* apple.rs:1857-1883 Batch::gemm_q8_0_tiled: the same product for prompt passes; also needs
+ * rows % 64 == 0 and n % 32 == 0 (the caller pads the positions). */
+int lng_hip_gemm_q8_0_tiled(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x,
+                            lng_slice y, uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride,
+                            uint64_t y_stride);
+
 /* Deterministic synthetic data written on the device (benchmarks and full-size tests):
  * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
  * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The

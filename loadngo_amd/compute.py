@@ -123,6 +123,9 @@ SYMBOLS = {
     "lng_hip_fill_synthetic": (ctypes.c_int, [_P, _Slice, ctypes.c_int, _U64, ctypes.c_float, _U64]),
     "lng_hip_add_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64]),
     "lng_hip_rotate_halves": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, _U64]),
+    "lng_hip_gemv_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64]),
+    "lng_hip_gemm_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
+    "lng_hip_gemm_q8_0_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_prepare_attention": (ctypes.c_int, [_P, ctypes.POINTER(_PrepareBuffers), ctypes.POINTER(_PrepareItem),
                                                  ctypes.c_size_t, _U64, _U64, _U64, _U64, ctypes.c_int]),
 }
@@ -228,6 +231,18 @@ class PrepareItem:
 def prepare_items(items):
     """A prepared table of ``PrepareItem`` (built once, reused while the offsets hold)."""
     return (_PrepareItem * len(items))(*[_PrepareItem(*[getattr(i, n) for n in _PREPARE_FIELDS]) for i in items])
+
+
+def split_q8_0_blocks(raw):
+    """ggml ``Q8_0`` blocks (2-byte binary16 scale, then 32 signed bytes) as the two arrays the
+    kernels take: the codes in order (int8) and the scales in order (uint16 bit patterns). Moves bytes
+    only (weights/src/q8_0.rs:17-31 ``split_blocks``)."""
+    blocks = np.frombuffer(raw, dtype=np.uint8) if isinstance(raw, (bytes, bytearray, memoryview)) else np.asarray(raw, np.uint8)
+    if blocks.size % 34 != 0:
+        raise ValueError("whole Q8_0 blocks")
+    blocks = blocks.reshape(-1, 34)
+    return (np.ascontiguousarray(blocks[:, 2:]).view(np.int8).reshape(-1),
+            np.ascontiguousarray(blocks[:, :2]).view("<u2").reshape(-1))
 
 
 def rope_table(inv_freq, scale, start, n):
@@ -426,6 +441,23 @@ class Batch:
         arr = items if isinstance(items, ctypes.Array) else prepare_items(items)
         _check(library().lng_hip_prepare_attention(self._h, ctypes.byref(pb), arr, len(arr), heads, kv_heads, dim,
                                                    dim if rotary is None else rotary, out_dtype))
+
+    def gemv_q8_0(self, matrix, x, y, rows, cols):
+        """``gemv_q8_0((codes, scales), x, y, rows, cols)`` (apple.rs:1812)."""
+        codes, scales = matrix
+        _check(library().lng_hip_gemv_q8_0(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols))
+
+    def gemm_q8_0(self, matrix, x, y, rows, cols, n, strides):
+        """``gemm_q8_0((codes, scales), x, y, rows, cols, n, (x_stride, y_stride))`` (apple.rs:1833)."""
+        codes, scales = matrix
+        _check(library().lng_hip_gemm_q8_0(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols, n,
+                                           strides[0], strides[1]))
+
+    def gemm_q8_0_tiled(self, matrix, x, y, rows, cols, n, strides):
+        """``gemm_q8_0_tiled(...)`` (apple.rs:1857): needs rows % 64, cols % 32 and n % 32 == 0."""
+        codes, scales = matrix
+        _check(library().lng_hip_gemm_q8_0_tiled(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols, n,
+                                                 strides[0], strides[1]))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))

@@ -87,7 +87,8 @@ struct lng_gpu {
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
                   decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
-                  add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr;
+                  add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
+                  q8_split_x = nullptr, q8_stream = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -97,6 +98,8 @@ struct lng_gpu {
     float *scratch_ml = nullptr; // split-K partial (max, sum)
     uint32_t *tickets = nullptr; // split-K arrival counters, zero whenever no dispatch is running
     size_t scratch_o_len = 0, scratch_ml_len = 0, tickets_len = 0;
+    char *scratch_x = nullptr;   // bf16 planes of the positions of a Q8_0 product
+    size_t scratch_x_len = 0;
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
     std::atomic<long> live_buffers{0};
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
@@ -586,6 +589,8 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_rotate_halves", &g->rotate_halves, true},
         {"lng_prepare_v4", &g->prepare_v4, true},
         {"lng_prepare_v1", &g->prepare_v1, true},
+        {"lng_q8_split_x", &g->q8_split_x, true},
+        {"lng_q8_stream", &g->q8_stream, true},
     };
     for (auto &w : wanted) {
         e = hipModuleGetFunction(w.fn, g->module, w.name);
@@ -629,6 +634,7 @@ extern "C" void lng_hip_close(lng_gpu *g) {
     if (g->scratch_o) hipFree(g->scratch_o);
     if (g->scratch_ml) hipFree(g->scratch_ml);
     if (g->tickets) hipFree(g->tickets);
+    if (g->scratch_x) hipFree(g->scratch_x);
     hipStreamDestroy(g->stream);
     hipModuleUnload(g->module);
     delete g;
@@ -1191,6 +1197,112 @@ extern "C" int lng_hip_prepare_attention(lng_batch *b, const lng_prepare_buffers
     b->cmds.push_back(std::move(c));
     b->dispatches += 1;
     return LNG_OK;
+}
+
+namespace {
+
+// Device scratch for the two bf16 planes of x, shared by every Q8_0 product of the gpu (they run
+// in order on one stream, each split immediately before its product).
+int reserve_x(lng_gpu *g, size_t bytes, char **out) {
+    std::lock_guard<std::mutex> lock(g->mu);
+    if (bytes > g->scratch_x_len) {
+        void *p = nullptr;
+        const size_t want = std::max(bytes, g->scratch_x_len * 2);
+        if (hipMalloc(&p, want) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte scratch buffer", want);
+        if (g->scratch_x) g->retired.push_back(g->scratch_x);
+        g->scratch_x = (char *)p;
+        g->scratch_x_len = want;
+    }
+    *out = g->scratch_x;
+    return LNG_OK;
+}
+
+// The three Q8_0 products share their checks (apple.rs:1792-1883) and their kernels.
+int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, const lng_slice &x, const lng_slice &y,
+               uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled) {
+    if (int rc = need_recording(b)) return rc;
+    if (tiled && (rows % 64 != 0 || cols % 32 != 0 || n % 32 != 0)) { // apple.rs:1868-1872
+        return fail(LNG_ERR_DISPATCH, "tiled Q8_0 product needs rows %% 64, cols %% 32 and n %% 32 == 0: %llu x %llu, n %llu",
+                    (unsigned long long)rows, (unsigned long long)cols, (unsigned long long)n);
+    }
+    if (rows == 0 || cols == 0 || !fits_u32(rows) || !fits_u32(cols)) { // apple.rs:889-894
+        return fail(LNG_ERR_DISPATCH, "unsupported shape %llux%llu", (unsigned long long)rows, (unsigned long long)cols);
+    }
+    if (gemm && (n == 0 || x_stride < cols || y_stride < rows || x_stride % 4 != 0)) { // apple.rs:995-999
+        return fail(LNG_ERR_DISPATCH, "%llu positions of %llux%llu with strides %llu/%llu", (unsigned long long)n,
+                    (unsigned long long)rows, (unsigned long long)cols, (unsigned long long)x_stride,
+                    (unsigned long long)y_stride);
+    }
+    for (uint64_t v : {n, x_stride, y_stride}) {
+        if (!fits_u32(v)) return fail(LNG_ERR_DISPATCH, "too large");
+    }
+    if (cols % 32 != 0) return fail(LNG_ERR_DISPATCH, "Q8_0 rows of %llu are not whole blocks", (unsigned long long)cols); // apple.rs:1799-1803
+    Operand oc, os, ox, oy;
+    if (int rc = check_slice(b, "codes", codes, rows * cols, 16, &oc)) return rc;
+    if (int rc = check_slice(b, "scales", scales, rows * cols / 32 * 2, 2, &os)) return rc;
+    if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * 4, 16, &ox)) return rc;
+    if (int rc = check_slice(b, "y", y, ((n - 1) * y_stride + rows) * 4, 4, &oy)) return rc;
+    if (int rc = check_output(b, oy, {&oc, &os, &ox})) return rc;
+    const uint64_t n_pad = (n + 15) / 16 * 16;
+    if (!fits_u32(n_pad * cols)) return fail(LNG_ERR_DISPATCH, "too large");
+    char *planes = nullptr;
+    if (int rc = reserve_x(b->gpu, 2 * n_pad * cols * 2, &planes)) return rc;
+
+    lng_k_q8_split sp{};
+    sp.x = (const float *)((const char *)ox.buf->ptr + x.offset);
+    sp.hi = (uint16_t *)planes;
+    sp.lo = (uint16_t *)(planes + n_pad * cols * 2);
+    sp.n = (uint32_t)n;
+    sp.n_pad = (uint32_t)n_pad;
+    sp.cols = (uint32_t)cols;
+    sp.x_stride = (uint32_t)x_stride;
+    Cmd c0;
+    c0.fn = b->gpu->q8_split_x;
+    c0.name = "lng_q8_split_x";
+    c0.grid[0] = (unsigned)((n_pad * (cols / 4) + 255) / 256);
+    c0.block = 256;
+    set_args(c0, sp);
+    b->cmds.push_back(std::move(c0));
+
+    lng_k_q8 a{};
+    a.codes = (const int8_t *)((const char *)oc.buf->ptr + codes.offset);
+    a.scales = (const uint16_t *)((const char *)os.buf->ptr + scales.offset);
+    a.x_hi = sp.hi;
+    a.x_lo = sp.lo;
+    a.y = (float *)((char *)oy.buf->ptr + y.offset);
+    a.rows = (uint32_t)rows;
+    a.cols = (uint32_t)cols;
+    a.n = (uint32_t)n;
+    a.y_stride = (uint32_t)y_stride;
+    Cmd c1;
+    c1.fn = b->gpu->q8_stream;
+    c1.name = "lng_q8_stream";
+    c1.grid[0] = (unsigned)((rows + 15) / 16);
+    c1.grid[1] = (unsigned)(n_pad / 16);
+    c1.block = 256;
+    if (c1.grid[1] > 65535) return fail(LNG_ERR_DISPATCH, "too many positions for one dispatch");
+    set_args(c1, a);
+    b->cmds.push_back(std::move(c1));
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+} // namespace
+
+extern "C" int lng_hip_gemv_q8_0(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                                 uint64_t rows, uint64_t cols) {
+    return q8_product(b, codes, scales, x, y, rows, cols, 1, cols, rows, false, false);
+}
+
+extern "C" int lng_hip_gemm_q8_0(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                                 uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride) {
+    return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, false);
+}
+
+extern "C" int lng_hip_gemm_q8_0_tiled(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                                       uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride,
+                                       uint64_t y_stride) {
+    return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, true);
 }
 
 extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, uint64_t seed, float scale,

@@ -116,6 +116,31 @@ typedef struct lng_k_prepare {
     uint32_t vec;            /* 1 or 4 */
 } lng_k_prepare;
 
+/* x[n][x_stride] f32 -> two bf16 planes [n_pad][cols]: hi = nearest bf16 of x, lo = nearest bf16
+ * of x - hi; rows n..n_pad are zero. */
+typedef struct lng_k_q8_split {
+    const float *x;
+    uint16_t *hi;
+    uint16_t *lo;
+    uint32_t n;
+    uint32_t n_pad;
+    uint32_t cols;
+    uint32_t x_stride;
+} lng_k_q8_split;
+
+/* y[p][r] = sum over blocks b of scale[r][b] * sum_i codes[r][32b+i] * x[p][32b+i]. */
+typedef struct lng_k_q8 {
+    const int8_t *codes;     /* [rows][cols] */
+    const uint16_t *scales;  /* [rows][cols/32] binary16 */
+    const uint16_t *x_hi;    /* [n_pad][cols] bf16 */
+    const uint16_t *x_lo;
+    float *y;                /* [n][y_stride] */
+    uint32_t rows;
+    uint32_t cols;
+    uint32_t n;
+    uint32_t y_stride;
+} lng_k_q8;
+
 /* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with
  * i' = period ? i % period : i; s = sum of the four 16-bit fields of z; value =
  * (float)(s - 131070) * factor, one f32 multiply, then narrowed if the dtype is bf16.

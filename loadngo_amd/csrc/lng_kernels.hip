@@ -668,6 +668,98 @@ template <int W> static __device__ __forceinline__ void prepare_body(const lng_k
 extern "C" __global__ __launch_bounds__(256) void lng_prepare_v4(lng_k_prepare a) { prepare_body<4>(a); }
 extern "C" __global__ __launch_bounds__(256) void lng_prepare_v1(lng_k_prepare a) { prepare_body<1>(a); }
 
+// =============================================================================================
+// Q8_0 products (Batch::gemv_q8_0 / gemm_q8_0 / gemm_q8_0_tiled, apple.rs:1812-1883):
+// y[p] = W x[p], W = signed bytes with one binary16 scale per 32 of a row, x and y f32.
+//
+// The bytes are exact in bf16 and one 16x16x32 product spans exactly one block of a row, so the
+// matrix unit computes each block's sum of code * x and the block's scale multiplies it once,
+// as the CPU form does (weights/src/q8_0.rs:103-123). x is split beforehand into two bf16
+// planes, hi + lo = x to 16 significant bits, and both go through the matrix unit: the
+// result is within 1e-5 of the float64 definition relative to the largest |y|, the bound the
+// reference holds its own kernels to.
+// =============================================================================================
+extern "C" __global__ __launch_bounds__(256) void lng_q8_split_x(lng_k_q8_split a) {
+    const uint32_t per_row = a.cols / 4;
+    const uint32_t idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= a.n_pad * per_row) return;
+    const uint32_t p = idx / per_row, c = (idx % per_row) * 4u;
+    float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    if (p < a.n) v = *(const float4 *)(a.x + (uint64_t)p * a.x_stride + c);
+    const float x[4] = {v.x, v.y, v.z, v.w};
+    uint16_t hi[4], lo[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        hi[e] = f32_to_bf16_bits(x[e]);
+        lo[e] = f32_to_bf16_bits(x[e] - bf16_bits_to_f32(hi[e]));
+    }
+    const uint64_t at = (uint64_t)p * a.cols + c;
+    *(uint2 *)(a.hi + at) = make_uint2((uint32_t)hi[0] | ((uint32_t)hi[1] << 16), (uint32_t)hi[2] | ((uint32_t)hi[3] << 16));
+    *(uint2 *)(a.lo + at) = make_uint2((uint32_t)lo[0] | ((uint32_t)lo[1] << 16), (uint32_t)lo[2] | ((uint32_t)lo[3] << 16));
+}
+
+// Eight signed bytes as eight bf16 values (exact: |code| <= 128 has at most 8 significant bits, so
+// the upper half of its f32 form is the whole number).
+__device__ __forceinline__ bf16x8 q8_codes_to_bf16(uint2 raw) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t word = i < 2 ? raw.x : raw.y;
+        const float f0 = (float)(int8_t)(word >> (16 * (i & 1)));
+        const float f1 = (float)(int8_t)(word >> (16 * (i & 1) + 8));
+        w[i] = (__float_as_uint(f0) >> 16) | (__float_as_uint(f1) & 0xffff0000u);
+    }
+    return as_bf16x8(make_uint4(w[0], w[1], w[2], w[3]));
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t bits) {
+    return (float)__builtin_bit_cast(_Float16, bits);
+}
+
+// Few positions (one pass of the matrix per 16): a workgroup takes 16 rows, its four wavefronts
+// take every fourth block of the rows and their partial sums meet in LDS. Lane l holds row
+// l % 16 and, of each block, the 8 columns of group l / 16 - as the B operand; positions are the
+// A operand, read as bf16 from the two planes. Grid: x = 16-row tiles, y = 16-position tiles.
+extern "C" __global__ __launch_bounds__(256) void lng_q8_stream(lng_k_q8 a) {
+    __shared__ float s_part[3][64][4];
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t j = lane & 15u, kg = lane >> 4;
+    const uint32_t r0 = blockIdx.x * 16u, p0 = blockIdx.y * 16u;
+    const uint32_t row = r0 + j < a.rows ? r0 + j : a.rows - 1u;
+    const uint32_t blocks = a.cols / 32u;
+    const int8_t *wrow = a.codes + (uint64_t)row * a.cols + 8u * kg;
+    const uint16_t *srow = a.scales + (uint64_t)row * blocks;
+    const uint64_t xoff = (uint64_t)(p0 + j) * a.cols + 8u * kg;
+    floatx4 y = {0.0f, 0.0f, 0.0f, 0.0f};
+    const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t steps = (blocks - wave + 3u) / 4u; // blocks >= 1 > wave - 3
+#pragma unroll 4
+    for (uint32_t step = 0; step < steps; ++step) {
+        const uint32_t b = wave + 4u * step;
+        const uint2 raw = *(const uint2 *)(wrow + 32u * b);
+        const float scale = f16_bits_to_f32(srow[b]);
+        const uint4 xh = *(const uint4 *)(a.x_hi + xoff + 32u * b);
+        const uint4 xl = *(const uint4 *)(a.x_lo + xoff + 32u * b);
+        const bf16x8 wb = q8_codes_to_bf16(raw);
+        floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xh), wb, zero4, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xl), wb, acc, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(scale, acc[i], y[i]);
+    }
+    if (wave != 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) s_part[wave - 1][lane][i] = y[i];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float sum = (y[i] + s_part[0][lane][i]) + (s_part[1][lane][i] + s_part[2][lane][i]);
+        const uint32_t p = p0 + 4u * kg + i; // accumulator row = position, column = matrix row
+        if (p < a.n && r0 + j < a.rows) a.y[(uint64_t)p * a.y_stride + r0 + j] = sum;
+    }
+}
+
 // Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).
 extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill a) {
     const uint64_t stride = (uint64_t)gridDim.x * 256u;

@@ -1,0 +1,156 @@
+"""GPU parity of the Q8_0 products (Batch::gemv_q8_0 / gemm_q8_0 / gemm_q8_0_tiled) through the C
+ABI: the reference's own test (metal-compute/tests/q8_0_and_gpt_oss_glue.rs:155-177: its matrices,
+shapes and bound, largest error below 1e-5 of the largest |y| against float64), strides, refusals,
+and the tiny-model golden with the device doing projections, pre-attention step and attention."""
+import os
+
+import numpy as np
+import pytest
+
+from loadngo_amd import compute as C
+from oracle import oracle as orc
+from oracle import tiny_model as tm
+from tests.gpu_common import gpu  # noqa: F401
+from tests.helpers import REF_Q8_CASES, q8_test_matrix, xorshift_values
+from tests.test_gpu_tiny_model import FIXTURE, TOLERANCE, DeviceSession
+
+pytestmark = pytest.mark.gpu
+
+
+def q8_run(gpu, codes, bits, x, rows, cols, kind, y_stride=None):
+    n, x_stride = x.shape
+    y_stride = rows if y_stride is None else y_stride
+    y_len = ((n - 1) * y_stride + rows) * 4
+    bufs = [gpu.upload(codes), gpu.upload(bits), gpu.upload(x), gpu.buffer(y_len)]
+    bufs[3].fill(0xFF)
+    batch = gpu.batch(bufs)
+    m = (C.Slice(0, 0, codes.nbytes), C.Slice(1, 0, bits.nbytes))
+    xs, ys = C.Slice(2, 0, ((n - 1) * x_stride + cols) * 4), C.Slice(3, 0, y_len)
+    try:
+        if kind == "gemv":
+            batch.gemv_q8_0(m, xs, ys, rows, cols)
+        elif kind == "gemm":
+            batch.gemm_q8_0(m, xs, ys, rows, cols, n, (x_stride, y_stride))
+        else:
+            batch.gemm_q8_0_tiled(m, xs, ys, rows, cols, n, (x_stride, y_stride))
+        assert batch.dispatches() == 1
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        raw = bufs[3].read(np.float32)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    out = np.full((n, y_stride), np.nan, np.float32)
+    out.reshape(-1)[:raw.size] = raw
+    return out
+
+
+@pytest.mark.parametrize("rows,cols,n,kind", REF_Q8_CASES + [(4096, 2880, 16, "gemm"), (2880, 4096, 31, "gemm"),
+                                                             (5120, 2880, 512, "tiled"), (64, 32, 32, "tiled")])
+def test_products_match_the_float64_definition(gpu, rows, cols, n, kind):
+    codes, bits, elements = q8_test_matrix(rows, cols, 7 + rows)
+    x = xorshift_values(11, n * cols).reshape(n, cols)
+    want = x.astype(np.float64) @ elements.T
+    got = q8_run(gpu, codes, bits, x, rows, cols, kind)
+    assert not np.isnan(got).any()
+    error = np.abs(got - want).max() / np.abs(want).max()
+    assert error < 1e-5, f"{rows} x {cols}, {n} positions, {kind}: relative error {error:e}"  # glue.rs:171
+    # and against the f32 CPU form, whose own distance from float64 is of the same size
+    cpu = orc.q8_mul(codes, bits, x, rows, cols)
+    assert np.abs(got - cpu).max() / np.abs(want).max() < 2e-5
+
+
+def test_strided_positions_and_untouched_gaps(gpu):
+    rows, cols, n = 80, 96, 21
+    codes, bits, elements = q8_test_matrix(rows, cols, 3)
+    x = np.full((n, cols + 8), np.nan, np.float32)   # the gap between rows of x is never read
+    x[:, :cols] = xorshift_values(5, n * cols).reshape(n, cols)
+    got = q8_run(gpu, codes, bits, x, rows, cols, "gemm", y_stride=rows + 12)
+    want = x[:, :cols].astype(np.float64) @ elements.T
+    assert np.abs(got[:, :rows] - want).max() / np.abs(want).max() < 1e-5
+    assert np.isnan(got[:-1, rows:]).all()           # 0xFF fill: gaps of y untouched
+
+
+def test_refusals_of_the_reference(gpu):
+    """q8_0_and_gpt_oss_glue.rs:180-210 and the checks of apple.rs:889-894, 995-999, 1799-1806, 1868-1872."""
+    bufs = [gpu.buffer(1 << 16) for _ in range(4)]
+    res = gpu.resident(np.zeros(1 << 14, np.float32))
+    batch = gpu.batch(bufs)
+    s = lambda b, n: C.Slice(b, 0, n)
+    with pytest.raises(C.Dispatch):   # rows of 40 are not whole blocks
+        batch.gemv_q8_0((s(0, 160), s(1, 10)), s(2, 160), s(3, 16), 4, 40)
+    with pytest.raises(C.Dispatch):   # 31 positions in the tiled product
+        batch.gemm_q8_0_tiled((s(0, 2048), s(1, 128)), s(2, 31 * 128), s(3, 31 * 256), 64, 32, 31, (32, 64))
+    with pytest.raises(C.Dispatch):   # 48 rows in the tiled product
+        batch.gemm_q8_0_tiled((s(0, 48 * 32), s(1, 96)), s(2, 32 * 128), s(3, 32 * 48 * 4), 48, 32, 32, (32, 48))
+    good = ((s(0, 64 * 64), s(1, 64 * 2 * 2)), s(2, 5 * 64 * 4), s(3, 5 * 64 * 4), 64, 64, 5, (64, 64))
+    bad = [
+        (good[0], good[1], good[2], 0, 64, 5, (64, 64)),                        # no rows
+        (good[0], good[1], good[2], 64, 64, 0, (64, 64)),                       # no positions
+        (good[0], s(2, 5 * 64 * 4), good[2], 64, 64, 5, (60, 64)),              # x rows closer than cols
+        (good[0], s(2, (4 * 66 + 64) * 4), good[2], 64, 64, 5, (66, 64)),       # x stride not a multiple of 4
+        (good[0], good[1], good[2], 64, 64, 5, (64, 63)),                       # y rows closer than rows
+        ((C.Slice(0, 8, 64 * 64), good[0][1]), good[1], good[2], 64, 64, 5, (64, 64)),   # codes off 16 bytes
+        ((good[0][0], s(1, 100)), good[1], good[2], 64, 64, 5, (64, 64)),       # scales of the wrong length
+        (good[0], C.Slice(2, 4, 5 * 64 * 4), good[2], 64, 64, 5, (64, 64)),     # x off 16 bytes
+        (good[0], good[1], s(0, 5 * 64 * 4), 64, 64, 5, (64, 64)),              # y over the codes
+    ]
+    for case in bad:
+        with pytest.raises(C.Dispatch):
+            batch.gemm_q8_0(*case)
+    with pytest.raises(C.Dispatch):   # output in resident memory
+        att = batch.attach(res)
+        batch.gemm_q8_0(good[0], good[1], C.Slice(att.buffer, 0, 5 * 64 * 4), 64, 64, 5, (64, 64))
+    assert batch.dispatches() == 0
+    batch.gemm_q8_0(*good)
+    assert batch.dispatches() == 1
+    batch.drop()
+    for b in bufs:
+        b.free()
+    res.free()
+
+
+def test_split_blocks_host_helper_matches_the_oracle():
+    raw = np.random.default_rng(0).integers(0, 256, 34 * 50, dtype=np.uint8)
+    codes, scales = C.split_q8_0_blocks(raw.tobytes())
+    want_codes, want_scales = orc.q8_split_blocks(raw)
+    assert np.array_equal(codes, want_codes) and np.array_equal(scales, want_scales)
+
+
+@pytest.mark.parametrize("chunk", [1, 40])
+def test_tiny_model_golden_with_device_projections(gpu, chunk):
+    """Projections (Q8_0), pre-attention step and attention on the device; transformers' logits within 2e-3."""
+    model = tm.TinyModel(os.path.join(FIXTURE, "model.gguf"))
+    ids, want = tm.load_fixture(FIXTURE)
+    held = {}
+    for name, (raw, rows, cols) in model.q8_raw.items():
+        codes, scales = C.split_q8_0_blocks(raw)
+        held[name] = (gpu.resident(codes), gpu.resident(scales), rows, cols)
+
+    def project(name, x):
+        codes, scales, rows, cols = held[name]
+        n = x.shape[0]
+        xb, yb = gpu.upload(x), gpu.buffer(n * rows * 4)
+        batch = gpu.batch([xb, yb])
+        m = (batch.attach(codes), batch.attach(scales))
+        if n == 1:
+            batch.gemv_q8_0(m, C.Slice(0, 0, x.nbytes), C.Slice(1, 0, n * rows * 4), rows, cols)
+        else:
+            batch.gemm_q8_0(m, C.Slice(0, 0, x.nbytes), C.Slice(1, 0, n * rows * 4), rows, cols, n, (cols, rows))
+        batch.run()
+        batch.drop()
+        y = yb.read(np.float32).reshape(n, rows)
+        xb.free()
+        yb.free()
+        return y
+
+    s = DeviceSession(gpu, model, chunk, C.F32, False)
+    try:
+        got = model.forward(ids, s.prepare, s.attention, chunk=chunk, project=project)
+    finally:
+        s.close()
+        for codes, scales, _, _ in held.values():
+            codes.free()
+            scales.free()
+    assert np.abs(got - want).max() < TOLERANCE
