@@ -294,6 +294,52 @@ def run_prefill_activity(gpu, steps, warmup, t=8192):
     return res
 
 
+def run_q8(gpu, steps, warmup):
+    """The Q8_0 projection of gpt-oss-20b's queries (4096 x 2880) for one position, for one decoding
+    step of 16 sequences and for a prompt pass of 8192 positions; the first two are bound by reading the
+    matrix once (rows * cols code bytes + 2 bytes per 32), the last by the matrix unit."""
+    rows, cols = 4096, 2880
+    rng = np.random.default_rng(12)
+    codes = gpu.resident(rng.integers(-127, 128, rows * cols, dtype=np.int8))
+    scales = gpu.resident((rng.random(rows * cols // 32, dtype=np.float32) * 0.01 + 0.001).astype(np.float16).view(np.uint16))
+    out = {}
+    for label, n, kind in (("one_position", 1, "gemv"), ("decode_16_sequences", 16, "gemm"), ("prompt_8192", 8192, "tiled")):
+        x, y = gpu.buffer(n * cols * 4), gpu.buffer(n * rows * 4)
+        b = gpu.batch([x])
+        b.fill_synthetic(C.Slice(0, 0, x.len), C.F32, 77, 0.5, 0)
+        b.run()
+        b.drop()
+
+        def go():
+            batch = gpu.batch([x, y])
+            m = (batch.attach(codes), batch.attach(scales))
+            xs, ys = C.Slice(0, 0, x.len), C.Slice(1, 0, y.len)
+            if kind == "gemv":
+                batch.gemv_q8_0(m, xs, ys, rows, cols)
+            elif kind == "gemm":
+                batch.gemm_q8_0(m, xs, ys, rows, cols, n, (cols, rows))
+            else:
+                batch.gemm_q8_0_tiled(m, xs, ys, rows, cols, n, (cols, rows))
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        for _ in range(warmup):
+            go()
+        runs = sorted(go() for _ in range(max(steps, 5)))
+        g = runs[len(runs) // 2]
+        nbytes = rows * cols + rows * cols // 32 * 2 + n * cols * 4 + n * rows * 4
+        flops = 2 * n * rows * cols
+        out[label] = {"positions": n, "gpu_us": g * 1e6, "bytes": nbytes, "gbs": nbytes / g / 1e9,
+                      "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS, "tflops": flops / g / 1e12}
+        x.free()
+        y.free()
+    codes.free()
+    scales.free()
+    out["workload"] = "Q8_0 product, 4096 x 2880 (gpt-oss-20b query projection), f32 positions"
+    return out
+
+
 def run_copy(gpu, steps, warmup, nbytes=1 << 30):
     """A plain copy of known size through lng_copy_rows: the yardstick that the FETCH_SIZE and
     WRITE_SIZE counters of a profile are scaled by (it reads nbytes and writes nbytes)."""
@@ -399,7 +445,7 @@ def main():
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -411,7 +457,7 @@ def main():
     extra = {}
     if args.only:
         runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare,
-                "c4act": run_prefill_activity}
+                "c4act": run_prefill_activity, "q8": run_q8}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -425,6 +471,8 @@ def main():
         log("c4", extra["c4_prefill"])
         extra["pre_attention_step"] = run_prepare(gpu, args.steps, args.warmup)
         log("prep", extra["pre_attention_step"])
+        extra["q8_0_projection"] = run_q8(gpu, args.steps, args.warmup)
+        log("q8", extra["q8_0_projection"])
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx)
     log("c5", r)
     gpu.close()

@@ -88,7 +88,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
                   decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
-                  q8_split_x = nullptr, q8_stream = nullptr;
+                  q8_split_x = nullptr, q8_stream = nullptr, q8_tiled = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -591,6 +591,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prepare_v1", &g->prepare_v1, true},
         {"lng_q8_split_x", &g->q8_split_x, true},
         {"lng_q8_stream", &g->q8_stream, true},
+        {"lng_q8_tiled", &g->q8_tiled, true},
     };
     for (auto &w : wanted) {
         e = hipModuleGetFunction(w.fn, g->module, w.name);
@@ -1243,44 +1244,52 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
     if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * 4, 16, &ox)) return rc;
     if (int rc = check_slice(b, "y", y, ((n - 1) * y_stride + rows) * 4, 4, &oy)) return rc;
     if (int rc = check_output(b, oy, {&oc, &os, &ox})) return rc;
-    const uint64_t n_pad = (n + 15) / 16 * 16;
-    if (!fits_u32(n_pad * cols)) return fail(LNG_ERR_DISPATCH, "too large");
-    char *planes = nullptr;
-    if (int rc = reserve_x(b->gpu, 2 * n_pad * cols * 2, &planes)) return rc;
-
-    lng_k_q8_split sp{};
-    sp.x = (const float *)((const char *)ox.buf->ptr + x.offset);
-    sp.hi = (uint16_t *)planes;
-    sp.lo = (uint16_t *)(planes + n_pad * cols * 2);
-    sp.n = (uint32_t)n;
-    sp.n_pad = (uint32_t)n_pad;
-    sp.cols = (uint32_t)cols;
-    sp.x_stride = (uint32_t)x_stride;
-    Cmd c0;
-    c0.fn = b->gpu->q8_split_x;
-    c0.name = "lng_q8_split_x";
-    c0.grid[0] = (unsigned)((n_pad * (cols / 4) + 255) / 256);
-    c0.block = 256;
-    set_args(c0, sp);
-    b->cmds.push_back(std::move(c0));
-
     lng_k_q8 a{};
     a.codes = (const int8_t *)((const char *)oc.buf->ptr + codes.offset);
     a.scales = (const uint16_t *)((const char *)os.buf->ptr + scales.offset);
-    a.x_hi = sp.hi;
-    a.x_lo = sp.lo;
+    a.x = (const float *)((const char *)ox.buf->ptr + x.offset);
     a.y = (float *)((char *)oy.buf->ptr + y.offset);
     a.rows = (uint32_t)rows;
     a.cols = (uint32_t)cols;
     a.n = (uint32_t)n;
+    a.x_stride = (uint32_t)x_stride;
     a.y_stride = (uint32_t)y_stride;
     Cmd c1;
-    c1.fn = b->gpu->q8_stream;
-    c1.name = "lng_q8_stream";
-    c1.grid[0] = (unsigned)((rows + 15) / 16);
-    c1.grid[1] = (unsigned)(n_pad / 16);
-    c1.block = 256;
-    if (c1.grid[1] > 65535) return fail(LNG_ERR_DISPATCH, "too many positions for one dispatch");
+    if (n < 32) {
+        // bound by reading the matrix: one pass over it per 16 positions, x split in registers
+        c1.fn = b->gpu->q8_stream;
+        c1.name = "lng_q8_stream";
+        c1.grid[0] = (unsigned)((rows + 15) / 16);
+        c1.grid[1] = (unsigned)((n + 15) / 16);
+        c1.block = 1024;
+    } else {
+        const uint64_t n_pad = (n + 127) / 128 * 128;
+        if (!fits_u32(n_pad * cols) || n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
+        char *planes = nullptr;
+        if (int rc = reserve_x(b->gpu, 2 * n_pad * cols * 2, &planes)) return rc;
+        lng_k_q8_split sp{};
+        sp.x = a.x;
+        sp.hi = (uint16_t *)planes;
+        sp.lo = (uint16_t *)(planes + n_pad * cols * 2);
+        sp.n = (uint32_t)n;
+        sp.n_pad = (uint32_t)n_pad;
+        sp.cols = (uint32_t)cols;
+        sp.x_stride = (uint32_t)x_stride;
+        Cmd c0;
+        c0.fn = b->gpu->q8_split_x;
+        c0.name = "lng_q8_split_x";
+        c0.grid[0] = (unsigned)((n_pad * (cols / 4) + 255) / 256);
+        c0.block = 256;
+        set_args(c0, sp);
+        b->cmds.push_back(std::move(c0));
+        a.x_hi = sp.hi;
+        a.x_lo = sp.lo;
+        c1.fn = b->gpu->q8_tiled;
+        c1.name = "lng_q8_tiled";
+        c1.grid[0] = (unsigned)((rows + 255) / 256);
+        c1.grid[1] = (unsigned)(n_pad / 128);
+        c1.block = 512;
+    }
     set_args(c1, a);
     b->cmds.push_back(std::move(c1));
     b->dispatches += 1;

@@ -132,13 +132,16 @@ typedef struct lng_k_q8_split {
 typedef struct lng_k_q8 {
     const int8_t *codes;     /* [rows][cols] */
     const uint16_t *scales;  /* [rows][cols/32] binary16 */
-    const uint16_t *x_hi;    /* [n_pad][cols] bf16 */
+    const float *x;          /* [n][x_stride] (few positions: split in registers) */
+    const uint16_t *x_hi;    /* [n_pad][cols] bf16 (many positions: the planes lng_q8_split_x wrote) */
     const uint16_t *x_lo;
     float *y;                /* [n][y_stride] */
     uint32_t rows;
     uint32_t cols;
     uint32_t n;
+    uint32_t x_stride;
     uint32_t y_stride;
+    uint32_t pad;
 } lng_k_q8;
 
 /* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with

@@ -674,8 +674,9 @@ extern "C" __global__ __launch_bounds__(256) void lng_prepare_v1(lng_k_prepare a
 //
 // The bytes are exact in bf16 and one 16x16x32 product spans exactly one block of a row, so the
 // matrix unit computes each block's sum of code * x and the block's scale multiplies it once,
-// as the CPU form does (weights/src/q8_0.rs:103-123). x is split beforehand into two bf16
-// planes, hi + lo = x to 16 significant bits, and both go through the matrix unit: the
+// as the CPU form does (weights/src/q8_0.rs:103-123). x is split into two bf16 values,
+// hi + lo = x to 16 significant bits (in registers for few positions, into two planes by
+// lng_q8_split_x beforehand for many), and both go through the matrix unit: the
 // result is within 1e-5 of the float64 definition relative to the largest |y|, the bound the
 // reference holds its own kernels to.
 // =============================================================================================
@@ -716,47 +717,213 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t bits) {
     return (float)__builtin_bit_cast(_Float16, bits);
 }
 
-// Few positions (one pass of the matrix per 16): a workgroup takes 16 rows, its four wavefronts
-// take every fourth block of the rows and their partial sums meet in LDS. Lane l holds row
-// l % 16 and, of each block, the 8 columns of group l / 16 - as the B operand; positions are the
-// A operand, read as bf16 from the two planes. Grid: x = 16-row tiles, y = 16-position tiles.
-extern "C" __global__ __launch_bounds__(256) void lng_q8_stream(lng_k_q8 a) {
-    __shared__ float s_part[3][64][4];
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+// hi + lo = x to 16 significant bits, both bf16.
+__device__ __forceinline__ void q8_split8(const float (&x)[8], bf16x8 &hi, bf16x8 &lo) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const __bf16 h = (__bf16)x[e];
+        hi[e] = h;
+        lo[e] = (__bf16)(x[e] - (float)h);
+    }
+}
+
+// Few positions (one pass of the matrix per 16; bound by reading the matrix): a workgroup takes
+// 16 rows, its sixteen wavefronts take every sixteenth block of the rows and their partial sums
+// meet in LDS. Lane l holds row l % 16 and, of each block, the 8 columns of group l / 16 - the B
+// operand; positions are the A operand, read as f32 and split in registers. All loads of four
+// blocks are issued before the first product. Grid: x = 16-row tiles, y = 16-position tiles.
+#define Q8S_WAVES 16
+extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k_q8 a) {
+    __shared__ float s_part[Q8S_WAVES - 1][4][64];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
     const uint32_t r0 = blockIdx.x * 16u, p0 = blockIdx.y * 16u;
     const uint32_t row = r0 + j < a.rows ? r0 + j : a.rows - 1u;
+    const uint32_t pos = p0 + j < a.n ? p0 + j : a.n - 1u; // rows of the product past n are not stored
     const uint32_t blocks = a.cols / 32u;
     const int8_t *wrow = a.codes + (uint64_t)row * a.cols + 8u * kg;
     const uint16_t *srow = a.scales + (uint64_t)row * blocks;
-    const uint64_t xoff = (uint64_t)(p0 + j) * a.cols + 8u * kg;
+    const float *xrow = a.x + (uint64_t)pos * a.x_stride + 8u * kg;
     floatx4 y = {0.0f, 0.0f, 0.0f, 0.0f};
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    const uint32_t steps = (blocks - wave + 3u) / 4u; // blocks >= 1 > wave - 3
-#pragma unroll 4
-    for (uint32_t step = 0; step < steps; ++step) {
-        const uint32_t b = wave + 4u * step;
-        const uint2 raw = *(const uint2 *)(wrow + 32u * b);
-        const float scale = f16_bits_to_f32(srow[b]);
-        const uint4 xh = *(const uint4 *)(a.x_hi + xoff + 32u * b);
-        const uint4 xl = *(const uint4 *)(a.x_lo + xoff + 32u * b);
-        const bf16x8 wb = q8_codes_to_bf16(raw);
-        floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xh), wb, zero4, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(xl), wb, acc, 0, 0, 0);
+    for (uint32_t b0 = wave; b0 < blocks; b0 += 4u * Q8S_WAVES) {
+        uint2 raw[4];
+        float scale[4];
+        float4 xa[4], xb[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(scale, acc[i], y[i]);
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t b = b0 + u * Q8S_WAVES;
+            const uint32_t bb = b < blocks ? b : b0; // a block past the end repeats a real one, scaled by 0
+            raw[u] = *(const uint2 *)(wrow + 32u * bb);
+            scale[u] = b < blocks ? f16_bits_to_f32(srow[bb]) : 0.0f;
+            xa[u] = *(const float4 *)(xrow + 32u * bb);
+            xb[u] = *(const float4 *)(xrow + 32u * bb + 4u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+            bf16x8 hi, lo;
+            q8_split8(xs, hi, lo);
+            const bf16x8 wb = q8_codes_to_bf16(raw[u]);
+            floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, wb, acc, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(scale[u], acc[i], y[i]);
+        }
     }
     if (wave != 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_part[wave - 1][lane][i] = y[i];
+        for (int i = 0; i < 4; ++i) s_part[wave - 1][i][lane] = y[i];
     }
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const float sum = (y[i] + s_part[0][lane][i]) + (s_part[1][lane][i] + s_part[2][lane][i]);
+        float sum = y[i];
+#pragma unroll
+        for (int w = 0; w < Q8S_WAVES - 1; ++w) sum += s_part[w][i][lane];
         const uint32_t p = p0 + 4u * kg + i; // accumulator row = position, column = matrix row
         if (p < a.n && r0 + j < a.rows) a.y[(uint64_t)p * a.y_stride + r0 + j] = sum;
+    }
+}
+
+// Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128
+// positions, wavefront (w % 4, w / 4) the 64 x 64 corner of it: four 16-row B operands made from
+// the codes it loads itself, four 16-position A operands per plane read from an LDS tile of the
+// two bf16 planes of x that the workgroup stages 64 columns (two blocks) at a time, double
+// buffered. Every (rows, positions) pair of operands gives one block sum per lane-held output;
+// the row's block scale multiplies it into the f32 result.
+#define Q8T_THREADS 512
+#define Q8T_KC 64       // columns per stage
+#define Q8T_XSTRIDE 72  // bf16 per LDS row (144 bytes): conflict-free 16-byte reads down a column
+#define Q8T_POS 128
+extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 a) {
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_POS * Q8T_XSTRIDE]; // [stage][plane]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t j = lane & 15u, kg = lane >> 4;
+    const uint32_t r0 = blockIdx.x * 256u + 64u * (wave & 3u);
+    const uint32_t p0 = blockIdx.y * Q8T_POS;
+    const uint32_t pw = 64u * (wave >> 2); // this wavefront's positions within the tile
+    const uint32_t blocks = a.cols / 32u;
+    const uint32_t stages = (blocks + 1u) / 2u;
+    const bool rows_here = r0 < a.rows; // wavefronts past the last row only help staging
+
+    const int8_t *wrow[4];
+    const uint16_t *srow[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+        const uint32_t r = r0 + 16u * nt + j;
+        const uint32_t row = r < a.rows ? r : a.rows - 1u;
+        wrow[nt] = a.codes + (uint64_t)row * a.cols + 8u * kg;
+        srow[nt] = a.scales + (uint64_t)row * blocks;
+    }
+    // staging: thread -> (plane, position, 16-byte chunk of the stage's 128 bytes), four chunks each
+    const uint32_t st_chunk = tid & 7u, st_pos = tid >> 3; // 64 positions per sweep, 2 sweeps, 2 planes
+    auto fetch = [&](uint32_t stage, uint4 (&v)[4]) {
+        uint32_t col = stage * Q8T_KC + 8u * st_chunk;
+        col = col + 8u <= a.cols ? col : a.cols - 8u; // past the last column: any real data, its block is skipped
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const uint16_t *plane = (q & 1) ? a.x_lo : a.x_hi;
+            const uint32_t p = p0 + st_pos + 64u * (q >> 1); // planes are padded with zero rows to whole tiles
+            v[q] = *(const uint4 *)(plane + (uint64_t)p * a.cols + col);
+        }
+    };
+    auto stash = [&](uint32_t buf, const uint4 (&v)[4]) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            *(uint4 *)(&s_x[buf][q & 1][(st_pos + 64u * (q >> 1)) * Q8T_XSTRIDE + 8u * st_chunk]) = v[q];
+        }
+    };
+    auto load_w = [&](uint32_t stage, uint2 (&raw)[2][4], float (&scale)[2][4]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            const uint32_t b = 2u * stage + kb;
+            const uint32_t bb = b < blocks ? b : blocks - 1u;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                raw[kb][nt] = *(const uint2 *)(wrow[nt] + 32u * bb);
+                scale[kb][nt] = b < blocks ? f16_bits_to_f32(srow[nt][bb]) : 0.0f;
+            }
+        }
+    };
+
+    floatx4 y[4][4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    uint4 xv[4];
+    uint2 raw[2][4];
+    float scale[2][4];
+    fetch(0, xv);
+    stash(0, xv);
+    load_w(0, raw, scale);
+    __syncthreads();
+    for (uint32_t stage = 0; stage < stages; ++stage) {
+        const uint32_t buf = stage & 1u;
+        const bool more = stage + 1u < stages;
+        if (more) fetch(stage + 1u, xv);
+        uint2 raw_next[2][4];
+        float scale_next[2][4];
+        if (more && rows_here) load_w(stage + 1u, raw_next, scale_next);
+        if (rows_here) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                bf16x8 xh[4], xl[4];
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) {
+                    const uint32_t at = (pw + 16u * mt + j) * Q8T_XSTRIDE + 32u * kb + 8u * kg;
+                    xh[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][0][at]));
+                    xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][1][at]));
+                }
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const bf16x8 wb = q8_codes_to_bf16(raw[kb][nt]);
+                    floatx4 acc[4];
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) y[nt][mt][i] = __builtin_fmaf(scale[kb][nt], acc[mt][i], y[nt][mt][i]);
+                    }
+                }
+            }
+        }
+        if (more) {
+            stash(buf ^ 1u, xv);
+            if (rows_here) {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                    for (int nt = 0; nt < 4; ++nt) {
+                        raw[kb][nt] = raw_next[kb][nt];
+                        scale[kb][nt] = scale_next[kb][nt];
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (!rows_here) return;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+        const uint32_t r = r0 + 16u * nt + j;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t p = p0 + pw + 16u * mt + 4u * kg + i;
+                if (p < a.n && r < a.rows) a.y[(uint64_t)p * a.y_stride + r] = y[nt][mt][i];
+            }
+        }
     }
 }
 
