@@ -790,16 +790,32 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128
 // positions, wavefront (w % 4, w / 4) the 64 x 64 corner of it: four 16-row B operands made from
-// the codes it loads itself, four 16-position A operands per plane read from an LDS tile of the
-// two bf16 planes of x that the workgroup stages 64 columns (two blocks) at a time, double
-// buffered. Every (rows, positions) pair of operands gives one block sum per lane-held output;
-// the row's block scale multiplies it into the f32 result.
+// the codes it loads itself (one stage ahead, into registers), four 16-position A operands per
+// plane read from an LDS tile of the two bf16 planes of x. The tile is staged 64 columns (two
+// blocks) at a time, double buffered, by loads that go from global memory straight into LDS
+// (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l, whatever address the lane names;
+// no staging registers, no LDS store instructions). A row of the tile is 8 chunks of 16 bytes
+// with no padding; chunk c of position p is kept at chunk c ^ ((p >> 1) & 7), which makes the 16
+// positions x 16 bytes that one operand read touches fall in 64 different banks.
+// Every (rows, positions) pair of operands gives one block sum per lane-held output; the row's
+// block scale multiplies it into the f32 result.
 #define Q8T_THREADS 512
-#define Q8T_KC 64       // columns per stage
-#define Q8T_XSTRIDE 72  // bf16 per LDS row (144 bytes): conflict-free 16-byte reads down a column
 #define Q8T_POS 128
+#define Q8T_PLANE (Q8T_POS * 64) // bf16 elements of one plane of one stage
+__device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t word = i < 2 ? raw.x : raw.y;
+        const float f0 = (float)(int8_t)(word >> (16 * (i & 1)));
+        const float f1 = (float)(int8_t)(word >> (16 * (i & 1) + 8));
+        w[i] = __builtin_amdgcn_perm(__float_as_uint(f1), __float_as_uint(f0), 0x07060302u); // upper halves
+    }
+    return as_bf16x8(make_uint4(w[0], w[1], w[2], w[3]));
+}
+
 extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 a) {
-    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_POS * Q8T_XSTRIDE]; // [stage][plane]
+    __shared__ __attribute__((aligned(1024))) uint16_t s_x[2][2][Q8T_PLANE]; // [stage][plane]
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
@@ -819,25 +835,30 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         wrow[nt] = a.codes + (uint64_t)row * a.cols + 8u * kg;
         srow[nt] = a.scales + (uint64_t)row * blocks;
     }
-    // staging: thread -> (plane, position, 16-byte chunk of the stage's 128 bytes), four chunks each
-    const uint32_t st_chunk = tid & 7u, st_pos = tid >> 3; // 64 positions per sweep, 2 sweeps, 2 planes
-    auto fetch = [&](uint32_t stage, uint4 (&v)[4]) {
-        uint32_t col = stage * Q8T_KC + 8u * st_chunk;
-        col = col + 8u <= a.cols ? col : a.cols - 8u; // past the last column: any real data, its block is skipped
+    // Staging: wavefront w issues four loads per stage; load q covers plane (4w + q) / 16 and the 8
+    // positions of group (4w + q) % 16; lane l brings position 8 * group + l / 8, physical chunk l % 8.
+    const uint16_t *st_src[4];
+    uint32_t st_chunk[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t idx = 4u * wave + q;
+        const uint32_t pos = 8u * (idx & 15u) + (lane >> 3);
+        st_chunk[q] = (lane & 7u) ^ ((pos >> 1) & 7u); // the logical chunk kept at this physical place
+        const uint16_t *plane = (idx >> 4) ? a.x_lo : a.x_hi;
+        st_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
+    }
+    auto stage_x = [&](uint32_t stage, uint32_t buf) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const uint16_t *plane = (q & 1) ? a.x_lo : a.x_hi;
-            const uint32_t p = p0 + st_pos + 64u * (q >> 1); // planes are padded with zero rows to whole tiles
-            v[q] = *(const uint4 *)(plane + (uint64_t)p * a.cols + col);
+            const uint32_t idx = 4u * wave + q;
+            uint32_t col = stage * 64u + 8u * st_chunk[q];
+            col = col < a.cols ? col : col - 32u; // odd block count: the last stage's second block repeats its first
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(st_src[q] + col),
+                                             (__attribute__((address_space(3))) void *)(&s_x[buf][idx >> 4][(idx & 15u) * 512u]),
+                                             16, 0, 0);
         }
     };
-    auto stash = [&](uint32_t buf, const uint4 (&v)[4]) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            *(uint4 *)(&s_x[buf][q & 1][(st_pos + 64u * (q >> 1)) * Q8T_XSTRIDE + 8u * st_chunk]) = v[q];
-        }
-    };
-    auto load_w = [&](uint32_t stage, uint2 (&raw)[2][4], float (&scale)[2][4]) {
+    auto load_w = [&](uint32_t stage, uint2 (&raw)[2][4], uint16_t (&sbits)[2][4]) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             const uint32_t b = 2u * stage + kb;
@@ -845,7 +866,7 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
                 raw[kb][nt] = *(const uint2 *)(wrow[nt] + 32u * bb);
-                scale[kb][nt] = b < blocks ? f16_bits_to_f32(srow[nt][bb]) : 0.0f;
+                sbits[kb][nt] = b < blocks ? srow[nt][bb] : (uint16_t)0; // a block past the end counts for nothing
             }
         }
     };
@@ -857,59 +878,64 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         for (int mt = 0; mt < 4; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    uint4 xv[4];
-    uint2 raw[2][4];
-    float scale[2][4];
-    fetch(0, xv);
-    stash(0, xv);
-    load_w(0, raw, scale);
-    __syncthreads();
-    for (uint32_t stage = 0; stage < stages; ++stage) {
-        const uint32_t buf = stage & 1u;
-        const bool more = stage + 1u < stages;
-        if (more) fetch(stage + 1u, xv);
-        uint2 raw_next[2][4];
-        float scale_next[2][4];
-        if (more && rows_here) load_w(stage + 1u, raw_next, scale_next);
-        if (rows_here) {
+    // per-lane parts of the operand reads: position pw + 16 mt + j, logical chunk 4 kb + kg
+    uint32_t x_at[4], x_sw[4];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                bf16x8 xh[4], xl[4];
+    for (int mt = 0; mt < 4; ++mt) {
+        const uint32_t pos = pw + 16u * mt + j;
+        x_at[mt] = pos * 64u;
+        x_sw[mt] = (pos >> 1) & 7u;
+    }
+    auto compute = [&](uint32_t buf, const uint2 (&raw)[2][4], const uint16_t (&sbits)[2][4]) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            bf16x8 xh[4], xl[4];
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                const uint32_t at = x_at[mt] + 8u * ((4u * kb + kg) ^ x_sw[mt]);
+                xh[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][0][at]));
+                xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][1][at]));
+            }
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const bf16x8 wb = q8_codes_to_bf16_perm(raw[kb][nt]);
+                const float scale = f16_bits_to_f32(sbits[kb][nt]);
+                floatx4 acc[4];
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) {
-                    const uint32_t at = (pw + 16u * mt + j) * Q8T_XSTRIDE + 32u * kb + 8u * kg;
-                    xh[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][0][at]));
-                    xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][1][at]));
-                }
 #pragma unroll
-                for (int nt = 0; nt < 4; ++nt) {
-                    const bf16x8 wb = q8_codes_to_bf16(raw[kb][nt]);
-                    floatx4 acc[4];
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) y[nt][mt][i] = __builtin_fmaf(scale[kb][nt], acc[mt][i], y[nt][mt][i]);
-                    }
+                    for (int i = 0; i < 4; ++i) y[nt][mt][i] = __builtin_fmaf(scale, acc[mt][i], y[nt][mt][i]);
                 }
             }
         }
-        if (more) {
-            stash(buf ^ 1u, xv);
-            if (rows_here) {
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                    for (int nt = 0; nt < 4; ++nt) {
-                        raw[kb][nt] = raw_next[kb][nt];
-                        scale[kb][nt] = scale_next[kb][nt];
-                    }
-                }
-            }
+    };
+
+    uint2 raw_a[2][4], raw_b[2][4];
+    uint16_t sb_a[2][4], sb_b[2][4];
+    stage_x(0, 0);
+    load_w(0, raw_a, sb_a);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    // two stages per turn so that the register sets swap roles without copies
+    for (uint32_t stage = 0; stage < stages; stage += 2u) {
+        if (stage + 1u < stages) {
+            stage_x(stage + 1u, 1);
+            if (rows_here) load_w(stage + 1u, raw_b, sb_b);
         }
+        if (rows_here) compute(0, raw_a, sb_a);
+        __builtin_amdgcn_s_waitcnt(0); // the direct loads into LDS are counted like any other load
+        __syncthreads();
+        if (stage + 1u >= stages) break;
+        if (stage + 2u < stages) {
+            stage_x(stage + 2u, 0);
+            if (rows_here) load_w(stage + 2u, raw_a, sb_a);
+        }
+        if (rows_here) compute(1, raw_b, sb_b);
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     }
     if (!rows_here) return;
