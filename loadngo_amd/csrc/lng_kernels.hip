@@ -790,17 +790,19 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128
 // positions, wavefront (w % 4, w / 4) the 64 x 64 corner of it: four 16-row B operands made from
-// the codes it loads itself (one stage ahead, into registers), four 16-position A operands per
-// plane read from an LDS tile of the two bf16 planes of x. The tile is staged 64 columns (two
-// blocks) at a time, double buffered, by loads that go from global memory straight into LDS
-// (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l, whatever address the lane names;
-// no staging registers, no LDS store instructions). A row of the tile is 8 chunks of 16 bytes
-// with no padding; chunk c of position p is kept at chunk c ^ ((p >> 1) & 7), which makes the 16
-// positions x 16 bytes that one operand read touches fall in 64 different banks.
-// Every (rows, positions) pair of operands gives one block sum per lane-held output; the row's
-// block scale multiplies it into the f32 result.
+// the codes, four 16-position A operands per plane of x. Codes, planes and block scales are
+// staged in LDS 64 columns (two blocks) at a time, double buffered: the loads of stage s + 1 are
+// issued before stage s is computed and stored to LDS after it, so every byte of the matrix is
+// fetched once per workgroup, in 64-byte runs. Rows of the tiles are unpadded; the 16-byte chunk
+// c of position p is kept at chunk c ^ ((p >> 1) & 7) and chunk c of matrix row r at
+// c ^ ((r >> 2) & 3), which makes the 16 rows that one operand read touches fall in different
+// banks. (Loads that go from global memory straight into LDS were tried for the staging: the
+// compiler then waits for every outstanding one before the first LDS read of a stage, which
+// undoes the overlap.) Every (rows, positions) pair of operands gives one block sum per
+// lane-held output; the row's block scale multiplies it into the f32 result.
 #define Q8T_THREADS 512
 #define Q8T_POS 128
+#define Q8T_ROWS 256
 #define Q8T_PLANE (Q8T_POS * 64) // bf16 elements of one plane of one stage
 __device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
     uint32_t w[4];
@@ -815,60 +817,79 @@ __device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
 }
 
 extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 a) {
-    __shared__ __attribute__((aligned(1024))) uint16_t s_x[2][2][Q8T_PLANE]; // [stage][plane]
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_PLANE]; // [stage % 2][plane]
+    __shared__ __attribute__((aligned(16))) uint8_t s_w[2][Q8T_ROWS * 64];  // [stage % 2]: 64 code bytes per row
+    __shared__ uint16_t s_sc[2][Q8T_ROWS * 2];                              // [stage % 2]: two block scales per row
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
-    const uint32_t r0 = blockIdx.x * 256u + 64u * (wave & 3u);
+    const uint32_t rw = 64u * (wave & 3u); // this wavefront's rows within the tile
+    const uint32_t pw = 64u * (wave >> 2); // and its positions
+    const uint32_t r0 = blockIdx.x * Q8T_ROWS;
     const uint32_t p0 = blockIdx.y * Q8T_POS;
-    const uint32_t pw = 64u * (wave >> 2); // this wavefront's positions within the tile
     const uint32_t blocks = a.cols / 32u;
     const uint32_t stages = (blocks + 1u) / 2u;
-    const bool rows_here = r0 < a.rows; // wavefronts past the last row only help staging
+    const bool rows_here = r0 + rw < a.rows; // wavefronts past the last row only help staging
 
-    const int8_t *wrow[4];
-    const uint16_t *srow[4];
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-        const uint32_t r = r0 + 16u * nt + j;
-        const uint32_t row = r < a.rows ? r : a.rows - 1u;
-        wrow[nt] = a.codes + (uint64_t)row * a.cols + 8u * kg;
-        srow[nt] = a.scales + (uint64_t)row * blocks;
-    }
-    // Staging: wavefront w issues four loads per stage; load q covers plane (4w + q) / 16 and the 8
+    // x staging: wavefront w issues four loads per stage; load q covers plane (4w + q) / 16 and the 8
     // positions of group (4w + q) % 16; lane l brings position 8 * group + l / 8, physical chunk l % 8.
-    const uint16_t *st_src[4];
-    uint32_t st_chunk[4];
+    const uint16_t *x_src[4];
+    uint32_t x_chunk[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
         const uint32_t idx = 4u * wave + q;
         const uint32_t pos = 8u * (idx & 15u) + (lane >> 3);
-        st_chunk[q] = (lane & 7u) ^ ((pos >> 1) & 7u); // the logical chunk kept at this physical place
+        x_chunk[q] = (lane & 7u) ^ ((pos >> 1) & 7u); // the logical chunk kept at this physical place
         const uint16_t *plane = (idx >> 4) ? a.x_lo : a.x_hi;
-        st_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
+        x_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
     }
-    auto stage_x = [&](uint32_t stage, uint32_t buf) {
+    // code staging: two loads per stage; load q covers the 16 rows of group 2w + q; lane l brings row
+    // 16 * group + l / 4, physical chunk l % 4.
+    const int8_t *w_src[2];
+    uint32_t w_chunk[2];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t idx = 4u * wave + q;
-            uint32_t col = stage * 64u + 8u * st_chunk[q];
-            col = col < a.cols ? col : col - 32u; // odd block count: the last stage's second block repeats its first
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(st_src[q] + col),
-                                             (__attribute__((address_space(3))) void *)(&s_x[buf][idx >> 4][(idx & 15u) * 512u]),
-                                             16, 0, 0);
-        }
+    for (int q = 0; q < 2; ++q) {
+        const uint32_t row = 16u * (2u * wave + q) + (lane >> 2);
+        w_chunk[q] = (lane & 3u) ^ ((row >> 2) & 3u);
+        const uint32_t r = r0 + row < a.rows ? r0 + row : a.rows - 1u;
+        w_src[q] = a.codes + (uint64_t)r * a.cols;
+    }
+    // scale staging: thread t brings the scale of row t / 2, block t % 2 of the stage
+    const uint32_t sc_row = r0 + (tid >> 1) < a.rows ? r0 + (tid >> 1) : a.rows - 1u;
+    const uint16_t *sc_src = a.scales + (uint64_t)sc_row * blocks;
+    auto x_col = [&](uint32_t stage, int q) {
+        const uint32_t col = stage * 64u + 8u * x_chunk[q];
+        return col < a.cols ? col : col - 32u; // odd block count: the last stage's second block repeats its first
     };
-    auto load_w = [&](uint32_t stage, uint2 (&raw)[2][4], uint16_t (&sbits)[2][4]) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            const uint32_t b = 2u * stage + kb;
-            const uint32_t bb = b < blocks ? b : blocks - 1u;
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                raw[kb][nt] = *(const uint2 *)(wrow[nt] + 32u * bb);
-                sbits[kb][nt] = b < blocks ? srow[nt][bb] : (uint16_t)0; // a block past the end counts for nothing
-            }
-        }
+    auto w_col = [&](uint32_t stage, int q) {
+        const uint32_t col = stage * 64u + 16u * w_chunk[q];
+        return col < a.cols ? col : col - 32u;
+    };
+    // staged values live in plain scalars so that they stay in registers
+    uint4 sx0, sx1, sx2, sx3, sw0, sw1;
+    uint16_t ssc;
+    auto fetch = [&](uint32_t stage) {
+        sx0 = *(const uint4 *)(x_src[0] + x_col(stage, 0));
+        sx1 = *(const uint4 *)(x_src[1] + x_col(stage, 1));
+        sx2 = *(const uint4 *)(x_src[2] + x_col(stage, 2));
+        sx3 = *(const uint4 *)(x_src[3] + x_col(stage, 3));
+        sw0 = *(const uint4 *)(w_src[0] + w_col(stage, 0));
+        sw1 = *(const uint4 *)(w_src[1] + w_col(stage, 1));
+        const uint32_t b = 2u * stage + (tid & 1u);
+        ssc = b < blocks ? sc_src[b] : (uint16_t)0; // a block past the end counts for nothing
+    };
+    auto x_slot = [&](uint32_t buf, uint32_t q) {
+        const uint32_t idx = 4u * wave + q;
+        return (uint4 *)(&s_x[buf][idx >> 4][(idx & 15u) * 512u + 8u * lane]);
+    };
+    auto stash = [&](uint32_t buf) {
+        *x_slot(buf, 0) = sx0;
+        *x_slot(buf, 1) = sx1;
+        *x_slot(buf, 2) = sx2;
+        *x_slot(buf, 3) = sx3;
+        *(uint4 *)(&s_w[buf][(2u * wave) * 1024u + 16u * lane]) = sw0;
+        *(uint4 *)(&s_w[buf][(2u * wave + 1u) * 1024u + 16u * lane]) = sw1;
+        s_sc[buf][tid] = ssc;
     };
 
     floatx4 y[4][4];
@@ -878,15 +899,18 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         for (int mt = 0; mt < 4; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    // per-lane parts of the operand reads: position pw + 16 mt + j, logical chunk 4 kb + kg
-    uint32_t x_at[4], x_sw[4];
+    // per-lane parts of the operand reads
+    uint32_t x_at[4], x_sw[4], w_at[4], w_sw[4];
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const uint32_t pos = pw + 16u * mt + j;
-        x_at[mt] = pos * 64u;
-        x_sw[mt] = (pos >> 1) & 7u;
+    for (int t = 0; t < 4; ++t) {
+        const uint32_t pos = pw + 16u * t + j; // position, logical chunk 4 kb + kg
+        x_at[t] = pos * 64u;
+        x_sw[t] = (pos >> 1) & 7u;
+        const uint32_t row = rw + 16u * t + j; // matrix row, logical chunk 2 kb + kg / 2, half kg % 2
+        w_at[t] = row * 64u + 8u * (kg & 1u);
+        w_sw[t] = (row >> 2) & 3u;
     }
-    auto compute = [&](uint32_t buf, const uint2 (&raw)[2][4], const uint16_t (&sbits)[2][4]) {
+    auto compute = [&](uint32_t buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
             bf16x8 xh[4], xl[4];
@@ -898,8 +922,9 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
             }
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
-                const bf16x8 wb = q8_codes_to_bf16_perm(raw[kb][nt]);
-                const float scale = f16_bits_to_f32(sbits[kb][nt]);
+                const uint2 raw = *(const uint2 *)(&s_w[buf][w_at[nt] + 16u * ((2u * kb + (kg >> 1)) ^ w_sw[nt])]);
+                const bf16x8 wb = q8_codes_to_bf16_perm(raw);
+                const float scale = f16_bits_to_f32(s_sc[buf][2u * (rw + 16u * nt + j) + kb]);
                 floatx4 acc[4];
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
@@ -914,34 +939,21 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         }
     };
 
-    uint2 raw_a[2][4], raw_b[2][4];
-    uint16_t sb_a[2][4], sb_b[2][4];
-    stage_x(0, 0);
-    load_w(0, raw_a, sb_a);
-    __builtin_amdgcn_s_waitcnt(0);
+    fetch(0);
+    stash(0);
     __syncthreads();
-    // two stages per turn so that the register sets swap roles without copies
-    for (uint32_t stage = 0; stage < stages; stage += 2u) {
-        if (stage + 1u < stages) {
-            stage_x(stage + 1u, 1);
-            if (rows_here) load_w(stage + 1u, raw_b, sb_b);
-        }
-        if (rows_here) compute(0, raw_a, sb_a);
-        __builtin_amdgcn_s_waitcnt(0); // the direct loads into LDS are counted like any other load
-        __syncthreads();
-        if (stage + 1u >= stages) break;
-        if (stage + 2u < stages) {
-            stage_x(stage + 2u, 0);
-            if (rows_here) load_w(stage + 2u, raw_a, sb_a);
-        }
-        if (rows_here) compute(1, raw_b, sb_b);
-        __builtin_amdgcn_s_waitcnt(0);
+    for (uint32_t stage = 0; stage < stages; ++stage) {
+        const uint32_t buf = stage & 1u;
+        const bool more = stage + 1u < stages;
+        if (more) fetch(stage + 1u);
+        if (rows_here) compute(buf);
+        if (more) stash(buf ^ 1u);
         __syncthreads();
     }
     if (!rows_here) return;
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
-        const uint32_t r = r0 + 16u * nt + j;
+        const uint32_t r = r0 + rw + 16u * nt + j;
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
