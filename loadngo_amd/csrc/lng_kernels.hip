@@ -730,9 +730,10 @@ __device__ __forceinline__ void q8_split8(const float (&x)[8], bf16x8 &hi, bf16x
 // Few positions (one pass of the matrix per 16; bound by reading the matrix): a workgroup takes
 // 16 rows, its sixteen wavefronts take every sixteenth block of the rows and their partial sums
 // meet in LDS. Lane l holds row l % 16 and, of each block, the 8 columns of group l / 16 - the B
-// operand; positions are the A operand, read as f32 and split in registers. All loads of four
+// operand; positions are the A operand, read as f32 and split in registers. All loads of eight
 // blocks are issued before the first product. Grid: x = 16-row tiles, y = 16-position tiles.
 #define Q8S_WAVES 16
+#define Q8S_UNROLL 8 // blocks in flight per wavefront: 128 blocks (4096 columns) in one turn
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k_q8 a) {
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
     const uint32_t lane = threadIdx.x & 63u;
@@ -747,12 +748,12 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
     const float *xrow = a.x + (uint64_t)pos * a.x_stride + 8u * kg;
     floatx4 y = {0.0f, 0.0f, 0.0f, 0.0f};
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t b0 = wave; b0 < blocks; b0 += 4u * Q8S_WAVES) {
-        uint2 raw[4];
-        float scale[4];
-        float4 xa[4], xb[4];
+    for (uint32_t b0 = wave; b0 < blocks; b0 += Q8S_UNROLL * Q8S_WAVES) {
+        uint2 raw[Q8S_UNROLL];
+        float scale[Q8S_UNROLL];
+        float4 xa[Q8S_UNROLL], xb[Q8S_UNROLL];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < Q8S_UNROLL; ++u) {
             const uint32_t b = b0 + u * Q8S_WAVES;
             const uint32_t bb = b < blocks ? b : b0; // a block past the end repeats a real one, scaled by 0
             raw[u] = *(const uint2 *)(wrow + 32u * bb);
@@ -761,7 +762,7 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
             xb[u] = *(const float4 *)(xrow + 32u * bb + 4u);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < Q8S_UNROLL; ++u) {
             const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
             bf16x8 hi, lo;
             q8_split8(xs, hi, lo);
