@@ -196,6 +196,12 @@ int lng_hip_attention_decode_batched(lng_batch *batch, uint64_t q_buffer, uint64
 
 /* ---- The step before attention (gpt-oss/src/gpu.rs:733-759) -------------------------------- */
 
+/* apple.rs:1731-1758 Batch::rmsnorm_rows((v, w), rows, (d, stride), eps), f32, in place over the
+ * first d floats of `rows` rows `stride` floats apart: v = w * v / sqrt(mean(v^2) + eps), w of d
+ * floats (gpt-oss/src/model.rs:274-280). Refused: rows == 0, d == 0, stride < d. */
+int lng_hip_rmsnorm_rows(lng_batch *batch, lng_slice v, lng_slice w, uint64_t rows, uint64_t d,
+                         uint64_t stride, float eps);
+
 /* apple.rs:1886-1911 Batch::add_rows(dst, (src, src_stride), rows, width), f32:
  * dst[r][i] += src[r * src_stride + i]; src_stride == 0 adds one row (a bias) to every row.
  * Refused like the reference: rows == 0, width == 0, 0 < src_stride < width. */

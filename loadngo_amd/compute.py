@@ -121,6 +121,7 @@ SYMBOLS = {
                                                         ctypes.c_size_t, _U64, _U64, _U64, ctypes.c_float,
                                                         ctypes.c_int]),
     "lng_hip_fill_synthetic": (ctypes.c_int, [_P, _Slice, ctypes.c_int, _U64, ctypes.c_float, _U64]),
+    "lng_hip_rmsnorm_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, ctypes.c_float]),
     "lng_hip_add_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64]),
     "lng_hip_rotate_halves": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, _U64]),
     "lng_hip_gemv_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64]),
@@ -414,6 +415,11 @@ class Batch:
         _check(library().lng_hip_attention_decode_batched(self._h, q_buffer, k_buffer, v_buffer, out_buffer,
                                                           sinks_buffer, arr, len(items), heads, kv_heads, dim,
                                                           scale, dtype))
+
+    def rmsnorm_rows(self, v_w, rows, d_stride, eps):
+        """``rmsnorm_rows((v, w), rows, (d, stride), eps)`` (apple.rs:1733), f32, in place."""
+        (v, w), (d, stride) = v_w, d_stride
+        _check(library().lng_hip_rmsnorm_rows(self._h, v._c(), w._c(), rows, d, stride, eps))
 
     def add_rows(self, dst, src, rows, width):
         """``add_rows(dst, (src, src_stride), rows, width)`` (apple.rs:1886), f32."""

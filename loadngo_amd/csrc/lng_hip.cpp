@@ -88,7 +88,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
                   decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
-                  q8_split_x = nullptr, q8_stream = nullptr, q8_tiled = nullptr;
+                  q8_split_x = nullptr, q8_stream = nullptr, q8_tiled = nullptr, rmsnorm_rows = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -592,6 +592,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_q8_split_x", &g->q8_split_x, true},
         {"lng_q8_stream", &g->q8_stream, true},
         {"lng_q8_tiled", &g->q8_tiled, true},
+        {"lng_rmsnorm_rows", &g->rmsnorm_rows, true},
     };
     for (auto &w : wanted) {
         e = hipModuleGetFunction(w.fn, g->module, w.name);
@@ -995,6 +996,40 @@ extern "C" int lng_hip_attention_decode_batched(lng_batch *b, uint64_t q_buffer,
     a.dtype = (uint32_t)dtype;
     a.scale = scale;
     if (int rc = record_rows(b, a, (const lng_k_row *)host, n_items, 0, aligned16)) return rc;
+    b->dispatches += 1;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_rmsnorm_rows(lng_batch *b, lng_slice v, lng_slice w, uint64_t rows, uint64_t d, uint64_t stride,
+                                    float eps) {
+    if (int rc = need_recording(b)) return rc;
+    // apple.rs:1740-1744
+    if (rows == 0 || d == 0 || stride < d) {
+        return fail(LNG_ERR_DISPATCH, "unsupported rows: %llu x %llu, stride %llu", (unsigned long long)rows,
+                    (unsigned long long)d, (unsigned long long)stride);
+    }
+    for (uint64_t n : {rows, d, stride}) {
+        if (!fits_u32(n)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)n);
+    }
+    if (!fits_u32(rows * stride)) return fail(LNG_ERR_DISPATCH, "%llu does not fit in u32", (unsigned long long)(rows * stride));
+    Operand ov, ow;
+    if (int rc = check_slice(b, "v", v, ((rows - 1) * stride + d) * 4, 4, &ov)) return rc;
+    if (int rc = check_slice(b, "w", w, d * 4, 4, &ow)) return rc;
+    if (int rc = check_output(b, ov, {&ow})) return rc;
+    lng_k_rmsnorm a{};
+    a.v = (float *)((char *)ov.buf->ptr + v.offset);
+    a.w = (const float *)((const char *)ow.buf->ptr + w.offset);
+    a.rows = (uint32_t)rows;
+    a.d = (uint32_t)d;
+    a.stride = (uint32_t)stride;
+    a.eps = eps;
+    Cmd c;
+    c.fn = b->gpu->rmsnorm_rows;
+    c.name = "lng_rmsnorm_rows";
+    c.grid[0] = (unsigned)((rows + 3) / 4);
+    c.block = 256;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
     b->dispatches += 1;
     return LNG_OK;
 }

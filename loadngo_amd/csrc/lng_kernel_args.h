@@ -87,6 +87,16 @@ typedef struct lng_k_add {
     uint64_t src_stride;
 } lng_k_add;
 
+/* In place: the first d floats of each row (stride floats apart) times w / sqrt(mean of squares + eps). */
+typedef struct lng_k_rmsnorm {
+    float *v;
+    const float *w;
+    uint32_t rows;
+    uint32_t d;
+    uint32_t stride;
+    float eps;
+} lng_k_rmsnorm;
+
 /* In-place rotation by halves of x[rows][heads][dim], f32. */
 typedef struct lng_k_rotate {
     float *x;

@@ -523,6 +523,32 @@ extern "C" __global__ __launch_bounds__(256) void lng_copy_rows(lng_k_copy a) {
 // is switched off in these functions.
 // =============================================================================================
 
+// Batch::rmsnorm_rows (apple.rs:1731-1758; kernels.metal:1087-1117; CPU form model.rs:274-280),
+// in place. One wavefront per row: squares summed in f32 (four partial sums per lane, then across
+// the lanes), scale = 1 / sqrt(mean + eps), each element (v * scale) * w as the CPU form orders it.
+extern "C" __global__ __launch_bounds__(256) void lng_rmsnorm_rows(lng_k_rmsnorm a) {
+#pragma clang fp contract(off)
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t row = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (row >= a.rows) return;
+    float *x = a.v + (uint64_t)row * a.stride;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    uint32_t i = lane;
+    for (; i + 192u < a.d; i += 256u) {
+        const float v0 = x[i], v1 = x[i + 64u], v2 = x[i + 128u], v3 = x[i + 192u];
+        s0 += v0 * v0;
+        s1 += v1 * v1;
+        s2 += v2 * v2;
+        s3 += v3 * v3;
+    }
+    for (; i < a.d; i += 64u) s0 += x[i] * x[i];
+    float ss = (s0 + s1) + (s2 + s3);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    const float scale = 1.0f / sqrtf(ss / (float)a.d + a.eps);
+    for (i = lane; i < a.d; i += 64u) x[i] = x[i] * scale * a.w[i];
+}
+
 // Batch::add_rows (apple.rs:1886-1911; kernels.metal:1648-1660). One thread per element.
 extern "C" __global__ __launch_bounds__(256) void lng_add_rows(lng_k_add a) {
     const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;

@@ -444,3 +444,16 @@ void lng_oracle_q8_mul_f64(const int8_t *codes, const uint16_t *scales, const fl
             y[p * y_stride + r] = acc;
         }
 }
+
+/* gpt-oss/src/model.rs:274-280 rms_norm over rows (the GPU operator's strided form,
+ * metal-compute/src/apple.rs:1731-1758, in place on the first d floats of each row): the mean of
+ * squares in f64, scale = (1 / sqrt(mean + eps)) rounded to f32, each element (v * scale) * w. */
+void lng_oracle_rms_norm_rows(float *v, const float *w, uint64_t rows, uint64_t d, uint64_t stride, float eps) {
+    for (uint64_t r = 0; r < rows; ++r) {
+        float *x = v + r * stride;
+        double ss = 0.0;
+        for (uint64_t i = 0; i < d; ++i) ss += (double)x[i] * (double)x[i];
+        const float scale = (float)(1.0 / sqrt(ss / (double)d + (double)eps));
+        for (uint64_t i = 0; i < d; ++i) x[i] = x[i] * scale * w[i];
+    }
+}

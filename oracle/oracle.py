@@ -61,6 +61,7 @@ def _load():
     lib.lng_oracle_q8_split_blocks.argtypes = [ctypes.POINTER(ctypes.c_uint8), ctypes.c_size_t, _bp, _hp]
     lib.lng_oracle_q8_mul.argtypes = [_bp, _hp, _fp, _fp] + [_u64] * 5
     lib.lng_oracle_q8_mul_f64.argtypes = [_bp, _hp, _fp, ctypes.POINTER(ctypes.c_double)] + [_u64] * 5
+    lib.lng_oracle_rms_norm_rows.argtypes = [_fp, _fp, _u64, _u64, _u64, ctypes.c_float]
     return lib
 
 
@@ -266,3 +267,13 @@ def q8_mul(codes, scales, x, rows, cols, y_stride=None):
 def q8_mul_f64(codes, scales, x, rows, cols, y_stride=None):
     """The same product by its float64 definition."""
     return _q8(_lib.lng_oracle_q8_mul_f64, np.float64, codes, scales, x, rows, cols, y_stride)
+
+
+def rms_norm_rows(v, w, d=None, eps=1e-5):
+    """The first d floats of each row of v [rows][stride] normalised and weighted (a copy)."""
+    out = np.ascontiguousarray(v, dtype=np.float32).copy()
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    rows, stride = out.shape
+    d = stride if d is None else d
+    _lib.lng_oracle_rms_norm_rows(_f(out), _f(w), rows, d, stride, float(eps))
+    return out

@@ -246,7 +246,7 @@ class TinyModel:
             out += weight * y
         return out
 
-    def forward(self, ids, prepare, attention, chunk=1, project=None):
+    def forward(self, ids, prepare, attention, chunk=1, project=None, block=None):
         """Logits [len(ids)][vocab]. Positions are fed `chunk` at a time (1 = `Model::step`,
         model.rs:408-478; more = a prompt pass, gpu.rs:703-827).
 
@@ -255,6 +255,9 @@ class TinyModel:
             q and k, and append k and v to layer l's cache, keeping q for `attention`.
         attention(l, start, n, window) -> [n][heads*dim] f32: layer l's attention output for the
             rows `prepare` was just given.
+        block(l, h, start) -> [n][hidden] f32, optional: the whole attention block of layer l
+            (gpu.rs:703-827 up to the residual add: norm, projections, biases, rotation, cache append,
+            attention, output projection and bias, h + result) in place of everything above.
         project(name, x) -> [n][rows] f32, optional: the product with the Q8_0 tensor `name`
             (blk.{l}.attn_{q,k,v,output}.weight; its blocks are in self.q8_raw) instead of this
             file's dequantise-and-multiply.
@@ -271,11 +274,14 @@ class TinyModel:
             n = len(tokens)
             h = self.embedding[tokens].copy()
             for l, layer in enumerate(self.layers):
-                x = rms_norm(h, layer["attn_norm"], self.eps)
-                prepare(l, mul(l, "q", x), mul(l, "k", x), mul(l, "v", x), start)
-                window = self.window if self.is_sliding(l) else FULL
-                attended = np.asarray(attention(l, start, n, window), dtype=np.float32).reshape(n, -1)
-                h = h + (mul(l, "output", attended) + layer["o_bias"])
+                if block is not None:
+                    h = np.asarray(block(l, np.ascontiguousarray(h, dtype=np.float32), start), dtype=np.float32)
+                else:
+                    x = rms_norm(h, layer["attn_norm"], self.eps)
+                    prepare(l, mul(l, "q", x), mul(l, "k", x), mul(l, "v", x), start)
+                    window = self.window if self.is_sliding(l) else FULL
+                    attended = np.asarray(attention(l, start, n, window), dtype=np.float32).reshape(n, -1)
+                    h = h + (mul(l, "output", attended) + layer["o_bias"])
                 x = rms_norm(h, layer["ffn_norm"], self.eps)
                 h = h + np.stack([self.experts_out(layer, x[i]) for i in range(n)])
             logits[start:start + n] = _mul(self.output, rms_norm(h, self.output_norm, self.eps))

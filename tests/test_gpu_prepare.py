@@ -8,6 +8,7 @@ import pytest
 from loadngo_amd import compute as C
 from oracle import oracle as orc
 from tests.gpu_common import gpu  # noqa: F401
+from tests.helpers import xorshift_values
 
 pytestmark = pytest.mark.gpu
 
@@ -214,3 +215,71 @@ def test_prepare_refuses_what_it_cannot_do_before_recording(gpu):
     for b in bufs:
         b.free()
     res.free()
+
+
+def test_strided_rmsnorm_and_row_copy_touch_only_their_columns(gpu):
+    """metal-compute/tests/glue.rs:241-297: rows of 20 floats, the first 12 normalised in place, columns
+    12..20 copied elsewhere first; bound 2e-6 * (1 + |want|) against the float64 mean of squares."""
+    rows, d, stride = 9, 12, 20
+    v = xorshift_values(20, rows * stride)
+    w = xorshift_values(21, d)
+
+    def record(batch):
+        batch.copy_rows((C.Slice(0, d * 4, ((rows - 1) * stride + 8) * 4), stride),
+                        (C.Slice(2, 0, ((rows - 1) * 16 + 8) * 4), 16), rows, 8)
+        batch.rmsnorm_rows((C.Slice(0, 0, ((rows - 1) * stride + d) * 4), C.Slice(1, 0, d * 4)), rows, (d, stride), 1e-5)
+        for bad in [(0, d, stride), (rows, 0, stride), (rows, d, d - 1)]:   # apple.rs:1740-1744
+            with pytest.raises(C.Dispatch):
+                batch.rmsnorm_rows((C.Slice(0, 0, ((rows - 1) * stride + d) * 4), C.Slice(1, 0, d * 4)), bad[0],
+                                   (bad[1], bad[2]), 1e-5)
+
+    got, copied = _run(gpu, [v, w, np.zeros(rows * 16, np.float32)], record, [0, 2])
+    got = got.view(np.float32).reshape(rows, stride)
+    vv = v.reshape(rows, stride)
+    want = vv.copy()
+    ss = (vv[:, :d].astype(np.float64) ** 2).sum(axis=1)
+    inv = (1.0 / np.sqrt(ss / d + 1e-5)).astype(np.float32)
+    want[:, :d] = w[None, :] * vv[:, :d] * inv[:, None]
+    assert (np.abs(got - want) <= 2e-6 * (1 + np.abs(want))).all()
+    assert np.array_equal(got[:, d:], vv[:, d:])
+    copied = copied.view(np.float32).reshape(rows, 16)
+    assert np.array_equal(copied[:, :8], vv[:, d:d + 8])
+    # and the CPU model's form of the same operator
+    assert (np.abs(got - orc.rms_norm_rows(vv, w, d, 1e-5)) <= 2e-6 * (1 + np.abs(want))).all()
+
+
+def test_rmsnorm_at_the_model_width(gpu):
+    rng = np.random.default_rng(8)
+    rows, d = 37, 2880
+    v = (rng.standard_normal((rows, d)) * 4).astype(np.float32)
+    w = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    (got,) = _run(gpu, [v, w], lambda b: b.rmsnorm_rows((C.Slice(0, 0, v.nbytes), C.Slice(1, 0, w.nbytes)), rows,
+                                                        (d, d), 1e-5), [0])
+    want = orc.rms_norm_rows(v, w, d, 1e-5)
+    assert (np.abs(got.view(np.float32).reshape(rows, d) - want) <= 2e-6 * (1 + np.abs(want))).all()
+
+
+def test_glue_adds_and_rotates_as_the_reference_defines(gpu):
+    """metal-compute/tests/q8_0_and_gpt_oss_glue.rs:212-300, the rotation and the row add with the
+    reference's inputs and bounds (1e-6 against float64; the add exact)."""
+    rows, heads, dim, width = 3, 4, 64, 96
+    x = xorshift_values(1, rows * heads * dim)
+    bias = xorshift_values(2, width)
+    h = xorshift_values(3, rows * width)
+    angle = np.arange(rows * dim // 2, dtype=np.float64) * 0.37
+    table = np.stack([np.cos(angle).astype(np.float32) * np.float32(1.3),
+                      np.sin(angle).astype(np.float32) * np.float32(1.3)], axis=-1).reshape(-1)
+
+    def record(batch):
+        f = lambda b, n: C.Slice(b, 0, n * 4)
+        batch.rotate_halves(f(0, x.size), f(1, table.size), rows, (heads, dim))
+        batch.add_rows(f(2, h.size), (f(3, width), 0), rows, width)
+
+    rotated, added = _run(gpu, [x, table, h, bias], record, [0, 2])
+    rotated = rotated.view(np.float32).reshape(rows, heads, dim).astype(np.float64)
+    xs = x.reshape(rows, heads, dim).astype(np.float64)
+    cs = table.reshape(rows, 1, dim // 2, 2).astype(np.float64)
+    a, b = xs[..., :dim // 2], xs[..., dim // 2:]
+    assert np.abs(rotated[..., :dim // 2] - (a * cs[..., 0] - b * cs[..., 1])).max() < 1e-6
+    assert np.abs(rotated[..., dim // 2:] - (b * cs[..., 0] + a * cs[..., 1])).max() < 1e-6
+    assert np.array_equal(added.view(np.float32), (h.reshape(rows, width) + bias[None, :]).reshape(-1))

@@ -147,3 +147,113 @@ def test_bf16_session_follows_the_bf16_oracle_layer_by_layer(gpu, model, chunk, 
     finally:
         s.close()
     assert shadow.worst <= 2e-2, shadow.worst
+
+
+class DeviceBlocks:
+    """Every layer's whole attention block recorded in one batch, as gpt-oss/src/gpu.rs:703-827 records it:
+    H -> X, RMS norm, the three Q8_0 projections, biases + rotation + cache append (one dispatch here), attention,
+    output projection, its bias, the residual add into H. The host only uploads H and the rotary table and reads
+    H back (the experts stay in numpy)."""
+
+    def __init__(self, gpu, model, chunk, tiled):
+        m = self.m = model
+        self.gpu, self.chunk, self.tiled = gpu, chunk, tiled
+        self.qw, self.kw = m.heads * m.dim, m.kv_heads * m.dim
+        self.pad = pad = (chunk + 31) // 32 * 32
+        self.slots = [((m.window + chunk + 31) // 32 * 32) if m.is_sliding(l) else 64 for l in range(m.layers_n)]
+        f = lambda n: gpu.buffer(n * 4)
+        self.H, self.X, self.TMP = f(pad * m.hidden), f(pad * m.hidden), f(pad * m.hidden)
+        self.Q, self.K, self.V = f(pad * self.qw), f(pad * self.kw), f(pad * self.kw)
+        self.QR, self.ATT, self.TABLE = f(pad * self.qw), f(pad * self.qw), f(pad * m.dim)
+        for b in (self.X, self.QR, self.ATT):
+            b.fill(0)  # padded rows of a tiled pass must be finite
+        self.caches = []
+        for l in range(m.layers_n):
+            pair = (f(self.slots[l] * self.kw), f(self.slots[l] * self.kw))
+            for b in pair:
+                b.fill(0 if tiled else 0xFF)
+            self.caches.append(pair)
+        self.res = []
+        for l in range(m.layers_n):
+            layer, r = m.layers[l], {}
+            for part in ("q", "k", "v", "output"):
+                raw, rows, cols = m.q8_raw[f"blk.{l}.attn_{part}.weight"]
+                codes, scales = C.split_q8_0_blocks(raw)
+                r[part] = (gpu.resident(codes), gpu.resident(scales), rows, cols)
+            for name in ("attn_norm", "q_bias", "k_bias", "v_bias", "o_bias", "sinks"):
+                r[name] = gpu.resident(layer[name])
+            self.res.append(r)
+
+    def block(self, l, h, start):
+        m, n, r = self.m, h.shape[0], self.res[l]
+        hidden, qw, kw = m.hidden, self.qw, self.kw
+        self.H.write(h)
+        self.TABLE.write(C.rope_table(m.inv_freq, m.rope_scale, start, n))
+        kc, vc = self.caches[l]
+        bufs = [self.H, self.X, self.Q, self.K, self.V, self.TABLE, self.QR, kc, vc, self.ATT, self.TMP]
+        H, X, Q, K, V, TABLE, QR, KC, VC, ATT, TMP = range(11)
+        batch = self.gpu.batch(bufs)
+        rows_of = lambda b, w, count=n: C.Slice(b, 0, count * w * 4)
+        tiled = self.tiled and n >= 32
+        n_run = (n + 31) // 32 * 32 if tiled else n
+
+        def mul(part, x, y):  # gpu.rs:119-137
+            codes, scales, rows, cols = r[part]
+            mat = (batch.attach(codes), batch.attach(scales))
+            xs, ys = rows_of(x, cols, n_run), rows_of(y, rows, n_run)
+            if n == 1:
+                batch.gemv_q8_0(mat, xs, ys, rows, cols)
+            elif tiled and rows % 64 == 0:
+                batch.gemm_q8_0_tiled(mat, xs, ys, rows, cols, n_run, (cols, rows))
+            else:
+                batch.gemm_q8_0(mat, xs, ys, rows, cols, n_run, (cols, rows))
+
+        batch.copy_rows((rows_of(H, hidden), hidden), (rows_of(X, hidden), hidden), n, hidden)
+        batch.rmsnorm_rows((rows_of(X, hidden), batch.attach(r["attn_norm"])), n, (hidden, hidden), m.eps)
+        mul("q", X, Q)
+        mul("k", X, K)
+        mul("v", X, V)
+        item = C.PrepareItem(n=n, start=start, slots=self.slots[l])
+        batch.prepare_attention(dict(q=Q, k=K, v=V, table=TABLE, q_out=QR, k_cache=KC, v_cache=VC), [item], m.heads,
+                                m.kv_heads, m.dim, m.dim, C.F32, batch.attach(r["q_bias"]), batch.attach(r["k_bias"]),
+                                batch.attach(r["v_bias"]))
+        window = m.window if m.is_sliding(l) else C.FULL
+        slots, end = self.slots[l], start + n
+        shape = C.GroupedShape(n, start, m.heads, m.kv_heads, m.dim, window, slots, 1.0 / np.sqrt(np.float32(m.dim)))
+        sinks = batch.attach(r["sinks"])
+        if tiled:
+            rows = slots if slots < end else (end + 31) // 32 * 32
+            batch.attention_grouped_tiled_with_sinks((rows_of(QR, qw, n_run), rows_of(KC, kw, rows), rows_of(VC, kw, rows)),
+                                                     sinks, rows_of(ATT, qw, n_run), shape, C.F32)
+        else:
+            rows = min(slots, end)
+            batch.attention_grouped_with_sinks((rows_of(QR, qw), rows_of(KC, kw, rows), rows_of(VC, kw, rows)), sinks,
+                                               rows_of(ATT, qw), shape, C.F32)
+        mul("output", ATT, TMP)
+        batch.add_rows(rows_of(TMP, hidden), (batch.attach(r["o_bias"]), 0), n, hidden)
+        batch.add_rows(rows_of(H, hidden), (rows_of(TMP, hidden), hidden), n, hidden)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        batch.drop()
+        return self.H.read(np.float32, count=n * hidden).reshape(n, hidden)
+
+    def close(self):
+        for b in [self.H, self.X, self.TMP, self.Q, self.K, self.V, self.QR, self.ATT, self.TABLE] + \
+                [b for p in self.caches for b in p]:
+            b.free()
+        for r in self.res:
+            for v in r.values():
+                for b in (v[:2] if isinstance(v, tuple) else (v,)):
+                    b.free()
+
+
+@pytest.mark.parametrize("chunk,tiled", [(1, False), (9, False), (40, False), (40, True)])
+def test_whole_attention_blocks_on_the_device_match_transformers(gpu, model, chunk, tiled):
+    ids, want = tm.load_fixture(FIXTURE)
+    s = DeviceBlocks(gpu, model, chunk, tiled)
+    try:
+        got = model.forward(ids, None, None, chunk=chunk, block=s.block)
+    finally:
+        s.close()
+    worst = np.abs(got - want).max(axis=1)
+    assert worst.max() < TOLERANCE, f"position {worst.argmax()}: max error {worst.max()}"

@@ -102,3 +102,20 @@ def test_prepare_is_bias_rotation_and_a_ring_append(n, start, slots, bf16):
     # without biases
     q2 = orc.prepare(q, k, v, None, None, None, table, kc, vc, start, heads, kv_heads, dim, bf16=bf16)
     np.testing.assert_array_equal(q2, cast(tm.rotate_halves(q, table, heads, dim)))
+
+
+def test_rms_norm_is_the_cpu_models_and_has_unit_mean_square():
+    """model.rs:274-280: against an independent numpy restatement bit for bit, the strided form
+    leaves the other columns alone, and with unit weights the result has mean square 1 - eps-ish."""
+    rng = np.random.default_rng(6)
+    rows, d, stride = 7, 2880, 2890
+    v = rng.standard_normal((rows, stride)).astype(np.float32) * np.float32(3.0)
+    w = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    got = orc.rms_norm_rows(v, w, d, 1e-5)
+    assert np.array_equal(got[:, :d], tm.rms_norm(v[:, :d], w, 1e-5))
+    assert np.array_equal(got[:, d:], v[:, d:])
+    unit = orc.rms_norm_rows(v, np.ones(d, np.float32), d, 1e-5)[:, :d].astype(np.float64)
+    np.testing.assert_allclose((unit ** 2).mean(axis=1), 1.0, rtol=1e-5)
+    # scaling the input changes nothing but what eps contributes
+    np.testing.assert_allclose(orc.rms_norm_rows(v * 8, w, d, 0.0)[:, :d], orc.rms_norm_rows(v, w, d, 0.0)[:, :d],
+                               rtol=3e-7, atol=0)
