@@ -128,7 +128,10 @@ int lng_hip_batch_barrier(lng_batch *batch);
 /* apple.rs:2202 Batch::commit(proactor, on_done) — submits without blocking. `on_done` runs
  * once on a library thread when the GPU has finished (the Rust shim re-posts it to the
  * caller's proactor, as apple.rs:2231-2232 does); it may be NULL. The batch handle stays
- * valid for lng_hip_batch_wait / lng_hip_batch_drop. */
+ * valid for lng_hip_batch_wait / lng_hip_batch_drop, neither of which may be called from
+ * inside `on_done` (they wait for the thread that is running it). Batches may be recorded on
+ * different threads at once; their submissions are serialised, and the dispatches of one batch
+ * run back to back on the device. */
 int lng_hip_batch_commit(lng_batch *batch, lng_on_done on_done, void *user);
 /* Blocks until a committed batch has finished; gpu_seconds (may be NULL) receives the time
  * between its first and last dispatch on the device (Completed.gpu_time, apple.rs:2219-2221). */

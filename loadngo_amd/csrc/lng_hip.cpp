@@ -93,6 +93,7 @@ struct lng_gpu {
     unsigned cus = 256;
 
     std::mutex mu;
+    std::mutex submit_mu; // one batch at a time puts its kernels on the stream: they share the scratch buffers
     std::vector<Table> free_tables;
     float *scratch_o = nullptr;  // split-K partial outputs, grown on demand
     float *scratch_ml = nullptr; // split-K partial (max, sum)
@@ -356,10 +357,12 @@ void worker_loop(lng_gpu *g) {
             b->on_done(&done, b->user);
         }
         {
+            // Notified under the lock: a waiter may delete the batch as soon as it sees Done, and
+            // it cannot see it before this thread has let go of the batch for good.
             std::lock_guard<std::mutex> lock(b->mu);
             b->state = lng_batch::Done;
+            b->cv.notify_all();
         }
-        b->cv.notify_all();
     }
 }
 
@@ -777,6 +780,9 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
     hipSetDevice(g->device);
     hipError_t e = hipEventCreate(&b->ev0);
     if (e == hipSuccess) e = hipEventCreate(&b->ev1);
+    // The dispatches of one batch stay together on the stream: split-K partials, arrival counters and
+    // the planes of a Q8_0 product live in scratch that the next dispatch of any batch reuses.
+    std::unique_lock<std::mutex> submitting(g->submit_mu);
     if (e == hipSuccess) e = hipEventRecord(b->ev0, g->stream);
     // the row tables of every batched dispatch, one copy per table block, ahead of the kernels
     for (size_t i = 0; e == hipSuccess && i < b->tables.size(); ++i) {
@@ -799,6 +805,7 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
         }
     }
     if (e == hipSuccess) e = hipEventRecord(b->ev1, g->stream);
+    submitting.unlock();
     b->on_done = on_done;
     b->user = user;
     b->state = lng_batch::Committed;
