@@ -258,8 +258,21 @@ __device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_ro
         const uint32_t d = idx & 63u;
         const float *po = a.partial_o + (((uint64_t)blockIdx.y * a.n_chunks) * group + h) * 64u + d;
         const uint64_t step = (uint64_t)group * 64u;
+        // sixteen loads in flight per turn: the merge is a chain of memory latencies otherwise
         float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
         uint32_t c = 0;
+        for (; c + 16 <= row_chunks; c += 16) {
+            float x[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) x[u] = load_partial<COHERENT>(po + (c + u) * step);
+#pragma unroll
+            for (int u = 0; u < 16; u += 4) {
+                o0 += x[u] * s_w[h][c + u];
+                o1 += x[u + 1] * s_w[h][c + u + 1];
+                o2 += x[u + 2] * s_w[h][c + u + 2];
+                o3 += x[u + 3] * s_w[h][c + u + 3];
+            }
+        }
         for (; c + 4 <= row_chunks; c += 4) {
             const float x0 = load_partial<COHERENT>(po + (c + 0) * step);
             const float x1 = load_partial<COHERENT>(po + (c + 1) * step);
