@@ -61,19 +61,28 @@ def fill(gpu, buf, seed, scale=0.5, period=0):
 
 
 # ------------------------------------------------------------------------------------------------
-def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
-    """Configuration 5: the 24-layer decode stack."""
+def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24, kv_gap_gib=None):
+    """Configuration 5: the 24-layer decode stack. Caches are allocated layer by layer, K then V, as
+    gpt-oss/src/gpu.rs:567-578 does; kv_gap_gib = N allocates all K caches, N GiB left unused, then all
+    V caches (an experiment on how placement in HBM changes the rate)."""
     log("allocating %.1f GiB of KV cache" % (layers * 2 * batch_size * ctx * ROW / 2**30))
     q = gpu.buffer(layers * batch_size * QO)
     out = gpu.buffer(layers * batch_size * QO)
     sinks = gpu.upload(np.random.default_rng(5).standard_normal((layers, H)).astype(np.float32))
     fill(gpu, q, 1000)
-    caches = []
-    for l in range(layers):
-        k, v = gpu.buffer(batch_size * ctx * ROW), gpu.buffer(batch_size * ctx * ROW)
-        fill(gpu, k, 2 * l + 1)
-        fill(gpu, v, 2 * l + 2)
-        caches += [k, v]
+    caches, unused = [], []
+    if kv_gap_gib is None:
+        for l in range(layers):
+            caches += [gpu.buffer(batch_size * ctx * ROW), gpu.buffer(batch_size * ctx * ROW)]
+    else:
+        ks = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
+        if kv_gap_gib:
+            unused.append(gpu.buffer(kv_gap_gib << 30))
+        vs = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
+        for l in range(layers):
+            caches += [ks[l], vs[l]]
+    for i, b in enumerate(caches):
+        fill(gpu, b, i + 1)
     bufs = [q, out, sinks] + caches
     tables = []
     step_bytes = 0
@@ -113,7 +122,7 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24):
         _, (ks, kn) = step(True)
         kern_s += ks
         launches += kn
-    for b in bufs:
+    for b in bufs + unused:
         b.free()
     per_launch_bytes = step_bytes * steps / launches
     per_launch_s = kern_s / launches
@@ -444,6 +453,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--ctx", type=int, default=131072, help="context of the decode stack")
     ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
+                    "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8: run just these and print their results "
                     "(a development aid; no headline line)")
@@ -473,7 +484,7 @@ def main():
         log("prep", extra["pre_attention_step"])
         extra["q8_0_projection"] = run_q8(gpu, args.steps, args.warmup)
         log("q8", extra["q8_0_projection"])
-    r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx)
+    r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)
     log("c5", r)
     gpu.close()
     cpu = None if args.no_cpu else cpu_baseline(0, args.ctx)
