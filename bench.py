@@ -166,9 +166,9 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
         batch.drop()
         return done.gpu_time, wall
 
-    for _ in range(warmup):
+    for _ in range(max(warmup, 5)):
         go(1)
-    one = sorted(go(1) for _ in range(max(steps, 5)))
+    one = sorted(go(1) for _ in range(max(steps, 20)))
     many = sorted(go(burst) for _ in range(max(steps, 5)))
     for b in bufs:
         b.free()
@@ -216,9 +216,9 @@ def run_ragged(gpu, steps, warmup, n_seq=32):
         batch.drop()
         return done.gpu_time, wall
 
-    for _ in range(warmup):
+    for _ in range(max(warmup, 5)):
         go()
-    runs = sorted(go() for _ in range(max(steps, 5)))
+    runs = sorted(go() for _ in range(max(steps, 20)))
     for b in bufs:
         b.free()
     g, w = runs[len(runs) // 2]
@@ -254,9 +254,9 @@ def run_prefill(gpu, steps, warmup, t=8192):
             batch.drop()
             return done.gpu_time / n
 
-        for _ in range(warmup):
+        for _ in range(max(warmup, 5)):
             go()
-        runs = sorted(go() for _ in range(max(steps, 5)))
+        runs = sorted(go() for _ in range(max(steps, 20)))
         g = runs[len(runs) // 2]
         sustained = go(20)  # 20 launches back to back: no gap before each kernel, steady clocks
         traffic = 2 * t * QO + 2 * t * ROW
@@ -347,6 +347,99 @@ def run_q8(gpu, steps, warmup):
     scales.free()
     out["workload"] = "Q8_0 product, 4096 x 2880 (gpt-oss-20b query projection), f32 positions"
     return out
+
+
+def run_config1(gpu, steps, warmup):
+    """Configuration 1 (the reference's own CPU-runnable case): f32, 4 query heads over 1 kv head of 64,
+    32 positions, full causal, through the plain operator (the general kernel)."""
+    t, heads, kv = 32, 4, 1
+    rng = np.random.default_rng(0)
+    q = rng.standard_normal((t, heads, D)).astype(np.float32)
+    k = rng.standard_normal((t, kv, D)).astype(np.float32)
+    v = rng.standard_normal((t, kv, D)).astype(np.float32)
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.buffer(q.nbytes), gpu.upload(sinks)]
+    shape = C.GroupedShape(t, 0, heads, kv, D, C.FULL, t, SCALE)
+
+    def go():
+        batch = gpu.batch(bufs)
+        batch.attention_grouped_with_sinks((C.Slice(0, 0, q.nbytes), C.Slice(1, 0, k.nbytes), C.Slice(2, 0, v.nbytes)),
+                                           C.Slice(4, 0, heads * 4), C.Slice(3, 0, q.nbytes), shape, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(warmup):
+        go()
+    runs = sorted(go() for _ in range(max(steps, 20)))
+    for b in bufs:
+        b.free()
+    return {"workload": "C1 fp32: 4 q heads / 1 kv head of 64, 32 positions, full causal", "gpu_us": runs[len(runs) // 2] * 1e6}
+
+
+def cpu_extras():
+    """The oracle (f32 port of gpt-oss/src/model.rs:434-464) timed on the host for configurations 1-4, on
+    all cores (OpenMP over query rows and heads) and on one thread. Configuration 4 is timed on 64
+    query rows spread over the pass and scaled by the ratio of query-key pairs (stated as extrapolated)."""
+    from oracle import oracle
+    cores = min(16, os.cpu_count() or 1)
+    rng = np.random.default_rng(21)
+
+    def timed(fn):
+        out = {}
+        for label, threads in (("all", cores), ("one", 1)):
+            t0 = time.perf_counter()
+            fn(threads)
+            out[label] = time.perf_counter() - t0
+        return out
+
+    res = {}
+    # C1
+    q = rng.standard_normal((32, 4, D)).astype(np.float32)
+    k = rng.standard_normal((32, 1, D)).astype(np.float32)
+    v = rng.standard_normal((32, 1, D)).astype(np.float32)
+    s4 = rng.standard_normal(4).astype(np.float32)
+    t1 = timed(lambda th: oracle.attention_f32(q, k, v, s4, 0, scale=SCALE, threads=th))
+    res["c1"] = {"us": t1["all"] * 1e6, "us_1thread": t1["one"] * 1e6, "cores": cores, "kind": "port", "sample": "whole case"}
+    # C2
+    sinks = rng.standard_normal(H).astype(np.float32)
+    q = bf16_widen(bf16_bits(rng.standard_normal((1, H, D), dtype=np.float32) * 0.5))
+    k = bf16_widen(bf16_bits(rng.standard_normal((8192, G, D), dtype=np.float32) * 0.5))
+    v = bf16_widen(bf16_bits(rng.standard_normal((8192, G, D), dtype=np.float32) * 0.5))
+    t2 = timed(lambda th: oracle.attention_f32(q, k[:4096], v[:4096], sinks, 4095, scale=SCALE, threads=th))
+    nb = decode_bytes(4096, C.FULL)
+    res["c2"] = {"us": t2["all"] * 1e6, "gbs": nb / t2["all"] / 1e9, "us_1thread": t2["one"] * 1e6,
+                 "gbs_1thread": nb / t2["one"] / 1e9, "cores": cores, "kind": "port", "sample": "whole case"}
+    # C3: the same lengths as the GPU leg; every sequence reads a prefix of one 8192-position cache
+    lens = np.random.default_rng(3).integers(128, 8193, size=32)
+    nb = sum(decode_bytes(int(n), C.FULL) + decode_bytes(int(n), 128) for n in lens)
+
+    def c3(th):
+        for n in lens:
+            n = int(n)
+            oracle.attention_f32(q, k[:n], v[:n], sinks, n - 1, scale=SCALE, threads=th)
+            oracle.attention_f32(q, k[:n], v[:n], sinks, n - 1, window=128, scale=SCALE, threads=th)
+    t3 = timed(c3)
+    res["c3"] = {"ms": t3["all"] * 1e3, "gbs": nb / t3["all"] / 1e9, "tokens_per_s": 32 / t3["all"],
+                 "ms_1thread": t3["one"] * 1e3, "gbs_1thread": nb / t3["one"] / 1e9, "cores": cores, "kind": "port",
+                 "sample": "whole case (32 sequences x 2 layers)"}
+    # C4: 64 sampled query rows of the 8192-position pass
+    t = 8192
+    pos = np.linspace(63, t - 1, 64).astype(np.uint64)
+    qs = bf16_widen(bf16_bits(rng.standard_normal((64, H, D), dtype=np.float32) * 0.5))
+    res["c4"] = {}
+    for name, window in (("full", C.FULL), ("window128", 128)):
+        w = t if window == C.FULL else window
+        pairs = w * (w + 1) // 2 + (t - w) * w
+        sampled = int(sum(min(int(p) + 1, w) for p in pos))
+        t4 = timed(lambda th: oracle.attention_rows_f32(qs, k, v, sinks, pos, window=window, scale=SCALE, threads=th))
+        flops = 4 * D * H * pairs
+        scale_up = pairs / sampled
+        res["c4"][name] = {"extrapolated_s": t4["all"] * scale_up, "tflops": flops / (t4["all"] * scale_up) / 1e12,
+                           "extrapolated_s_1thread": t4["one"] * scale_up,
+                           "tflops_1thread": flops / (t4["one"] * scale_up) / 1e12, "cores": cores, "kind": "port",
+                           "sample": "64 of 8192 query rows, evenly spaced; time scaled by %.1f (ratio of query-key pairs)" % scale_up}
+    return res
 
 
 def run_copy(gpu, steps, warmup, nbytes=1 << 30):
@@ -484,10 +577,18 @@ def main():
         log("prep", extra["pre_attention_step"])
         extra["q8_0_projection"] = run_q8(gpu, args.steps, args.warmup)
         log("q8", extra["q8_0_projection"])
+        extra["c1_fp32"] = run_config1(gpu, args.steps, args.warmup)
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)
     log("c5", r)
     gpu.close()
     cpu = None if args.no_cpu else cpu_baseline(0, args.ctx)
+    if not args.no_cpu and not args.no_extras:
+        host = cpu_extras()
+        extra["c1_fp32"]["cpu_baseline"] = host["c1"]
+        extra["c2_single_decode"]["cpu_baseline"] = host["c2"]
+        extra["c3_ragged_batch"]["cpu_baseline"] = host["c3"]
+        for name in ("full", "window128"):
+            extra["c4_prefill"][name]["cpu_baseline"] = host["c4"][name]
     extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "step_bytes", "kernel_launches_per_step")}
     line = {
         "metric": METRIC, "value": r["value_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
