@@ -1133,13 +1133,6 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             }
             qreg[h][ks] = as_bf16x8(raw);
         }
-        m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
-        l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
-#pragma unroll
-        for (int db = 0; db < 2; ++db) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
-        }
     }
     const float sl2 = a.scale * LNG_LOG2E;
     bf16x2 ones2;
@@ -1163,11 +1156,6 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         *(uint4 *)(&s_v[buf][ld_key * PF_VSTRIDE + ld_chunk * 8u]) = vr;
     };
 
-    uint4 kr, vr;
-    fetch(0, kr, vr);
-    stash(0, kr, vr);
-    __syncthreads();
-
     // per-lane constant parts of the LDS addresses
     const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
     const uint32_t L = lane & 15u;
@@ -1175,10 +1163,36 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
     const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
 
+    // With two heads per wavefront (long causal runs) the pass is first made optimistically: once a
+    // first interior tile has set the running maximum from real scores, the remaining interior
+    // tiles keep it FIXED and compute neither maxima nor rescalings (a softmax does not depend on
+    // its reference point, only the number range does). Before the diagonal tile the workgroup
+    // checks that every normaliser stayed in a range that rules out overflow and any underflow
+    // that could matter, and that every accumulator is finite; if not, the pass is made again
+    // with the maximum tracked throughout.
+    constexpr int ATTEMPTS = NH == 2 ? 2 : 1;
+    uint4 kr, vr;
+    for (int attempt = 0; attempt < ATTEMPTS; ++attempt) {
+    const bool optimistic = NH == 2 && attempt == 0;
+#pragma unroll
+    for (int h = 0; h < NH; ++h) {
+        m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+        l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
+        }
+    }
+    fetch(0, kr, vr);
+    stash(0, kr, vr);
+    __syncthreads();
+
     // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
     // carries no position arithmetic at all.
-    auto step = [&](auto mask_tag, uint32_t tile) {
+    auto step = [&](auto mask_tag, auto fixed_tag, uint32_t tile) {
         constexpr bool MASK = decltype(mask_tag)::value;
+        constexpr bool FIXED = decltype(fixed_tag)::value;
         const uint32_t buf = tile & 1u;
         if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
         if (wave_active) {
@@ -1229,21 +1243,26 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                             st[h][i] = vis ? st[h][i] : LNG_NEG_INF;
                         }
                     }
-                    float tmax = LNG_NEG_INF;
+                    float m_safe;
+                    if constexpr (FIXED) {
+                        m_safe = m[h]; // not -inf once frozen
+                    } else {
+                        float tmax = LNG_NEG_INF;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
-                    tmax = other_half_max(tmax) * sl2; // scale > 0: max commutes with it
-                    const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
-                    const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
-                    if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
-                        const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
-                        l[h] *= alpha;
+                        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
+                        tmax = other_half_max(tmax) * sl2; // scale > 0: max commutes with it
+                        const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
+                        m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                        if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
+                            const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+                            l[h] *= alpha;
 #pragma unroll
-                        for (int db = 0; db < 2; ++db) {
+                            for (int db = 0; db < 2; ++db) {
 #pragma unroll
-                            for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
+                                for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
+                            }
+                            m[h] = m_new;
                         }
-                        m[h] = m_new;
                     }
                     float psum = 0.0f;
 #pragma unroll
@@ -1283,9 +1302,47 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         return kt0 + (PF_BN - 1) > pos_first || (windowed && kt0 + window < pos_first + PF_BM);
     };
     uint32_t tile = 0;
-    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tile);   // window edge
-    for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tile); // interior
-    for (; tile < n_tiles; ++tile) step(std::true_type{}, tile);                 // diagonal
+    bool frozen = false;
+    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, std::false_type{}, tile); // window edge
+    if (optimistic) {                                                                             // interior
+        if (tile < n_tiles && !edge(tile)) {
+            step(std::false_type{}, std::false_type{}, tile); // sets the maximum from real scores
+            ++tile;
+            frozen = true;
+#pragma unroll
+            for (int h = 0; h < NH; ++h) m[h] = m[h] == LNG_NEG_INF ? 0.0f : m[h];
+        }
+        // a loop of its own: one path through it, so its registers need no reconciling copies
+        for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, std::true_type{}, tile);
+    } else {
+        for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, std::false_type{}, tile);
+    }
+    bool again = false;
+    if (NH == 2 && frozen) { // frozen is uniform over the workgroup
+        int bad = 0;
+        if (wave_active) {
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                const float total = l[h] + __shfl_xor(l[h], 32, 64);
+                uint32_t top = 0;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) top = max(top, __float_as_uint(ot[h][db][i]) & 0x7fffffffu);
+                }
+                // 2^-80 .. 2^60: terms lost below 2^-126 are then under 2^-29 of the total even for 2^17
+                // keys, and nothing overflowed (a NaN fails the comparison)
+                bad |= !(total >= 8.271806e-25f && total <= 1.1529215e18f) || top >= 0x7f800000u;
+            }
+            bad = row_ok ? bad : 0;
+        }
+        again = __syncthreads_or(bad) != 0;
+    }
+    if (!again) {
+        for (; tile < n_tiles; ++tile) step(std::true_type{}, std::false_type{}, tile);           // diagonal
+        break;
+    }
+    }
 
 
     // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------

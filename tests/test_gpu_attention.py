@@ -310,6 +310,29 @@ def test_prefill_bf16_matches_the_cpu_reference(gpu, t, start, window, slots, he
     assert max_error(from_bf16_bits(plain), from_bf16_bits(want)) < BF16_TOL
 
 
+@pytest.mark.parametrize("spike_at,sinks_on", [(300, True), (300, False), (5, True), (5, False), (700, True)])
+def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on):
+    """Long causal passes first keep the running maximum fixed after one interior tile and check the
+    normalisers afterwards. A key whose score is about 10,000 above the rest (2^10000 cannot be held)
+    late in the pass must send the workgroup through the pass that tracks the maximum; the same key
+    early in the pass, or a cache whose scores all sit far below the first tile's, must not lose anything."""
+    t, heads, kv_heads = 1024, 16, 2
+    q, k, v, sinks = normal_inputs(91 + spike_at, t, t, heads, kv_heads, 64, scale=0.5)
+    q[:] = np.abs(q) + 1.0                      # every query has a large positive overlap with the spike key
+    k[spike_at] = 30.0                          # score = 0.125 * 30 * sum(q) ~ 0.125 * 30 * 64 * 1.4
+    if spike_at == 700:                         # and everything before it far below the first tile's scores
+        k[64:700] = -k[64:700] - 8.0
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    shape = C.GroupedShape(t, 0, heads, kv_heads, 64, FULL, t, 0.125)
+    sk = sinks if sinks_on else None
+    want = oracle.attention_bf16(qb, kb, vb, sk, 0, scale=0.125, threads=THREADS)
+    got = run_attention(gpu, qb, kb, vb, sk, shape, True, C.BF16)
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+    # rows after the spike attend to it alone: their output is its value row
+    late = from_bf16_bits(got)[spike_at + 1:]
+    assert np.abs(late - from_bf16_bits(vb)[spike_at][None, :, None, :].repeat(heads // kv_heads, 2).reshape(1, heads, 64)).max() < BF16_TOL
+
+
 @pytest.mark.parametrize("window", [FULL, 128])
 def test_config4_prefill_8192_sampled_rows(gpu, window):
     """The 8192-position prompt pass at its real size; a sample of query rows (first, last,
