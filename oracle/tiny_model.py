@@ -246,9 +246,10 @@ class TinyModel:
             out += weight * y
         return out
 
-    def forward(self, ids, prepare, attention, chunk=1, project=None, block=None):
+    def forward(self, ids, prepare, attention, chunk=1, project=None, block=None, first=0):
         """Logits [len(ids)][vocab]. Positions are fed `chunk` at a time (1 = `Model::step`,
-        model.rs:408-478; more = a prompt pass, gpu.rs:703-827).
+        model.rs:408-478; more = a prompt pass, gpu.rs:703-827). ids[0] sits at position `first`
+        (a session that was truncated to `first` positions, model.rs:203-213, and is fed again).
 
         prepare(l, q, k, v, start) -> None: q [n][heads*dim], k, v [n][kv_heads*dim] are the raw
             projections of layer l for positions start..start+n; it must add the biases, rotate
@@ -269,8 +270,9 @@ class TinyModel:
             return _mul(self.layers[l][{"output": "o"}.get(part, part)], x)
 
         logits = np.zeros((len(ids), self.vocab), dtype=np.float32)
-        for start in range(0, len(ids), chunk):
-            tokens = ids[start:start + chunk]
+        for at in range(0, len(ids), chunk):
+            tokens = ids[at:at + chunk]
+            start = first + at
             n = len(tokens)
             h = self.embedding[tokens].copy()
             for l, layer in enumerate(self.layers):
@@ -284,7 +286,7 @@ class TinyModel:
                     h = h + (mul(l, "output", attended) + layer["o_bias"])
                 x = rms_norm(h, layer["ffn_norm"], self.eps)
                 h = h + np.stack([self.experts_out(layer, x[i]) for i in range(n)])
-            logits[start:start + n] = _mul(self.output, rms_norm(h, self.output_norm, self.eps))
+            logits[at:at + n] = _mul(self.output, rms_norm(h, self.output_norm, self.eps))
         return logits
 
 

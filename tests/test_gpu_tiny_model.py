@@ -257,3 +257,20 @@ def test_whole_attention_blocks_on_the_device_match_transformers(gpu, model, chu
         s.close()
     worst = np.abs(got - want).max(axis=1)
     assert worst.max() < TOLERANCE, f"position {worst.argmax()}: max error {worst.max()}"
+
+
+@pytest.mark.parametrize("chunk,back", [(5, 5), (5, 3), (8, 8)])
+def test_truncating_a_session_and_feeding_it_again_gives_the_same_logits(gpu, model, chunk, back):
+    """`Session::truncate` (model.rs:203-213; gpu.rs:403-409: at most one chunk back, which the rings of
+    window + chunk rows still hold): after 40 positions the session goes back `back` positions and the
+    same tokens are fed again over the same device caches."""
+    ids, want = tm.load_fixture(FIXTURE)
+    s = DeviceSession(gpu, model, chunk, C.F32, False)
+    try:
+        got = model.forward(ids, s.prepare, s.attention, chunk=chunk)
+        again = model.forward(ids[40 - back:], s.prepare, s.attention, chunk=chunk, first=40 - back)
+    finally:
+        s.close()
+    assert np.abs(got - want).max() < TOLERANCE
+    assert np.abs(again - want[40 - back:]).max() < TOLERANCE
+    assert np.abs(again - got[40 - back:]).max() < 1e-5
