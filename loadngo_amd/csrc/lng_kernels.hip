@@ -1051,7 +1051,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill 
 #define PF_BN 64
 #define PF_THREADS 512
 #define PF_KSTRIDE 72 // bf16 elements per LDS row (144 bytes): conflict-free 16-byte row reads
-#define PF_VSTRIDE 72
+#define PF_VSTRIDE 96 // 192-byte rows: the four keys x 64 bytes that half a wavefront reads transposed fall in 64 different banks
 
 #define PF_TAU 8.0f
 typedef short short4v __attribute__((ext_vector_type(4)));
