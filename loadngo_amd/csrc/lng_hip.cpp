@@ -1328,8 +1328,16 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
         a.x_lo = sp.lo;
         c1.fn = b->gpu->q8_tiled;
         c1.name = "lng_q8_tiled";
-        c1.grid[0] = (unsigned)((rows + 255) / 256);
-        c1.grid[1] = (unsigned)(n_pad / 128);
+        // one-dimensional grid; the kernel maps ids to tiles (XCD-aware from eight position tiles on,
+        // rounded up to blocks of 8 row tiles x 4 position tiles per XCD)
+        const uint64_t row_tiles = (rows + 255) / 256, pos_tiles = n_pad / 128;
+        uint64_t ids = row_tiles * pos_tiles;
+        if (pos_tiles >= 8) {
+            const uint64_t per_xcd = (pos_tiles + 7) / 8;
+            ids = 8 * ((per_xcd + 3) / 4) * ((row_tiles + 7) / 8) * 32;
+        }
+        if (ids > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
+        c1.grid[0] = (unsigned)ids;
         c1.block = 512;
     }
     set_args(c1, a);

@@ -829,17 +829,21 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 }
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128
-// positions, wavefront (w % 4, w / 4) the 64 x 64 corner of it: four 16-row B operands made from
-// the codes, four 16-position A operands per plane of x. Codes, planes and block scales are
-// staged in LDS 64 columns (two blocks) at a time, double buffered: the loads of stage s + 1 are
-// issued before stage s is computed and stored to LDS after it, so every byte of the matrix is
-// fetched once per workgroup, in 64-byte runs. Rows of the tiles are unpadded; the 16-byte chunk
-// c of position p is kept at chunk c ^ ((p >> 1) & 7) and chunk c of matrix row r at
-// c ^ ((r >> 2) & 3), which makes the 16 rows that one operand read touches fall in different
-// banks. (Loads that go from global memory straight into LDS were tried for the staging: the
-// compiler then waits for every outstanding one before the first LDS read of a stage, which
-// undoes the overlap.) Every (rows, positions) pair of operands gives one block sum per
-// lane-held output; the row's block scale multiplies it into the f32 result.
+// positions, wavefront (w % 4, w / 4) the 64 x 64 corner of it: four 16-row B operands of codes
+// (as bf16, in which every code is exact), four 16-position A operands per plane of x. Codes,
+// planes and block scales are staged in LDS 64 columns (two blocks) at a time, double buffered:
+// the loads of stage s + 1 are issued before stage s is computed and stored to LDS after it, so
+// every byte of the matrix is fetched once per workgroup, in 64-byte runs. The thread that
+// fetched 16 codes widens them to bf16 on the way into LDS, once per workgroup, rather than
+// every wavefront that uses them doing so in its inner loop. Rows of both tiles are 128 bytes,
+// unpadded; the 16-byte chunk c of row r is kept at chunk c ^ ((r >> 1) & 7), which makes the
+// 16 rows that one operand read touches fall in different banks; rows of codes add r & 1 to
+// that, so that the eight lanes that store two rows' even (or odd) chunks together, 128 bytes a
+// cycle, also hit eight different places. (Loads that go from global
+// memory straight into LDS were tried for the staging: the compiler then waits for every
+// outstanding one before the first LDS read of a stage, which undoes the overlap.) Every
+// (rows, positions) pair of operands gives one block sum per lane-held output; the row's block
+// scale multiplies it into the f32 result.
 #define Q8T_THREADS 512
 #define Q8T_POS 128
 #define Q8T_ROWS 256
@@ -857,16 +861,38 @@ __device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
 }
 
 extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 a) {
-    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_PLANE]; // [stage % 2][plane]
-    __shared__ __attribute__((aligned(16))) uint8_t s_w[2][Q8T_ROWS * 64];  // [stage % 2]: 64 code bytes per row
-    __shared__ uint16_t s_sc[2][Q8T_ROWS * 2];                              // [stage % 2]: two block scales per row
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_PLANE];   // [stage % 2][plane]
+    __shared__ __attribute__((aligned(16))) uint16_t s_w[2][Q8T_ROWS * 64];  // [stage % 2]: 64 codes per row as bf16
+    __shared__ uint16_t s_sc[2][Q8T_ROWS * 2];                               // [stage % 2]: two block scales per row
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
     const uint32_t rw = 64u * (wave & 3u); // this wavefront's rows within the tile
     const uint32_t pw = 64u * (wave >> 2); // and its positions
-    const uint32_t r0 = blockIdx.x * Q8T_ROWS;
-    const uint32_t p0 = blockIdx.y * Q8T_POS;
+    // Which tile: workgroup ids go round the eight XCDs, each with an L2 of its own, and a few dozen
+    // consecutive ids of one XCD run at a time. With eight position tiles or more, XCD k takes the
+    // position tiles k, k + 8, ..; its ids walk blocks of 8 row tiles x 4 position tiles, so what
+    // runs together reads 4 tiles of x and 8 of the matrix, every x tile is read through one L2
+    // only, and the fetches from beyond L2 are about half of what row-major ids cost. The grid is
+    // rounded up to whole blocks; a workgroup whose tile does not exist leaves at once.
+    const uint32_t row_tiles = (a.rows + Q8T_ROWS - 1u) / Q8T_ROWS;
+    const uint32_t pos_tiles = (a.n + Q8T_POS - 1u) / Q8T_POS;
+    uint32_t row_tile, pos_tile;
+    if (pos_tiles >= 8u) {
+        const uint32_t xcd = blockIdx.x & 7u, seq = blockIdx.x >> 3;
+        const uint32_t per_xcd = (pos_tiles + 7u) / 8u;
+        const uint32_t row_blocks = (row_tiles + 7u) / 8u;
+        const uint32_t blk = seq >> 5, within = seq & 31u;
+        row_tile = (blk % row_blocks) * 8u + (within & 7u);
+        const uint32_t pi = (blk / row_blocks) * 4u + (within >> 3);
+        pos_tile = pi * 8u + xcd;
+        if (row_tile >= row_tiles || pi >= per_xcd || pos_tile >= pos_tiles) return;
+    } else {
+        row_tile = blockIdx.x % row_tiles;
+        pos_tile = blockIdx.x / row_tiles;
+    }
+    const uint32_t r0 = row_tile * Q8T_ROWS;
+    const uint32_t p0 = pos_tile * Q8T_POS;
     const uint32_t blocks = a.cols / 32u;
     const uint32_t stages = (blocks + 1u) / 2u;
     const bool rows_here = r0 + rw < a.rows; // wavefronts past the last row only help staging
@@ -884,15 +910,17 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         x_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
     }
     // code staging: two loads per stage; load q covers the 16 rows of group 2w + q; lane l brings row
-    // 16 * group + l / 4, physical chunk l % 4.
+    // 16 * group + l / 4 and its codes 16 * (l % 4) .. + 15, which become the row's bf16 chunks
+    // 2 * (l % 4) and 2 * (l % 4) + 1.
     const int8_t *w_src[2];
-    uint32_t w_chunk[2];
+    uint32_t w_to[2][2]; // element index in s_w[buf] of the two chunks
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         const uint32_t row = 16u * (2u * wave + q) + (lane >> 2);
-        w_chunk[q] = (lane & 3u) ^ ((row >> 2) & 3u);
         const uint32_t r = r0 + row < a.rows ? r0 + row : a.rows - 1u;
         w_src[q] = a.codes + (uint64_t)r * a.cols;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) w_to[q][h] = row * 64u + 8u * ((2u * (lane & 3u) + h) ^ ((row >> 1) & 7u) ^ (row & 1u));
     }
     // scale staging: thread t brings the scale of row t / 2, block t % 2 of the stage
     const uint32_t sc_row = r0 + (tid >> 1) < a.rows ? r0 + (tid >> 1) : a.rows - 1u;
@@ -901,8 +929,8 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         const uint32_t col = stage * 64u + 8u * x_chunk[q];
         return col < a.cols ? col : col - 32u; // odd block count: the last stage's second block repeats its first
     };
-    auto w_col = [&](uint32_t stage, int q) {
-        const uint32_t col = stage * 64u + 16u * w_chunk[q];
+    auto w_col = [&](uint32_t stage) { // the same, for this lane's 16 codes (col >= cols >= 32 where it applies)
+        const uint32_t col = stage * 64u + 16u * (lane & 3u);
         return col < a.cols ? col : col - 32u;
     };
     // staged values live in plain scalars so that they stay in registers
@@ -913,8 +941,9 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         sx1 = *(const uint4 *)(x_src[1] + x_col(stage, 1));
         sx2 = *(const uint4 *)(x_src[2] + x_col(stage, 2));
         sx3 = *(const uint4 *)(x_src[3] + x_col(stage, 3));
-        sw0 = *(const uint4 *)(w_src[0] + w_col(stage, 0));
-        sw1 = *(const uint4 *)(w_src[1] + w_col(stage, 1));
+        const uint32_t wc = w_col(stage);
+        sw0 = *(const uint4 *)(w_src[0] + wc);
+        sw1 = *(const uint4 *)(w_src[1] + wc);
         const uint32_t b = 2u * stage + (tid & 1u);
         ssc = b < blocks ? sc_src[b] : (uint16_t)0; // a block past the end counts for nothing
     };
@@ -922,13 +951,19 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         const uint32_t idx = 4u * wave + q;
         return (uint4 *)(&s_x[buf][idx >> 4][(idx & 15u) * 512u + 8u * lane]);
     };
+    auto widen = [&](uint32_t buf, int q, const uint4 &codes) {
+        const bf16x8 lo = q8_codes_to_bf16_perm(make_uint2(codes.x, codes.y));
+        const bf16x8 hi = q8_codes_to_bf16_perm(make_uint2(codes.z, codes.w));
+        *(bf16x8 *)(&s_w[buf][w_to[q][0]]) = lo;
+        *(bf16x8 *)(&s_w[buf][w_to[q][1]]) = hi;
+    };
     auto stash = [&](uint32_t buf) {
         *x_slot(buf, 0) = sx0;
         *x_slot(buf, 1) = sx1;
         *x_slot(buf, 2) = sx2;
         *x_slot(buf, 3) = sx3;
-        *(uint4 *)(&s_w[buf][(2u * wave) * 1024u + 16u * lane]) = sw0;
-        *(uint4 *)(&s_w[buf][(2u * wave + 1u) * 1024u + 16u * lane]) = sw1;
+        widen(buf, 0, sw0);
+        widen(buf, 1, sw1);
         s_sc[buf][tid] = ssc;
     };
 
@@ -939,16 +974,16 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         for (int mt = 0; mt < 4; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    // per-lane parts of the operand reads
+    // per-lane parts of the operand reads: row (position or matrix row) t * 16 + j, logical chunk 4 kb + kg
     uint32_t x_at[4], x_sw[4], w_at[4], w_sw[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-        const uint32_t pos = pw + 16u * t + j; // position, logical chunk 4 kb + kg
+        const uint32_t pos = pw + 16u * t + j;
         x_at[t] = pos * 64u;
         x_sw[t] = (pos >> 1) & 7u;
-        const uint32_t row = rw + 16u * t + j; // matrix row, logical chunk 2 kb + kg / 2, half kg % 2
-        w_at[t] = row * 64u + 8u * (kg & 1u);
-        w_sw[t] = (row >> 2) & 3u;
+        const uint32_t row = rw + 16u * t + j;
+        w_at[t] = row * 64u;
+        w_sw[t] = ((row >> 1) & 7u) ^ (row & 1u);
     }
     auto compute = [&](uint32_t buf) {
 #pragma unroll
@@ -962,8 +997,7 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
             }
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
-                const uint2 raw = *(const uint2 *)(&s_w[buf][w_at[nt] + 16u * ((2u * kb + (kg >> 1)) ^ w_sw[nt])]);
-                const bf16x8 wb = q8_codes_to_bf16_perm(raw);
+                const bf16x8 wb = as_bf16x8(*(const uint4 *)(&s_w[buf][w_at[nt] + 8u * ((4u * kb + kg) ^ w_sw[nt])]));
                 const float scale = f16_bits_to_f32(s_sc[buf][2u * (rw + 16u * nt + j) + kb]);
                 floatx4 acc[4];
 #pragma unroll
