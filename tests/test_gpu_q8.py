@@ -61,6 +61,21 @@ def test_products_match_the_float64_definition(gpu, rows, cols, n, kind):
     assert np.abs(got - cpu).max() / np.abs(want).max() < 2e-5
 
 
+@pytest.mark.parametrize("rows,cols,n,kind", [(320, 96, 1120, "tiled"), (2112, 64, 1056, "tiled"), (576, 160, 4224, "tiled"),
+                                              (256, 32, 1024, "tiled"), (300, 96, 1100, "gemm"), (2100, 64, 1030, "gemm")])
+def test_product_with_eight_position_tiles_or_more(gpu, rows, cols, n, kind):
+    """From eight tiles of 128 positions on, workgroup ids are mapped to tiles per XCD in blocks of 8 row
+    tiles x 4 position tiles and the grid is rounded up to whole blocks: every tile must be computed exactly
+    once (ragged tile counts in both directions, ids without a tile), nothing outside y written."""
+    codes, bits, elements = q8_test_matrix(rows, cols, 40 + rows)
+    x = xorshift_values(13, n * cols).reshape(n, cols)
+    want = x.astype(np.float64) @ elements.T
+    got = q8_run(gpu, codes, bits, x, rows, cols, kind, y_stride=rows + 4)
+    assert not np.isnan(got[:, :rows]).any()
+    assert np.abs(got[:, :rows] - want).max() / np.abs(want).max() < 1e-5
+    assert np.isnan(got[:-1, rows:]).all()           # 0xFF fill: gaps of y untouched
+
+
 def test_strided_positions_and_untouched_gaps(gpu):
     rows, cols, n = 80, 96, 21
     codes, bits, elements = q8_test_matrix(rows, cols, 3)
