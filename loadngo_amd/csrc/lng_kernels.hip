@@ -844,7 +844,6 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 // outstanding one before the first LDS read of a stage, which undoes the overlap.) Every
 // (rows, positions) pair of operands gives one block sum per lane-held output; the row's block
 // scale multiplies it into the f32 result.
-#define Q8T_THREADS 512
 #define Q8T_POS 128
 #define Q8T_ROWS 256
 #define Q8T_PLANE (Q8T_POS * 64) // bf16 elements of one plane of one stage
@@ -860,7 +859,12 @@ __device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
     return as_bf16x8(make_uint4(w[0], w[1], w[2], w[3]));
 }
 
-extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 a) {
+// WAVES wavefronts per workgroup: 8 (64 x 64 outputs each, two per SIMD) is what is launched; 16 (64 rows x
+// 32 positions each, four per SIMD with half the registers) measures the same and is not instantiated.
+template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q8 &a) {
+    constexpr int MT = WAVES == 8 ? 4 : 2;       // groups of 16 positions per wavefront
+    constexpr int XQ = 32 / WAVES;               // x loads per wavefront and stage (32 in all: 2 planes x 16 groups of 8 positions)
+    constexpr int WQ = 16 / WAVES;               // code loads (16 in all: groups of 16 rows)
     __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_PLANE];   // [stage % 2][plane]
     __shared__ __attribute__((aligned(16))) uint16_t s_w[2][Q8T_ROWS * 64];  // [stage % 2]: 64 codes per row as bf16
     __shared__ uint16_t s_sc[2][Q8T_ROWS * 2];                               // [stage % 2]: two block scales per row
@@ -868,7 +872,7 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
     const uint32_t rw = 64u * (wave & 3u); // this wavefront's rows within the tile
-    const uint32_t pw = 64u * (wave >> 2); // and its positions
+    const uint32_t pw = 16u * MT * (wave >> 2); // and its positions
     // Which tile: workgroup ids go round the eight XCDs, each with an L2 of its own, and a few dozen
     // consecutive ids of one XCD run at a time. With eight position tiles or more, XCD k takes the
     // position tiles k, k + 8, ..; its ids walk blocks of 8 row tiles x 4 position tiles, so what
@@ -897,33 +901,35 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
     const uint32_t stages = (blocks + 1u) / 2u;
     const bool rows_here = r0 + rw < a.rows; // wavefronts past the last row only help staging
 
-    // x staging: wavefront w issues four loads per stage; load q covers plane (4w + q) / 16 and the 8
-    // positions of group (4w + q) % 16; lane l brings position 8 * group + l / 8, physical chunk l % 8.
-    const uint16_t *x_src[4];
-    uint32_t x_chunk[4];
+    // x staging: wavefront w issues XQ loads per stage; load q covers plane idx / 16 and the 8 positions
+    // of group idx % 16, idx = XQ * w + q; lane l brings position 8 * group + l / 8, physical chunk l % 8.
+    const uint16_t *x_src[XQ];
+    uint32_t x_chunk[XQ];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t idx = 4u * wave + q;
+    for (int q = 0; q < XQ; ++q) {
+        const uint32_t idx = XQ * wave + q;
         const uint32_t pos = 8u * (idx & 15u) + (lane >> 3);
         x_chunk[q] = (lane & 7u) ^ ((pos >> 1) & 7u); // the logical chunk kept at this physical place
         const uint16_t *plane = (idx >> 4) ? a.x_lo : a.x_hi;
         x_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
     }
-    // code staging: two loads per stage; load q covers the 16 rows of group 2w + q; lane l brings row
+    // code staging: WQ loads per stage; load q covers the 16 rows of group WQ * w + q; lane l brings row
     // 16 * group + l / 4 and its codes 16 * (l % 4) .. + 15, which become the row's bf16 chunks
     // 2 * (l % 4) and 2 * (l % 4) + 1.
-    const int8_t *w_src[2];
-    uint32_t w_to[2][2]; // element index in s_w[buf] of the two chunks
+    const int8_t *w_src[WQ];
+    uint32_t w_to[WQ][2]; // element index in s_w[buf] of the two chunks
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const uint32_t row = 16u * (2u * wave + q) + (lane >> 2);
+    for (int q = 0; q < WQ; ++q) {
+        const uint32_t row = 16u * (WQ * wave + q) + (lane >> 2);
         const uint32_t r = r0 + row < a.rows ? r0 + row : a.rows - 1u;
         w_src[q] = a.codes + (uint64_t)r * a.cols;
 #pragma unroll
         for (int h = 0; h < 2; ++h) w_to[q][h] = row * 64u + 8u * ((2u * (lane & 3u) + h) ^ ((row >> 1) & 7u) ^ (row & 1u));
     }
-    // scale staging: thread t brings the scale of row t / 2, block t % 2 of the stage
-    const uint32_t sc_row = r0 + (tid >> 1) < a.rows ? r0 + (tid >> 1) : a.rows - 1u;
+    // scale staging: thread t < 512 brings the scale of row t / 2, block t % 2 of the stage
+    const bool sc_mine = WAVES == 8 || wave < 8u;
+    const uint32_t sc_t = tid & 511u;
+    const uint32_t sc_row = r0 + (sc_t >> 1) < a.rows ? r0 + (sc_t >> 1) : a.rows - 1u;
     const uint16_t *sc_src = a.scales + (uint64_t)sc_row * blocks;
     auto x_col = [&](uint32_t stage, int q) {
         const uint32_t col = stage * 64u + 8u * x_chunk[q];
@@ -933,54 +939,65 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         const uint32_t col = stage * 64u + 16u * (lane & 3u);
         return col < a.cols ? col : col - 32u;
     };
-    // staged values live in plain scalars so that they stay in registers
-    uint4 sx0, sx1, sx2, sx3, sw0, sw1;
-    uint16_t ssc;
-    auto fetch = [&](uint32_t stage) {
-        sx0 = *(const uint4 *)(x_src[0] + x_col(stage, 0));
-        sx1 = *(const uint4 *)(x_src[1] + x_col(stage, 1));
-        sx2 = *(const uint4 *)(x_src[2] + x_col(stage, 2));
-        sx3 = *(const uint4 *)(x_src[3] + x_col(stage, 3));
+    // Two sets of staging registers: the loads of stage s + 2 are issued when stage s starts and
+    // stored to LDS when stage s + 1 ends, two stages of time for a fetch that misses L2 (with one
+    // stage, nearly every stage had some wavefront waiting out a miss before the barrier).
+    // (plain scalars: arrays of staged values end up in scratch memory)
+    const uint4 zero_u4 = make_uint4(0, 0, 0, 0);
+    uint4 ax0 = zero_u4, ax1 = zero_u4, ax2 = zero_u4, ax3 = zero_u4, aw0 = zero_u4, aw1 = zero_u4;
+    uint4 bx0 = zero_u4, bx1 = zero_u4, bx2 = zero_u4, bx3 = zero_u4, bw0 = zero_u4, bw1 = zero_u4;
+    uint16_t asc = 0, bsc = 0;
+    auto fetch = [&](uint32_t stage, uint4 &x0, uint4 &x1, uint4 &x2, uint4 &x3, uint4 &w0, uint4 &w1, uint16_t &sc) {
+        x0 = *(const uint4 *)(x_src[0] + x_col(stage, 0));
+        x1 = *(const uint4 *)(x_src[1] + x_col(stage, 1));
+        if constexpr (XQ == 4) {
+            x2 = *(const uint4 *)(x_src[2] + x_col(stage, 2));
+            x3 = *(const uint4 *)(x_src[3] + x_col(stage, 3));
+        }
         const uint32_t wc = w_col(stage);
-        sw0 = *(const uint4 *)(w_src[0] + wc);
-        sw1 = *(const uint4 *)(w_src[1] + wc);
+        w0 = *(const uint4 *)(w_src[0] + wc);
+        if constexpr (WQ == 2) w1 = *(const uint4 *)(w_src[1] + wc);
         const uint32_t b = 2u * stage + (tid & 1u);
-        ssc = b < blocks ? sc_src[b] : (uint16_t)0; // a block past the end counts for nothing
+        if (sc_mine) sc = b < blocks ? sc_src[b] : (uint16_t)0; // a block past the end counts for nothing
     };
     auto x_slot = [&](uint32_t buf, uint32_t q) {
-        const uint32_t idx = 4u * wave + q;
+        const uint32_t idx = XQ * wave + q;
         return (uint4 *)(&s_x[buf][idx >> 4][(idx & 15u) * 512u + 8u * lane]);
     };
     auto widen = [&](uint32_t buf, int q, const uint4 &codes) {
-        const bf16x8 lo = q8_codes_to_bf16_perm(make_uint2(codes.x, codes.y));
-        const bf16x8 hi = q8_codes_to_bf16_perm(make_uint2(codes.z, codes.w));
-        *(bf16x8 *)(&s_w[buf][w_to[q][0]]) = lo;
-        *(bf16x8 *)(&s_w[buf][w_to[q][1]]) = hi;
+        *(bf16x8 *)(&s_w[buf][w_to[q][0]]) = q8_codes_to_bf16_perm(make_uint2(codes.x, codes.y));
+        *(bf16x8 *)(&s_w[buf][w_to[q][1]]) = q8_codes_to_bf16_perm(make_uint2(codes.z, codes.w));
     };
-    auto stash = [&](uint32_t buf) {
-        *x_slot(buf, 0) = sx0;
-        *x_slot(buf, 1) = sx1;
-        *x_slot(buf, 2) = sx2;
-        *x_slot(buf, 3) = sx3;
-        widen(buf, 0, sw0);
-        widen(buf, 1, sw1);
-        s_sc[buf][tid] = ssc;
+    auto stash = [&](uint32_t buf, const uint4 &x0, const uint4 &x1, const uint4 &x2, const uint4 &x3, const uint4 &w0,
+                     const uint4 &w1, uint16_t sc) {
+        *x_slot(buf, 0) = x0;
+        *x_slot(buf, 1) = x1;
+        if constexpr (XQ == 4) {
+            *x_slot(buf, 2) = x2;
+            *x_slot(buf, 3) = x3;
+        }
+        widen(buf, 0, w0);
+        if constexpr (WQ == 2) widen(buf, 1, w1);
+        if (sc_mine) s_sc[buf][sc_t] = sc;
     };
 
-    floatx4 y[4][4];
+    floatx4 y[4][MT];
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int mt = 0; mt < MT; ++mt) y[nt][mt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     }
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
     // per-lane parts of the operand reads: row (position or matrix row) t * 16 + j, logical chunk 4 kb + kg
-    uint32_t x_at[4], x_sw[4], w_at[4], w_sw[4];
+    uint32_t x_at[MT], x_sw[MT], w_at[4], w_sw[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
+    for (int t = 0; t < MT; ++t) {
         const uint32_t pos = pw + 16u * t + j;
         x_at[t] = pos * 64u;
         x_sw[t] = (pos >> 1) & 7u;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
         const uint32_t row = rw + 16u * t + j;
         w_at[t] = row * 64u;
         w_sw[t] = ((row >> 1) & 7u) ^ (row & 1u);
@@ -988,9 +1005,9 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
     auto compute = [&](uint32_t buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
-            bf16x8 xh[4], xl[4];
+            bf16x8 xh[MT], xl[MT];
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
+            for (int mt = 0; mt < MT; ++mt) {
                 const uint32_t at = x_at[mt] + 8u * ((4u * kb + kg) ^ x_sw[mt]);
                 xh[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][0][at]));
                 xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][1][at]));
@@ -999,13 +1016,13 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
             for (int nt = 0; nt < 4; ++nt) {
                 const bf16x8 wb = as_bf16x8(*(const uint4 *)(&s_w[buf][w_at[nt] + 8u * ((4u * kb + kg) ^ w_sw[nt])]));
                 const float scale = f16_bits_to_f32(s_sc[buf][2u * (rw + 16u * nt + j) + kb]);
-                floatx4 acc[4];
+                floatx4 acc[MT];
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
+                for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt) {
+                for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) y[nt][mt][i] = __builtin_fmaf(scale, acc[mt][i], y[nt][mt][i]);
                 }
@@ -1013,15 +1030,21 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
         }
     };
 
-    fetch(0);
-    stash(0);
+    fetch(0, ax0, ax1, ax2, ax3, aw0, aw1, asc);
+    stash(0, ax0, ax1, ax2, ax3, aw0, aw1, asc);
     __syncthreads();
-    for (uint32_t stage = 0; stage < stages; ++stage) {
-        const uint32_t buf = stage & 1u;
-        const bool more = stage + 1u < stages;
-        if (more) fetch(stage + 1u);
-        if (rows_here) compute(buf);
-        if (more) stash(buf ^ 1u);
+    if (stages > 1u) fetch(1, bx0, bx1, bx2, bx3, bw0, bw1, bsc);
+    for (uint32_t stage = 0; stage < stages; stage += 2u) {
+        // even stage, in buffer 0: stage + 1 waits in set b, stage + 2 goes to set a
+        if (stage + 2u < stages) fetch(stage + 2u, ax0, ax1, ax2, ax3, aw0, aw1, asc);
+        if (rows_here) compute(0);
+        if (stage + 1u < stages) stash(1, bx0, bx1, bx2, bx3, bw0, bw1, bsc);
+        __syncthreads();
+        if (stage + 1u >= stages) break;
+        // odd stage, in buffer 1: stage + 2 waits in set a, stage + 3 goes to set b
+        if (stage + 3u < stages) fetch(stage + 3u, bx0, bx1, bx2, bx3, bw0, bw1, bsc);
+        if (rows_here) compute(1);
+        if (stage + 2u < stages) stash(0, ax0, ax1, ax2, ax3, aw0, aw1, asc);
         __syncthreads();
     }
     if (!rows_here) return;
@@ -1029,7 +1052,7 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
     for (int nt = 0; nt < 4; ++nt) {
         const uint32_t r = r0 + rw + 16u * nt + j;
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint32_t p = p0 + pw + 16u * mt + 4u * kg + i;
@@ -1037,6 +1060,10 @@ extern "C" __global__ __launch_bounds__(Q8T_THREADS) void lng_q8_tiled(lng_k_q8 
             }
         }
     }
+}
+
+extern "C" __global__ __launch_bounds__(512) void lng_q8_tiled(lng_k_q8 a) {
+    q8_tiled_body<8>(a);
 }
 
 // Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).
