@@ -86,7 +86,7 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
+                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
                   q8_split_x = nullptr, q8_stream = nullptr, q8_tiled = nullptr, rmsnorm_rows = nullptr;
     std::string name;
@@ -505,13 +505,44 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const unsigned rows_per_wg = narrow ? 32 : 64;
         p.q_tiles = (uint32_t)((s.t + rows_per_wg - 1) / rows_per_wg);
         p.scale = s.scale;
+        // Few query tiles over many keys (a chunk of a long prompt, a handful of rows late in a long
+        // context) would leave most compute units idle with one workgroup per (query tile, kv head):
+        // the keys of a tile are then split between several workgroups and lng_prefill_merge combines
+        // them, as the decode path does. Splits for one workgroup per compute unit (what is resident at a
+        // time; measured best: the merge grows with the splits), each keeping at least four key tiles.
+        p.splits = 1;
+        const uint64_t visible = p.window == LNG_WINDOW_FULL ? end : std::min<uint64_t>(end, p.window + rows_per_wg);
+        const uint64_t key_tiles = (visible + 63) / 64;
+        const uint64_t plain_wgs = (uint64_t)p.q_tiles * s.kv_heads;
+        if (!narrow && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
+            uint64_t want = g->cus / plain_wgs;
+            want = std::min<uint64_t>(want, key_tiles / 4);
+            want = std::min<uint64_t>(want, 64);
+            if (const char *env = getenv("LNG_PREFILL_SPLITS")) want = std::min<uint64_t>(std::max(1, atoi(env)), 64);
+            if (want > 1) p.splits = (uint32_t)want;
+        }
+        if (p.splits > 1) {
+            const size_t slots = (size_t)s.t * s.heads * p.splits;
+            if (int rc = reserve_scratch(g, slots * 64, slots * 2, 0)) return rc;
+            p.partial_o = g->scratch_o;
+            p.partial_ml = g->scratch_ml;
+        }
         Cmd c;
         c.fn = narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
         c.name = narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
-        c.grid[0] = p.q_tiles * (unsigned)s.kv_heads; // kv head fastest: one XCD's L2 per kv head
+        c.grid[0] = p.q_tiles * (unsigned)s.kv_heads * p.splits; // kv head fastest: one XCD's L2 per kv head
         c.block = 512;
         set_args(c, p);
         b->cmds.push_back(std::move(c));
+        if (p.splits > 1) {
+            Cmd m;
+            m.fn = g->prefill_merge;
+            m.name = "lng_prefill_merge";
+            m.grid[1] = (unsigned)(s.t * s.kv_heads);
+            m.block = 256;
+            set_args(m, p);
+            b->cmds.push_back(std::move(m));
+        }
         b->dispatches += 1;
         return LNG_OK;
     }
@@ -586,6 +617,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_merge", &g->decode_merge, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
+        {"lng_prefill_merge", &g->prefill_merge, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
         {"lng_add_rows", &g->add_rows, true},

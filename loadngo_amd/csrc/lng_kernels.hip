@@ -1144,7 +1144,8 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
 
     const uint32_t g = blockIdx.x % a.kv_heads;
-    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads;
+    const uint32_t split = (blockIdx.x / a.kv_heads) % a.splits;
+    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads / a.splits;
     const uint32_t group = a.heads / a.kv_heads;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -1165,7 +1166,12 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     const uint32_t window = windowed ? (uint32_t)a.window : 0u;
     const uint32_t kfirst = (windowed && pos_first + 1 > window) ? pos_first + 1 - window : 0u;
     const uint32_t tile0 = kfirst & ~(uint32_t)(PF_BN - 1);
-    const uint32_t n_tiles = (pos_last - tile0) / PF_BN + 1;
+    const uint32_t all_tiles = (pos_last - tile0) / PF_BN + 1;
+    // With splits, this workgroup takes tiles [first_tile, n_tiles) of the query tile's run (possibly
+    // none) and leaves (max, sum, unnormalised output) for lng_prefill_merge, which also adds the sink.
+    const bool partial = a.splits > 1u;
+    const uint32_t first_tile = (uint32_t)((uint64_t)all_tiles * split / a.splits);
+    const uint32_t n_tiles = (uint32_t)((uint64_t)all_tiles * (split + 1u) / a.splits);
     const bool ring = a.slots < end;
     const uint32_t slots = (uint32_t)a.slots;
     const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
@@ -1237,16 +1243,19 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     const bool optimistic = NH == 2 && attempt == 0;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
-        m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
-        l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
+        const bool sink_here = a.sinks && !partial;
+        m[h] = sink_here ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+        l[h] = (sink_here && hh == 0) ? 1.0f : 0.0f;
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
         }
     }
-    fetch(0, kr, vr);
-    stash(0, kr, vr);
+    if (first_tile < n_tiles) {
+        fetch(first_tile, kr, vr);
+        stash(first_tile & 1u, kr, vr);
+    }
     __syncthreads();
 
     // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
@@ -1362,7 +1371,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         const uint32_t kt0 = tile0 + tile * PF_BN;
         return kt0 + (PF_BN - 1) > pos_first || (windowed && kt0 + window < pos_first + PF_BM);
     };
-    uint32_t tile = 0;
+    uint32_t tile = first_tile;
     bool frozen = false;
     for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, std::false_type{}, tile); // window edge
     if (optimistic) {                                                                             // interior
@@ -1406,6 +1415,29 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     }
 
 
+    // ---- with splits: leave the partial state, lane holds dims 32db + 8blk + 4hh + i of its query ----
+    if (partial) {
+        if (wave_active && row_ok) {
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                if (h == 1 && !second_ok) continue;
+                const float total = l[h] + __shfl_xor(l[h], 32, 64);
+                const uint64_t slot = (((uint64_t)my_row * a.kv_heads + g) * a.splits + split) * group + (head[h] - g * group);
+                float *po = a.partial_o + slot * 64u;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int blk = 0; blk < 4; ++blk) {
+                        *(float4 *)(po + 32 * db + 8 * blk + 4 * hh) = make_float4(ot[h][db][4 * blk + 0], ot[h][db][4 * blk + 1],
+                                                                                   ot[h][db][4 * blk + 2], ot[h][db][4 * blk + 3]);
+                    }
+                }
+                if (hh == 0) *(float2 *)(a.partial_ml + slot * 2u) = make_float2(m[h], total);
+            }
+        }
+        return;
+    }
+
     // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------
     if (wave_active && row_ok) {
 #pragma unroll
@@ -1436,4 +1468,21 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
 
 extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1(lng_k_prefill a) {
     prefill_body<1>(a);
+}
+
+// Combines the splits of a prompt pass: one workgroup per (query row, kv head), the same merge as the
+// decode path's (the layouts of the partials agree); the sink joins here.
+extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefill p) {
+    const uint32_t row = blockIdx.y / p.kv_heads;
+    const uint32_t g = blockIdx.y % p.kv_heads;
+    lng_k_attn a{};
+    a.out = p.out;
+    a.sinks = (const char *)p.sinks;
+    a.partial_o = p.partial_o;
+    a.partial_ml = p.partial_ml;
+    a.n_chunks = p.splits;
+    lng_k_row it{};
+    it.out_offset = (uint64_t)row * p.heads * 64u * 2u;
+    it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;
+    merge_chunks<false>(a, it, g, p.heads / p.kv_heads, p.splits);
 }

@@ -310,6 +310,30 @@ def test_prefill_bf16_matches_the_cpu_reference(gpu, t, start, window, slots, he
     assert max_error(from_bf16_bits(plain), from_bf16_bits(want)) < BF16_TOL
 
 
+@pytest.mark.parametrize("t,start,window,slots,forced", [
+    (512, 3584, FULL, 4096, None), (64, 4000, FULL, 4096, None), (33, 5000, 2048, 5056, None), (100, 8000, FULL, 8128, None),
+    (512, 1536, FULL, 2048, "7"), (64, 960, FULL, 1024, "64"), (96, 0, FULL, 96, "5"), (160, 2000, 1500, 2176, "3"),
+    (64, 4000, 3000, 3072, None), (96, 6000, 4000, 4096, "6"),
+])
+def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots, forced, monkeypatch):
+    """A chunk of a long prompt (the reference passes 512 rows at a time, engine.rs:51), or a few rows late
+    in a long context: too few query tiles to fill the device, so the keys of a tile are split between
+    workgroups and merged afterwards. Same bound as the unsplit pass; LNG_PREFILL_SPLITS forces split counts
+    that leave some workgroups without a tile, or with edge tiles only."""
+    if forced:
+        monkeypatch.setenv("LNG_PREFILL_SPLITS", forced)
+    heads, kv_heads = 64, 8
+    end = start + t
+    q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    kr, vr = ring_layout(kb, t, start, slots, True), ring_layout(vb, t, start, slots, True)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    for sk in (sinks, None):
+        want = oracle.attention_bf16(qb, kb, vb, sk, start, window=window, scale=0.125, threads=THREADS)
+        got = run_attention(gpu, qb, kr, vr, sk, shape, True, C.BF16)
+        assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
 @pytest.mark.parametrize("spike_at,sinks_on", [(300, True), (300, False), (5, True), (5, False), (700, True)])
 def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on):
     """Long causal passes first keep the running maximum fixed after one interior tile and check the
