@@ -88,7 +88,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
                   decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
-                  q8_split_x = nullptr, q8_stream = nullptr, q8_tiled = nullptr, rmsnorm_rows = nullptr;
+                  q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_tiled = nullptr, rmsnorm_rows = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -626,6 +626,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prepare_v1", &g->prepare_v1, true},
         {"lng_q8_split_x", &g->q8_split_x, true},
         {"lng_q8_stream", &g->q8_stream, true},
+        {"lng_q8_stream_one", &g->q8_stream_one, true},
         {"lng_q8_tiled", &g->q8_tiled, true},
         {"lng_rmsnorm_rows", &g->rmsnorm_rows, true},
     };
@@ -1331,8 +1332,9 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
     Cmd c1;
     if (n < 32) {
         // bound by reading the matrix: one pass over it per 16 positions, x split in registers
-        c1.fn = b->gpu->q8_stream;
-        c1.name = "lng_q8_stream";
+        const bool one = n == 1 && cols <= 12288; // x of a single position is held in LDS (Q8S_X1 floats)
+        c1.fn = one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
+        c1.name = one ? "lng_q8_stream_one" : "lng_q8_stream";
         c1.grid[0] = (unsigned)((rows + 15) / 16);
         c1.grid[1] = (unsigned)((n + 15) / 16);
         c1.block = 1024;

@@ -766,15 +766,24 @@ __device__ __forceinline__ void q8_split8(const float (&x)[8], bf16x8 &hi, bf16x
     }
 }
 
-// Few positions (one pass of the matrix per 16; bound by reading the matrix): a workgroup takes
+// Few positions (one pass of the matrix per 16; bound by reading the matrix, in practice by the
+// number of load instructions a compute unit can take: some 40 cycles each): a workgroup takes
 // 16 rows, its sixteen wavefronts take every sixteenth block of the rows and their partial sums
 // meet in LDS. Lane l holds row l % 16 and, of each block, the 8 columns of group l / 16 - the B
-// operand; positions are the A operand, read as f32 and split in registers. All loads of eight
-// blocks are issued before the first product. Grid: x = 16-row tiles, y = 16-position tiles.
+// operand; positions are the A operand, read as f32 and split in registers. All loads of up to
+// eight blocks are issued before the first product; blocks past the end are skipped, loads and
+// all (the test is the same for the whole wavefront); the rows' scales come through LDS. ONE: a
+// single position, whose x the
+// workgroup first copies to LDS with 16-byte loads (a wavefront's two x loads per block become
+// two LDS reads; x must fit Q8S_X1 floats). Grid: x = 16-row tiles, y = 16-position tiles.
 #define Q8S_WAVES 16
 #define Q8S_UNROLL 8 // blocks in flight per wavefront: 128 blocks (4096 columns) in one turn
-extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k_q8 a) {
+#define Q8S_X1 12288 // floats of x held in LDS by the one-position form (48 KB)
+#define Q8S_SC_BLOCKS 512 // rows of up to this many blocks (16,384 columns) have their scales staged through LDS
+template <bool ONE> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a) {
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
+    __shared__ __attribute__((aligned(16))) float s_x1[ONE ? Q8S_X1 : 4];
+    __shared__ __attribute__((aligned(4))) uint16_t s_sc[16 * Q8S_SC_BLOCKS];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
@@ -787,29 +796,60 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
     const float *xrow = a.x + (uint64_t)pos * a.x_stride + 8u * kg;
     floatx4 y = {0.0f, 0.0f, 0.0f, 0.0f};
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t b0 = wave; b0 < blocks; b0 += Q8S_UNROLL * Q8S_WAVES) {
+    // The scales of the workgroup's 16 rows are one contiguous run (rows follow each other): copied to
+    // LDS a dword per thread, instead of 2-byte loads from 16 different rows per block and wavefront.
+    const bool sc_staged = blocks <= Q8S_SC_BLOCKS && r0 + 16u <= a.rows && ((uintptr_t)a.scales & 3u) == 0;
+    bool staged = false;
+    for (uint32_t b0 = wave; b0 < blocks || !staged; b0 += Q8S_UNROLL * Q8S_WAVES) {
         uint2 raw[Q8S_UNROLL];
-        float scale[Q8S_UNROLL];
+        uint16_t scale[Q8S_UNROLL];
         float4 xa[Q8S_UNROLL], xb[Q8S_UNROLL];
 #pragma unroll
         for (int u = 0; u < Q8S_UNROLL; ++u) {
             const uint32_t b = b0 + u * Q8S_WAVES;
-            const uint32_t bb = b < blocks ? b : b0; // a block past the end repeats a real one, scaled by 0
-            raw[u] = *(const uint2 *)(wrow + 32u * bb);
-            scale[u] = b < blocks ? f16_bits_to_f32(srow[bb]) : 0.0f;
-            xa[u] = *(const float4 *)(xrow + 32u * bb);
-            xb[u] = *(const float4 *)(xrow + 32u * bb + 4u);
+            raw[u] = make_uint2(0, 0);
+            scale[u] = 0;
+            xa[u] = xb[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (b < blocks) { // the same for every lane of the wavefront
+                raw[u] = *(const uint2 *)(wrow + 32u * b);
+                if (!sc_staged) scale[u] = srow[b];
+                if (!ONE) {
+                    xa[u] = *(const float4 *)(xrow + 32u * b);
+                    xb[u] = *(const float4 *)(xrow + 32u * b + 4u);
+                }
+            }
+        }
+        if (!staged) { // every wavefront comes here exactly once, in its first turn
+            if (ONE) {
+                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                    *(float4 *)(&s_x1[i]) = *(const float4 *)(a.x + i);
+                }
+            }
+            if (sc_staged) { // 16 * blocks * 2 bytes from a 32-byte boundary
+                const uint32_t *src = (const uint32_t *)(a.scales + (uint64_t)r0 * blocks);
+                for (uint32_t i = threadIdx.x; i < 8u * blocks; i += 64u * Q8S_WAVES) ((uint32_t *)s_sc)[i] = src[i];
+            }
+            __syncthreads();
+            staged = true;
         }
 #pragma unroll
         for (int u = 0; u < Q8S_UNROLL; ++u) {
-            const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
-            bf16x8 hi, lo;
-            q8_split8(xs, hi, lo);
-            const bf16x8 wb = q8_codes_to_bf16(raw[u]);
-            floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, wb, acc, 0, 0, 0);
+            const uint32_t b = b0 + u * Q8S_WAVES;
+            if (b < blocks) {
+                if (ONE) {
+                    xa[u] = *(const float4 *)(&s_x1[32u * b + 8u * kg]);
+                    xb[u] = *(const float4 *)(&s_x1[32u * b + 8u * kg + 4u]);
+                }
+                const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                bf16x8 hi, lo;
+                q8_split8(xs, hi, lo);
+                const bf16x8 wb = q8_codes_to_bf16(raw[u]);
+                floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, wb, acc, 0, 0, 0);
+                const float sc = f16_bits_to_f32(sc_staged ? s_sc[j * blocks + b] : scale[u]);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(scale[u], acc[i], y[i]);
+                for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(sc, acc[i], y[i]);
+            }
         }
     }
     if (wave != 0) {
@@ -826,6 +866,14 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
         const uint32_t p = p0 + 4u * kg + i; // accumulator row = position, column = matrix row
         if (p < a.n && r0 + j < a.rows) a.y[(uint64_t)p * a.y_stride + r0 + j] = sum;
     }
+}
+
+extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k_q8 a) {
+    q8_stream_body<false>(a);
+}
+
+extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_one(lng_k_q8 a) {
+    q8_stream_body<true>(a);
 }
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128

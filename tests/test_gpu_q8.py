@@ -87,6 +87,33 @@ def test_strided_positions_and_untouched_gaps(gpu):
     assert np.isnan(got[:-1, rows:]).all()           # 0xFF fill: gaps of y untouched
 
 
+@pytest.mark.parametrize("n", [1, 9])
+def test_scales_at_an_offset_of_two_bytes(gpu, n):
+    """The reference asks 2-byte alignment of the scales (apple.rs:1799-1811); the few-position kernel copies
+    a workgroup's scales to LDS a dword at a time only when they start on a 4-byte boundary."""
+    rows, cols = 96, 160
+    codes, bits, elements = q8_test_matrix(rows, cols, 21)
+    x = xorshift_values(17, n * cols).reshape(n, cols)
+    padded = np.concatenate([np.array([0x7E00], np.uint16), bits])   # a NaN in front of the scales
+    bufs = [gpu.upload(codes), gpu.upload(padded), gpu.upload(x), gpu.buffer(n * rows * 4)]
+    batch = gpu.batch(bufs)
+    m = (C.Slice(0, 0, codes.nbytes), C.Slice(1, 2, bits.nbytes))
+    try:
+        if n == 1:
+            batch.gemv_q8_0(m, C.Slice(2, 0, x.nbytes), C.Slice(3, 0, rows * 4), rows, cols)
+        else:
+            batch.gemm_q8_0(m, C.Slice(2, 0, x.nbytes), C.Slice(3, 0, n * rows * 4), rows, cols, n, (cols, rows))
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        got = bufs[3].read(np.float32).reshape(n, rows)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    want = x.astype(np.float64) @ elements.T
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-5
+
+
 def test_refusals_of_the_reference(gpu):
     """q8_0_and_gpt_oss_glue.rs:180-210 and the checks of apple.rs:889-894, 995-999, 1799-1806, 1868-1872."""
     bufs = [gpu.buffer(1 << 16) for _ in range(4)]
