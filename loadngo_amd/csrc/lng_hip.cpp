@@ -538,7 +538,11 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             Cmd m;
             m.fn = g->prefill_merge;
             m.name = "lng_prefill_merge";
-            m.grid[1] = (unsigned)(s.t * s.kv_heads);
+            if (p.splits <= 8) {
+                m.grid[0] = (unsigned)((s.t * s.heads + 15) / 16); // a thread per (row, head, four dims)
+            } else {
+                m.grid[1] = (unsigned)(s.t * s.kv_heads);          // a workgroup per (row, kv head)
+            }
             m.block = 256;
             set_args(m, p);
             b->cmds.push_back(std::move(m));

@@ -1518,9 +1518,56 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     prefill_body<1>(a);
 }
 
-// Combines the splits of a prompt pass: one workgroup per (query row, kv head), the same merge as the
-// decode path's (the layouts of the partials agree); the sink joins here.
+// Combines the splits of a prompt pass; the sink joins here. Up to eight splits (the usual case: one
+// workgroup per compute unit needs few): a thread per (row, head, four dims) requests its splits' partial
+// outputs at once, works out the weights from the (max, sum) pairs itself - the 16 threads of a head all
+// do, it is a handful of exponentials - and writes four outputs: no LDS, no barrier, one wait for memory.
+// Grid x = ceil(t * heads / 16) workgroups of 256. More splits: one workgroup per (row, kv head), the
+// decode path's merge (the layouts of the partials agree), grid y = t * kv_heads.
 extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefill p) {
+    const uint32_t group = p.heads / p.kv_heads;
+    if (p.splits <= 8u) {
+        const uint64_t pair = (uint64_t)blockIdx.x * 16u + (threadIdx.x >> 4); // row * heads + head
+        if (pair >= p.t * p.heads) return;
+        const uint32_t row = (uint32_t)(pair / p.heads), head = (uint32_t)(pair % p.heads);
+        const uint32_t g = head / group, h = head % group, d4 = (threadIdx.x & 15u) * 4u;
+        const uint64_t slot0 = (((uint64_t)row * p.kv_heads + g) * p.splits) * group + h;
+        float4 o[8];
+        float2 ml[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if ((uint32_t)c < p.splits) {
+                o[c] = *(const float4 *)(p.partial_o + (slot0 + (uint64_t)c * group) * 64u + d4);
+                ml[c] = *(const float2 *)(p.partial_ml + (slot0 + (uint64_t)c * group) * 2u);
+            }
+        }
+        const float sink2 = p.sinks ? p.sinks[head] * LNG_LOG2E : LNG_NEG_INF;
+        float top = sink2;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if ((uint32_t)c < p.splits) top = fmaxf(top, ml[c].x);
+        }
+        float z = sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top);
+        float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if ((uint32_t)c < p.splits) {
+                const float w = ml[c].x == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(ml[c].x - top);
+                z += ml[c].y * w;
+                sum.x += o[c].x * w;
+                sum.y += o[c].y * w;
+                sum.z += o[c].z * w;
+                sum.w += o[c].w * w;
+            }
+        }
+        ushort4 r;
+        r.x = f32_to_bf16_bits(sum.x / z);
+        r.y = f32_to_bf16_bits(sum.y / z);
+        r.z = f32_to_bf16_bits(sum.z / z);
+        r.w = f32_to_bf16_bits(sum.w / z);
+        *(ushort4 *)((uint16_t *)p.out + pair * 64u + d4) = r;
+        return;
+    }
     const uint32_t row = blockIdx.y / p.kv_heads;
     const uint32_t g = blockIdx.y % p.kv_heads;
     lng_k_attn a{};
@@ -1532,5 +1579,5 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     lng_k_row it{};
     it.out_offset = (uint64_t)row * p.heads * 64u * 2u;
     it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;
-    merge_chunks<false>(a, it, g, p.heads / p.kv_heads, p.splits);
+    merge_chunks<false>(a, it, g, group, p.splits);
 }
