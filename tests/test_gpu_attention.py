@@ -377,6 +377,27 @@ def test_config4_prefill_8192_sampled_rows(gpu, window):
     assert max_error(from_bf16_bits(got[rows]), want) < BF16_TOL
 
 
+@pytest.mark.parametrize("chunk", [512, 96])
+def test_config4_prefill_in_calls_of_fewer_rows_equals_the_one_call(gpu, chunk):
+    """The 8192-position full-causal pass made the way the reference makes it (engine.rs:51: a run of rows per
+    call, each over the cache so far; the keys of a call are split between workgroups and merged) gives the
+    rows of the single call: the same softmax summed in another order, both rounded to bf16 once."""
+    t, heads, kv_heads = 8192, 64, 8
+    rng = np.random.default_rng(45)
+    qb = to_bf16_bits((rng.standard_normal((t, heads, 64), dtype=np.float32) * 0.5))
+    kb = to_bf16_bits((rng.standard_normal((t, kv_heads, 64), dtype=np.float32) * 0.5))
+    vb = to_bf16_bits((rng.standard_normal((t, kv_heads, 64), dtype=np.float32) * 0.5))
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    one = from_bf16_bits(run_attention(gpu, qb, kb, vb, sinks, C.GroupedShape(t, 0, heads, kv_heads, 64, FULL, t, 0.125), True, C.BF16))
+    starts = list(range(0, t, chunk))[-3:] + [0, chunk * 7]     # the last calls (longest caches), the first, one between
+    for start in starts:
+        n = min(chunk, t - start)
+        shape = C.GroupedShape(n, start, heads, kv_heads, 64, FULL, t, 0.125)
+        rows = (start + n + 31) // 32 * 32
+        part = from_bf16_bits(run_attention(gpu, qb[start:start + n], kb[:rows], vb[:rows], sinks, shape, True, C.BF16))
+        assert np.abs(part - one[start:start + n]).max() < 2.0 ** -7, (start, n)   # a bf16 step or two at |o| < 1
+
+
 # ---- configuration 5 at its real per-layer size, through a size-independent identity -----------
 def test_config5_layer_at_full_size_periodic_identity(gpu):
     """One layer of the long-context stack at its real shape (batch 16, context 131072, 2 GiB of K
