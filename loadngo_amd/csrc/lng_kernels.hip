@@ -1317,6 +1317,10 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             const uint32_t kt0 = tile0 + tile * PF_BN; // position of the tile's first key
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) { // the tile's two blocks of 32 keys
+                if constexpr (MASK && NH == 1) { // windows: a block no query of the workgroup sees (before the window, past the last row)
+                    const uint32_t b0 = kt0 + 32u * kb;
+                    if (b0 > pos_last || b0 + 31u < kfirst) continue;
+                }
                 // ---- S^T = K . Q^T, both heads ------------------------------------------------------
                 bf16x8 ka[4];
 #pragma unroll
