@@ -72,3 +72,41 @@ def test_random_shapes_agree_with_the_oracle_or_are_refused(gpu, tiled, dtype):
             assert max_error(got, want) <= 2e-2, f"{what}: {max_error(got, want)}"
         ran += 1
     assert ran >= 15 and refused >= 1, (ran, refused)
+
+
+def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
+    """bf16, head width 64, 32..600 rows after up to 6,000 cached positions, flat caches and rings, full
+    attention and windows above 1,024: the calls whose keys the library splits between workgroups, with the
+    library's own split count and with forced ones (including more splits than tiles)."""
+    rng = np.random.default_rng(77)
+    ran = 0
+    for _ in range(40):
+        kv_heads = int(rng.choice([1, 2, 4, 8]))
+        heads = kv_heads * int(rng.choice([1, 2, 3, 5, 8]))
+        t = int(rng.choice([32, 33, 64, 65, 96, 128, 200, 511, 512, 600]))
+        start = int(rng.choice([0, 31, 500, 1000, 2047, 3000, 4097, 6000]))
+        window = int(rng.choice([FULL, FULL, FULL, 1025, 1500, 3000]))
+        end = start + t
+        if rng.integers(0, 2):
+            slots = end + int(rng.integers(0, 70))
+        else:
+            slots = ((window if window != FULL else end) + t + int(rng.integers(0, 200)) + 31) // 32 * 32
+        forced = rng.choice([None, None, "1", "2", "3", "5", "8", "9", "17", "64"])
+        if forced:
+            monkeypatch.setenv("LNG_PREFILL_SPLITS", str(forced))
+        else:
+            monkeypatch.delenv("LNG_PREFILL_SPLITS", raising=False)
+        if not orc.accepts(t, start, heads, kv_heads, 64, window, slots, True):
+            continue
+        qb = to_bf16_bits((rng.standard_normal((t, heads, 64)) * 0.7).astype(np.float32))
+        kb = to_bf16_bits((rng.standard_normal((end, kv_heads, 64)) * 0.7).astype(np.float32))
+        vb = to_bf16_bits((rng.standard_normal((end, kv_heads, 64)) * 0.5).astype(np.float32))
+        sinks = rng.standard_normal(heads).astype(np.float32) if rng.integers(0, 3) else None
+        shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+        want = from_bf16_bits(orc.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS))
+        got = from_bf16_bits(run_attention(gpu, qb, ring_layout(kb, t, start, slots, True),
+                                           ring_layout(vb, t, start, slots, True), sinks, shape, True, C.BF16))
+        what = f"t={t} start={start} H={heads} G={kv_heads} window={window} slots={slots} splits={forced}"
+        assert not np.isnan(got).any() and max_error(got, want) <= 2e-2, f"{what}: {max_error(got, want)}"
+        ran += 1
+    assert ran >= 15, ran
