@@ -484,7 +484,14 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     lng_gpu *g = b->gpu;
     const bool aligned16 = ((q.offset | k.offset | v.offset | out.offset) & 15u) == 0;
 
-    if (tiled && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16) {
+    // The row-by-row operator with several rows over a long run of keys (the tail of a prompt, a few
+    // tokens at once late in a context) reads the cache once per row in the decode kernel; the prompt-pass
+    // kernel reads it once per call and gives the same rows (it touches no row outside
+    // [first visible position, last position], which is all the row-by-row operator promises to be there).
+    // Measured break-even on 64/8 heads: rows x visible keys of about 32 K (16 rows over 2,048 keys, 4 over 8,192).
+    const uint64_t seen = std::min<uint64_t>(end, s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t);
+    const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && s.t * seen >= 32768 && !getenv("LNG_PLAIN_ROW_BY_ROW");
+    if ((tiled || several_rows) && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16) {
         lng_k_prefill p{};
         p.q = (const char *)oq.buf->ptr + q.offset;
         p.k = (const char *)ok.buf->ptr + k.offset;

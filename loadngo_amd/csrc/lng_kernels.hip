@@ -1261,7 +1261,8 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
     auto fetch = [&](uint32_t tile, uint4 &kr, uint4 &vr) {
         uint32_t p = tile0 + tile * PF_BN + ld_key;
-        p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway
+        p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway,
+        p = p < kfirst ? kfirst : p;     // and so are rows before the first one (a ring may not hold them any more)
         const uint32_t r = ring ? p % slots : p;
         kr = *(const uint4 *)(kbase + (uint64_t)r * row_bytes);
         vr = *(const uint4 *)(vbase + (uint64_t)r * row_bytes);

@@ -334,6 +334,32 @@ def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots
         assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
 
 
+@pytest.mark.parametrize("t,start,window,slots", [(8, 5000, FULL, 5008), (31, 3000, 2000, 2031), (4, 9000, FULL, 9100),
+                                                  (16, 2100, FULL, 2116), (31, 40000, 1100, 1131), (5, 7000, 6999, 7004)])
+def test_several_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, monkeypatch):
+    """attention_grouped with a handful of rows over thousands of keys (the tail of a prompt: gpu.rs:760-806
+    takes this operator below 32 rows) is served by the prompt-pass kernel, which reads the cache once instead
+    of once per row. Same results as row by row (LNG_PLAIN_ROW_BY_ROW) and as the CPU reference; rows of the
+    cache outside [first visible, last] hold NaN, as in attention_grouped.rs:57; rings need not be multiples
+    of 32 rows here."""
+    heads, kv_heads = 64, 8
+    end = start + t
+    q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    kr, vr = ring_layout(kb, t, start, slots, False), ring_layout(vb, t, start, slots, False)
+    first = 0 if window == FULL else max(0, start + 1 - window)
+    if slots >= end:                               # flat: poison what no query may see
+        kr[:first] = 0x7FC0
+        vr[:first] = 0x7FC0
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    want = from_bf16_bits(oracle.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS))
+    got = from_bf16_bits(run_attention(gpu, qb, kr, vr, sinks, shape, False, C.BF16))
+    assert not np.isnan(got).any() and max_error(got, want) < BF16_TOL
+    monkeypatch.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
+    rows = from_bf16_bits(run_attention(gpu, qb, kr, vr, sinks, shape, False, C.BF16))
+    assert max_error(rows, want) < BF16_TOL and np.abs(rows - got).max() < 2.0 ** -6
+
+
 @pytest.mark.parametrize("spike_at,sinks_on", [(300, True), (300, False), (5, True), (5, False), (700, True)])
 def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on):
     """Long causal passes first keep the running maximum fixed after one interior tile and check the
