@@ -102,7 +102,43 @@ __device__ __forceinline__ void attn_generic(const lng_k_attn &a) {
         acc[i] = 0.0f;
     }
     float m = LNG_NEG_INF, l = 0.0f;
-    for (uint64_t p = first + wave; p <= last; p += 4) {
+    uint64_t p = first + wave;
+    if (dim <= 64u) {
+        // One element per lane and row: sixteen of the wavefront's positions at a time, all their K and V
+        // loads in flight together (one position per turn is a chain of memory latencies, 1 ms for 4,096
+        // keys), then one block step of the online softmax.
+        constexpr int U = 16;
+        const bool mine = lane < dim;
+        for (; p <= last; p += 4u * U) {
+            float kx[U], vx[U], sc[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint64_t pu = p + 4u * u;
+                const uint64_t r = (pu <= last ? pu : last) % it.slots;
+                kx[u] = mine ? load_elem<T>(kb + r * stride + lane) : 0.0f;
+                vx[u] = mine ? load_elem<T>(vb + r * stride + lane) : 0.0f;
+            }
+            float top = LNG_NEG_INF;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float s = wave_sum(qv[0] * kx[u]) * a.scale;
+                sc[u] = p + 4u * u <= last ? s : LNG_NEG_INF;
+                top = fmaxf(top, sc[u]);
+            }
+            const float next = fmaxf(m, top); // the first position of the block is always a real one
+            const float keep = m == LNG_NEG_INF ? 0.0f : expf(m - next);
+            l *= keep;
+            acc[0] *= keep;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const float w = sc[u] == LNG_NEG_INF ? 0.0f : expf(sc[u] - next);
+                l += w;
+                acc[0] += w * vx[u];
+            }
+            m = next;
+        }
+    }
+    for (; p <= last; p += 4) {
         const uint64_t r = p % it.slots;
         const T *kr = kb + r * stride;
         const T *vr = vb + r * stride;
