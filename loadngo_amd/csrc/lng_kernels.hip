@@ -61,10 +61,21 @@ __device__ __forceinline__ uint64_t first_visible(uint64_t last, uint64_t window
     return (window != LNG_WINDOW_FULL && last + 1 > window) ? last + 1 - window : 0;
 }
 
+// Sum over the 64 lanes, in every lane: four steps inside each row of 16 lanes with data-parallel
+// primitives (neighbour, pair, mirrored half row, mirrored row), then the two lane-swap instructions
+// across rows. All VALU: the shuffle form goes through the LDS crossbar six times, one after the other.
 __device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-    for (int s = 32; s >= 1; s >>= 1) x += __shfl_xor(x, s, 64);
-    return x;
+    auto dpp = [](float v, auto ctrl) {
+        return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), decltype(ctrl)::value, 0xf, 0xf, true));
+    };
+    x += dpp(x, std::integral_constant<int, 0xB1>{});  // quad_perm [1,0,3,2]
+    x += dpp(x, std::integral_constant<int, 0x4E>{});  // quad_perm [2,3,0,1]
+    x += dpp(x, std::integral_constant<int, 0x141>{}); // row_half_mirror
+    x += dpp(x, std::integral_constant<int, 0x140>{}); // row_mirror
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // =============================================================================================
