@@ -367,9 +367,33 @@ def run_q8(gpu, steps, warmup):
                       "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS, "tflops": flops / g / 1e12}
         x.free()
         y.free()
+    # the same matrix on bf16 positions (what a bf16 attention leaves for the output projection): one operand
+    # plane instead of two, no split of x
+    for label, n in (("decode_16_sequences_bf16_positions", 16), ("prompt_8192_bf16_positions", 8192)):
+        x, y = gpu.buffer(n * cols * 2), gpu.buffer(n * rows * 4)
+        b = gpu.batch([x])
+        b.fill_synthetic(C.Slice(0, 0, x.len), C.BF16, 78, 0.5, 0)
+        b.run()
+        b.drop()
+
+        def go16():
+            batch = gpu.batch([x, y])
+            batch.gemm_q8_0_bf16((batch.attach(codes), batch.attach(scales)), C.Slice(0, 0, x.len), C.Slice(1, 0, y.len),
+                                 rows, cols, n, (cols, rows))
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        for _ in range(warmup):
+            go16()
+        runs = sorted(go16() for _ in range(max(steps, 5)))
+        g = runs[len(runs) // 2]
+        out[label] = {"positions": n, "gpu_us": g * 1e6, "tflops": 2 * n * rows * cols / g / 1e12}
+        x.free()
+        y.free()
     codes.free()
     scales.free()
-    out["workload"] = "Q8_0 product, 4096 x 2880 (gpt-oss-20b query projection), f32 positions"
+    out["workload"] = "Q8_0 product, 4096 x 2880 (gpt-oss-20b query projection), f32 positions unless named otherwise"
     return out
 
 

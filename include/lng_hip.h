@@ -279,6 +279,15 @@ int lng_hip_gemm_q8_0_tiled(lng_batch *batch, lng_slice codes, lng_slice scales,
                             lng_slice y, uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride,
                             uint64_t y_stride);
 
+/* No counterpart in the reference (its attention output is f32): the same product for positions
+ * that are bf16 already - the output of a bf16 attention, feeding the output projection
+ * (gpt-oss/src/gpu.rs:807-817) without a widening pass. x holds n rows of cols bf16 values x_stride
+ * values apart (a multiple of 8, >= cols), on a 16-byte boundary; y is f32 as above. Any n >= 1 and
+ * any rows. A bf16 value is exact as a matrix operand, so this takes half the matrix instructions
+ * of the f32 form and no split of x. */
+int lng_hip_gemm_q8_0_bf16(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                           uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride);
+
 /* Deterministic synthetic data written on the device (benchmarks and full-size tests):
  * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
  * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The

@@ -127,6 +127,7 @@ SYMBOLS = {
     "lng_hip_gemv_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64]),
     "lng_hip_gemm_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_gemm_q8_0_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
+    "lng_hip_gemm_q8_0_bf16": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_prepare_attention": (ctypes.c_int, [_P, ctypes.POINTER(_PrepareBuffers), ctypes.POINTER(_PrepareItem),
                                                  ctypes.c_size_t, _U64, _U64, _U64, _U64, ctypes.c_int]),
 }
@@ -464,6 +465,12 @@ class Batch:
         codes, scales = matrix
         _check(library().lng_hip_gemm_q8_0_tiled(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols, n,
                                                  strides[0], strides[1]))
+
+    def gemm_q8_0_bf16(self, matrix, x, y, rows, cols, n, strides):
+        """The Q8_0 product of bf16 positions (no counterpart in the reference): x is [n][x_stride] bf16, y f32."""
+        codes, scales = matrix
+        _check(library().lng_hip_gemm_q8_0_bf16(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols, n,
+                                                strides[0], strides[1]))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))

@@ -88,7 +88,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
                   decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
-                  q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_tiled = nullptr, rmsnorm_rows = nullptr;
+                  q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr, q8_tiled_bf16 = nullptr, rmsnorm_rows = nullptr;
     std::string name;
     unsigned cus = 256;
 
@@ -639,6 +639,8 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_q8_stream", &g->q8_stream, true},
         {"lng_q8_stream_one", &g->q8_stream_one, true},
         {"lng_q8_tiled", &g->q8_tiled, true},
+        {"lng_q8_tiled_bf16", &g->q8_tiled_bf16, true},
+        {"lng_q8_stream_bf16", &g->q8_stream_bf16, true},
         {"lng_rmsnorm_rows", &g->rmsnorm_rows, true},
     };
     for (auto &w : wanted) {
@@ -1305,8 +1307,10 @@ int reserve_x(lng_gpu *g, size_t bytes, char **out) {
 }
 
 // The three Q8_0 products share their checks (apple.rs:1792-1883) and their kernels.
+// x_bf16: the positions are bf16 (exact as one operand plane: no split, one matrix instruction per block).
 int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, const lng_slice &x, const lng_slice &y,
-               uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled) {
+               uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled,
+               bool x_bf16 = false) {
     if (int rc = need_recording(b)) return rc;
     if (tiled && (rows % 64 != 0 || cols % 32 != 0 || n % 32 != 0)) { // apple.rs:1868-1872
         return fail(LNG_ERR_DISPATCH, "tiled Q8_0 product needs rows %% 64, cols %% 32 and n %% 32 == 0: %llu x %llu, n %llu",
@@ -1315,7 +1319,7 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
     if (rows == 0 || cols == 0 || !fits_u32(rows) || !fits_u32(cols)) { // apple.rs:889-894
         return fail(LNG_ERR_DISPATCH, "unsupported shape %llux%llu", (unsigned long long)rows, (unsigned long long)cols);
     }
-    if (gemm && (n == 0 || x_stride < cols || y_stride < rows || x_stride % 4 != 0)) { // apple.rs:995-999
+    if (gemm && (n == 0 || x_stride < cols || y_stride < rows || x_stride % (x_bf16 ? 8 : 4) != 0)) { // apple.rs:995-999 (16-byte rows)
         return fail(LNG_ERR_DISPATCH, "%llu positions of %llux%llu with strides %llu/%llu", (unsigned long long)n,
                     (unsigned long long)rows, (unsigned long long)cols, (unsigned long long)x_stride,
                     (unsigned long long)y_stride);
@@ -1327,7 +1331,7 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
     Operand oc, os, ox, oy;
     if (int rc = check_slice(b, "codes", codes, rows * cols, 16, &oc)) return rc;
     if (int rc = check_slice(b, "scales", scales, rows * cols / 32 * 2, 2, &os)) return rc;
-    if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * 4, 16, &ox)) return rc;
+    if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * (x_bf16 ? 2 : 4), 16, &ox)) return rc;
     if (int rc = check_slice(b, "y", y, ((n - 1) * y_stride + rows) * 4, 4, &oy)) return rc;
     if (int rc = check_output(b, oy, {&oc, &os, &ox})) return rc;
     lng_k_q8 a{};
@@ -1341,14 +1345,33 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
     a.x_stride = (uint32_t)x_stride;
     a.y_stride = (uint32_t)y_stride;
     Cmd c1;
+    if (x_bf16) {
+        a.x = nullptr;
+        a.x_hi = (const uint16_t *)((const char *)ox.buf->ptr + x.offset);
+        a.plane_stride = (uint32_t)x_stride;
+    }
     if (n < 32) {
         // bound by reading the matrix: one pass over it per 16 positions, x split in registers
-        const bool one = n == 1 && cols <= 12288; // x of a single position is held in LDS (Q8S_X1 floats)
-        c1.fn = one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
-        c1.name = one ? "lng_q8_stream_one" : "lng_q8_stream";
+        const bool one = n == 1 && cols <= 12288 && !x_bf16; // x of a single position is held in LDS (Q8S_X1 floats)
+        c1.fn = x_bf16 ? b->gpu->q8_stream_bf16 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
+        c1.name = x_bf16 ? "lng_q8_stream_bf16" : one ? "lng_q8_stream_one" : "lng_q8_stream";
         c1.grid[0] = (unsigned)((rows + 15) / 16);
         c1.grid[1] = (unsigned)((n + 15) / 16);
         c1.block = 1024;
+    } else if (x_bf16) {
+        const uint64_t n_pad = (n + 127) / 128 * 128;
+        if (n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
+        c1.fn = b->gpu->q8_tiled_bf16;
+        c1.name = "lng_q8_tiled_bf16";
+        const uint64_t row_tiles = (rows + 255) / 256, pos_tiles = n_pad / 128;
+        uint64_t ids = row_tiles * pos_tiles;
+        if (pos_tiles >= 8) {
+            const uint64_t per_xcd = (pos_tiles + 7) / 8;
+            ids = 8 * ((per_xcd + 3) / 4) * ((row_tiles + 7) / 8) * 32;
+        }
+        if (ids > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
+        c1.grid[0] = (unsigned)ids;
+        c1.block = 512;
     } else {
         const uint64_t n_pad = (n + 127) / 128 * 128;
         if (!fits_u32(n_pad * cols) || n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
@@ -1371,6 +1394,7 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
         b->cmds.push_back(std::move(c0));
         a.x_hi = sp.hi;
         a.x_lo = sp.lo;
+        a.plane_stride = (uint32_t)cols;
         c1.fn = b->gpu->q8_tiled;
         c1.name = "lng_q8_tiled";
         // one-dimensional grid; the kernel maps ids to tiles (XCD-aware from eight position tiles on,
@@ -1407,6 +1431,11 @@ extern "C" int lng_hip_gemm_q8_0_tiled(lng_batch *b, lng_slice codes, lng_slice 
                                        uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride,
                                        uint64_t y_stride) {
     return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, true);
+}
+
+extern "C" int lng_hip_gemm_q8_0_bf16(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
+                                      uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride) {
+    return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, false, true);
 }
 
 extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, uint64_t seed, float scale,

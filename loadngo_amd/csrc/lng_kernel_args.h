@@ -153,7 +153,8 @@ typedef struct lng_k_q8 {
     uint32_t n;
     uint32_t x_stride;
     uint32_t y_stride;
-    uint32_t pad;
+    uint32_t plane_stride;   /* elements between positions of x_hi / x_lo: cols for the split planes; x's own stride
+                                when the positions are bf16 already (x_hi = x, no x_lo, n rows only) */
 } lng_k_q8;
 
 /* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with

@@ -827,7 +827,7 @@ __device__ __forceinline__ void q8_split8(const float (&x)[8], bf16x8 &hi, bf16x
 #define Q8S_UNROLL 8 // blocks in flight per wavefront: 128 blocks (4096 columns) in one turn
 #define Q8S_X1 12288 // floats of x held in LDS by the one-position form (48 KB)
 #define Q8S_SC_BLOCKS 512 // rows of up to this many blocks (16,384 columns) have their scales staged through LDS
-template <bool ONE> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a) {
+template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a) {
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
     __shared__ __attribute__((aligned(16))) float s_x1[ONE ? Q8S_X1 : 4];
     __shared__ __attribute__((aligned(4))) uint16_t s_sc[16 * Q8S_SC_BLOCKS];
@@ -841,6 +841,7 @@ template <bool ONE> __device__ __forceinline__ void q8_stream_body(const lng_k_q
     const int8_t *wrow = a.codes + (uint64_t)row * a.cols + 8u * kg;
     const uint16_t *srow = a.scales + (uint64_t)row * blocks;
     const float *xrow = a.x + (uint64_t)pos * a.x_stride + 8u * kg;
+    const uint16_t *xrow16 = a.x_hi + (uint64_t)pos * a.plane_stride + 8u * kg; // XBF16: positions in bf16
     floatx4 y = {0.0f, 0.0f, 0.0f, 0.0f};
     const floatx4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
     // The scales of the workgroup's 16 rows are one contiguous run (rows follow each other): copied to
@@ -860,7 +861,9 @@ template <bool ONE> __device__ __forceinline__ void q8_stream_body(const lng_k_q
             if (b < blocks) { // the same for every lane of the wavefront
                 raw[u] = *(const uint2 *)(wrow + 32u * b);
                 if (!sc_staged) scale[u] = srow[b];
-                if (!ONE) {
+                if (XBF16) {
+                    xa[u] = *(const float4 *)(xrow16 + 32u * b); // eight bf16 values, used as they are
+                } else if (!ONE) {
                     xa[u] = *(const float4 *)(xrow + 32u * b);
                     xb[u] = *(const float4 *)(xrow + 32u * b + 4u);
                 }
@@ -887,12 +890,17 @@ template <bool ONE> __device__ __forceinline__ void q8_stream_body(const lng_k_q
                     xa[u] = *(const float4 *)(&s_x1[32u * b + 8u * kg]);
                     xb[u] = *(const float4 *)(&s_x1[32u * b + 8u * kg + 4u]);
                 }
-                const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
-                bf16x8 hi, lo;
-                q8_split8(xs, hi, lo);
                 const bf16x8 wb = q8_codes_to_bf16(raw[u]);
-                floatx4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, wb, acc, 0, 0, 0);
+                floatx4 acc;
+                if (XBF16) {
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[u]), wb, zero4, 0, 0, 0);
+                } else {
+                    const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                    bf16x8 hi, lo;
+                    q8_split8(xs, hi, lo);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(lo, wb, acc, 0, 0, 0);
+                }
                 const float sc = f16_bits_to_f32(sc_staged ? s_sc[j * blocks + b] : scale[u]);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) y[i] = __builtin_fmaf(sc, acc[i], y[i]);
@@ -921,6 +929,11 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_one(lng_k_q8 a) {
     q8_stream_body<true>(a);
+}
+
+// positions already in bf16 (the output of a bf16 attention): one matrix instruction per block
+extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_bf16(lng_k_q8 a) {
+    q8_stream_body<false, true>(a);
 }
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128
@@ -956,11 +969,13 @@ __device__ __forceinline__ bf16x8 q8_codes_to_bf16_perm(uint2 raw) {
 
 // WAVES wavefronts per workgroup: 8 (64 x 64 outputs each, two per SIMD) is what is launched; 16 (64 rows x
 // 32 positions each, four per SIMD with half the registers) measures the same and is not instantiated.
-template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q8 &a) {
+// PLANES: 2 for f32 positions split into hi and lo bf16 planes; 1 when the positions are bf16 already
+// (x_hi is then x itself, its rows plane_stride apart and only n of them: rows past n repeat the last).
+template <int WAVES, int PLANES = 2> __device__ __forceinline__ void q8_tiled_body(const lng_k_q8 &a) {
     constexpr int MT = WAVES == 8 ? 4 : 2;       // groups of 16 positions per wavefront
-    constexpr int XQ = 32 / WAVES;               // x loads per wavefront and stage (32 in all: 2 planes x 16 groups of 8 positions)
+    constexpr int XQ = 16 * PLANES / WAVES;      // x loads per wavefront and stage (PLANES x 16 groups of 8 positions in all)
     constexpr int WQ = 16 / WAVES;               // code loads (16 in all: groups of 16 rows)
-    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][2][Q8T_PLANE];   // [stage % 2][plane]
+    __shared__ __attribute__((aligned(16))) uint16_t s_x[2][PLANES][Q8T_PLANE]; // [stage % 2][plane]
     __shared__ __attribute__((aligned(16))) uint16_t s_w[2][Q8T_ROWS * 64];  // [stage % 2]: 64 codes per row as bf16
     __shared__ uint16_t s_sc[2][Q8T_ROWS * 2];                               // [stage % 2]: two block scales per row
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -1006,7 +1021,8 @@ template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q
         const uint32_t pos = 8u * (idx & 15u) + (lane >> 3);
         x_chunk[q] = (lane & 7u) ^ ((pos >> 1) & 7u); // the logical chunk kept at this physical place
         const uint16_t *plane = (idx >> 4) ? a.x_lo : a.x_hi;
-        x_src[q] = plane + (uint64_t)(p0 + pos) * a.cols; // planes are padded with zero rows to whole tiles
+        const uint32_t at = PLANES == 2 || p0 + pos < a.n ? p0 + pos : a.n - 1u; // split planes are padded to whole tiles
+        x_src[q] = plane + (uint64_t)at * a.plane_stride;
     }
     // code staging: WQ loads per stage; load q covers the 16 rows of group WQ * w + q; lane l brings row
     // 16 * group + l / 4 and its codes 16 * (l % 4) .. + 15, which become the row's bf16 chunks
@@ -1105,7 +1121,7 @@ template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q
             for (int mt = 0; mt < MT; ++mt) {
                 const uint32_t at = x_at[mt] + 8u * ((4u * kb + kg) ^ x_sw[mt]);
                 xh[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][0][at]));
-                xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][1][at]));
+                if constexpr (PLANES == 2) xl[mt] = as_bf16x8(*(const uint4 *)(&s_x[buf][PLANES - 1][at]));
             }
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
@@ -1114,8 +1130,10 @@ template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q
                 floatx4 acc[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh[mt], wb, zero4, 0, 0, 0);
+                if constexpr (PLANES == 2) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
+                    for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl[mt], wb, acc[mt], 0, 0, 0);
+                }
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
@@ -1159,6 +1177,11 @@ template <int WAVES> __device__ __forceinline__ void q8_tiled_body(const lng_k_q
 
 extern "C" __global__ __launch_bounds__(512) void lng_q8_tiled(lng_k_q8 a) {
     q8_tiled_body<8>(a);
+}
+
+// positions already in bf16: one plane, half the matrix instructions, no split kernel before it
+extern "C" __global__ __launch_bounds__(512) void lng_q8_tiled_bf16(lng_k_q8 a) {
+    q8_tiled_body<8, 1>(a);
 }
 
 // Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).

@@ -76,6 +76,40 @@ def test_product_with_eight_position_tiles_or_more(gpu, rows, cols, n, kind):
     assert np.isnan(got[:-1, rows:]).all()           # 0xFF fill: gaps of y untouched
 
 
+@pytest.mark.parametrize("rows,cols,n", [(4096, 2880, 1), (512, 2880, 5), (37, 96, 13), (2880, 4096, 32), (2880, 4096, 31),
+                                         (320, 96, 1120), (2100, 64, 1030), (64, 32, 32), (5120, 2880, 512)])
+def test_product_of_bf16_positions(gpu, rows, cols, n):
+    """gemm_q8_0_bf16 (no counterpart in the reference): positions given in bf16, as a bf16 attention leaves them
+    for the output projection. Against the float64 product of the same bf16 values, the reference's bound for
+    its f32 kernels (glue.rs:171); strided x and y, gaps of y untouched."""
+    from tests.helpers import from_bf16_bits, to_bf16_bits
+    codes, bits, elements = q8_test_matrix(rows, cols, 60 + rows)
+    x_stride, y_stride = cols + 8, rows + 4
+    xb = np.full((n, x_stride), 0x7FC0, np.uint16)            # NaN between the rows of x: never read
+    xb[:, :cols] = to_bf16_bits(xorshift_values(19, n * cols).reshape(n, cols))
+    want = from_bf16_bits(xb[:, :cols]).astype(np.float64) @ elements.T
+    y_len = ((n - 1) * y_stride + rows) * 4
+    bufs = [gpu.upload(codes), gpu.upload(bits), gpu.upload(xb), gpu.buffer(y_len)]
+    bufs[3].fill(0xFF)
+    batch = gpu.batch(bufs)
+    try:
+        batch.gemm_q8_0_bf16((C.Slice(0, 0, codes.nbytes), C.Slice(1, 0, bits.nbytes)),
+                             C.Slice(2, 0, ((n - 1) * x_stride + cols) * 2), C.Slice(3, 0, y_len), rows, cols, n,
+                             (x_stride, y_stride))
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        raw = bufs[3].read(np.float32)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    got = np.full((n, y_stride), np.nan, np.float32)
+    got.reshape(-1)[:raw.size] = raw
+    assert not np.isnan(got[:, :rows]).any()
+    assert np.abs(got[:, :rows] - want).max() / np.abs(want).max() < 1e-5
+    assert np.isnan(got[:-1, rows:]).all()
+
+
 def test_strided_positions_and_untouched_gaps(gpu):
     rows, cols, n = 80, 96, 21
     codes, bits, elements = q8_test_matrix(rows, cols, 3)
