@@ -178,9 +178,15 @@ def test_refusals_of_the_reference(gpu):
     with pytest.raises(C.Dispatch):   # output in resident memory
         att = batch.attach(res)
         batch.gemm_q8_0(good[0], good[1], C.Slice(att.buffer, 0, 5 * 64 * 4), 64, 64, 5, (64, 64))
+    with pytest.raises(C.Dispatch):   # bf16 positions: rows of x must stay on 16-byte boundaries (stride % 8)
+        batch.gemm_q8_0_bf16(good[0], s(2, (4 * 68 + 64) * 2), good[2], 64, 64, 5, (68, 64))
+    with pytest.raises(C.Dispatch):   # bf16 positions: x of the f32 length
+        batch.gemm_q8_0_bf16(good[0], good[1], good[2], 64, 64, 5, (64, 64))
     assert batch.dispatches() == 0
     batch.gemm_q8_0(*good)
     assert batch.dispatches() == 1
+    batch.gemm_q8_0_bf16(good[0], s(2, 5 * 64 * 2), good[2], 64, 64, 5, (64, 64))
+    assert batch.dispatches() == 2
     batch.drop()
     for b in bufs:
         b.free()
