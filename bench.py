@@ -172,10 +172,34 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
     many = sorted(go(burst) for _ in range(max(steps, 5)))
     for b in bufs:
         b.free()
+    # the same query over f32 caches (the reference's own element type; not the metric's): lng_decode_f32_d64
+    qf, of = gpu.buffer(2 * QO), gpu.buffer(2 * QO)
+    kf, vf = gpu.buffer(ctx * 2 * ROW), gpu.buffer(ctx * 2 * ROW)
+    for i, b in enumerate((qf, kf, vf)):
+        bb = gpu.batch([b])
+        bb.fill_synthetic(C.Slice(0, 0, b.len), C.F32, 10 + i, 0.5, 0)
+        bb.run()
+        bb.drop()
+    sinks32 = gpu.upload(np.random.default_rng(2).standard_normal(H).astype(np.float32))
+
+    def go32():
+        batch = gpu.batch([qf, kf, vf, of, sinks32])
+        batch.attention_grouped_with_sinks((C.Slice(0, 0, 2 * QO), C.Slice(1, 0, ctx * 2 * ROW), C.Slice(2, 0, ctx * 2 * ROW)),
+                                           C.Slice(4, 0, H * 4), C.Slice(3, 0, 2 * QO), shape, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(5):
+        go32()
+    f32_us = sorted(go32() for _ in range(max(steps, 20)))[max(steps, 20) // 2] * 1e6
+    for b in (qf, of, kf, vf, sinks32):
+        b.free()
     nbytes = decode_bytes(ctx, C.FULL)
     g1, w1 = one[len(one) // 2]
     gb, wb = many[len(many) // 2]
     return {"workload": "C2 decode, 1 query, 4096 cached positions, full-causal", "bytes": nbytes,
+            "f32_caches_single_launch_gpu_us": f32_us,
             "single_launch_gpu_us": g1 * 1e6, "single_launch_wall_us": w1 * 1e6,
             "single_launch_gbs": nbytes / g1 / 1e9 if g1 > 0 else None,
             "burst": burst, "burst_gpu_us_per_launch": gb / burst * 1e6,

@@ -86,7 +86,7 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
+                  decode_merge = nullptr, decode_f32_d64 = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
                   q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr, q8_tiled_bf16 = nullptr, rmsnorm_rows = nullptr;
     std::string name;
@@ -413,7 +413,9 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     lng_gpu *g = b->gpu;
     const uint32_t group = a.heads / a.kv_heads;
     const bool fast = a.dtype == LNG_BF16 && a.dim == 64 && group <= 16 && aligned16;
-    if (!fast) {
+    // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the VALU
+    const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 8 && aligned16 && !getenv("LNG_F32_GENERIC");
+    if (!fast && !fast_f32) {
         Cmd c;
         c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;
         c.name = a.dtype == LNG_BF16 ? "lng_attn_generic_bf16" : "lng_attn_generic_f32";
@@ -432,12 +434,12 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         a.partial_o = g->scratch_o;
         a.partial_ml = g->scratch_ml;
         a.tickets = g->tickets;
-        // Small grids merge inside the kernel; large ones with a second dispatch.
-        a.fused = (uint64_t)plan.n_chunks * n_rows * a.kv_heads <= 4ull * g->cus ? 1u : 0u;
+        // Small grids merge inside the kernel; large ones with a second dispatch (the f32 kernel always).
+        a.fused = fast && (uint64_t)plan.n_chunks * n_rows * a.kv_heads <= 4ull * g->cus ? 1u : 0u;
     }
     Cmd c;
-    c.fn = g->decode_bf16_d64;
-    c.name = "lng_decode_bf16_d64";
+    c.fn = fast ? g->decode_bf16_d64 : g->decode_f32_d64;
+    c.name = fast ? "lng_decode_bf16_d64" : "lng_decode_f32_d64";
     c.grid[0] = plan.n_chunks;
     c.grid[1] = (unsigned)(n_rows * a.kv_heads);
     c.block = 256;
@@ -626,6 +628,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_attn_generic_bf16", &g->generic_bf16, true},
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
         {"lng_decode_merge", &g->decode_merge, true},
+        {"lng_decode_f32_d64", &g->decode_f32_d64, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_prefill_merge", &g->prefill_merge, true},

@@ -331,8 +331,13 @@ __device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_ro
             o3 += x3 * s_w[h][c + 3];
         }
         for (; c < row_chunks; ++c) o0 += load_partial<COHERENT>(po + c * step) * s_w[h][c];
-        uint16_t *op = (uint16_t *)(a.out + it.out_offset) + ((uint64_t)g * group + h) * 64u + d;
-        *op = f32_to_bf16_bits(((o0 + o1) + (o2 + o3)) / s_z[h]);
+        const float res = ((o0 + o1) + (o2 + o3)) / s_z[h];
+        const uint64_t at = ((uint64_t)g * group + h) * 64u + d;
+        if (a.dtype == LNG_F32) {
+            ((float *)(a.out + it.out_offset))[at] = res;
+        } else {
+            ((uint16_t *)(a.out + it.out_offset))[at] = f32_to_bf16_bits(res);
+        }
     }
 }
 
@@ -537,6 +542,145 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
     if (threadIdx.x == 0) __hip_atomic_store(&a.tickets[blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
     merge_chunks<true>(a, it, g, group, row_chunks);
+}
+
+// =============================================================================================
+// Decode kernel, f32 (the reference's own element type), head width 64, up to 8 query heads per
+// kv head: the bf16 kernel's grid, chunks and partials, on the VALU. A wavefront takes 8
+// positions per turn: lane = (position l / 8, dims 8 * (l % 8) ..): two 16-byte loads of the K
+// row and two of the V row, every head's partial dot product over the lane's 8 dims, summed over
+// the 8 lanes of a position with data-parallel primitives; block maximum over the 8 positions
+// (row rotation by 8, the two lane swaps); accurate expf; the lane keeps its own position stream's
+// sum and 8 heads x 8 dims of output, reduced over positions once at the end. K and V rows are
+// read once for all heads of the group, as in the bf16 kernel; the generic kernel reads them once
+// per head, a row per turn.
+// =============================================================================================
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float sum_over_dim_lanes(float x) { // lanes that differ in bits 0..2
+    x += dpp_f32<0xB1>(x);  // quad_perm [1,0,3,2]
+    x += dpp_f32<0x4E>(x);  // quad_perm [2,3,0,1]
+    x += dpp_f32<0x141>(x); // row_half_mirror: the other quad of the 8 (every lane of a quad holds its sum)
+    return x;
+}
+template <bool MAX> __device__ __forceinline__ float over_position_lanes(float x) { // lanes that differ in bits 3..5
+    const float r = dpp_f32<0x128>(x); // row_ror:8
+    x = MAX ? fmaxf(x, r) : x + r;
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = MAX ? fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])) : __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return MAX ? fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1])) : __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn a) {
+    __shared__ float s_m[4][8];
+    __shared__ float s_l[4][8];
+    __shared__ float s_o[4][8][64];
+    const uint32_t row = blockIdx.y / a.kv_heads;
+    const uint32_t g = blockIdx.y % a.kv_heads;
+    const lng_k_row it = row_of(a, row);
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+    const uint64_t base = first & ~(uint64_t)31;
+    const uint64_t c0 = base + (uint64_t)blockIdx.x * a.chunk;
+    if (c0 > last) return; // this row has fewer chunks than the longest one
+    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t u = lane >> 3, d8 = lane & 7u;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint64_t row_floats = (uint64_t)a.kv_heads * 64u;
+    const float *kb = (const float *)(a.k + it.k_offset) + (uint64_t)g * 64u + 8u * d8;
+    const float *vb = (const float *)(a.v + it.v_offset) + (uint64_t)g * 64u + 8u * d8;
+
+    float qv[8][8], acc[8][8], l[8], m[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+        const float *qp = (const float *)(a.q + it.q_offset) + ((uint64_t)g * group + h) * 64u + 8u * d8;
+        float4 q0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), q1 = q0;
+        if ((uint32_t)h < group) {
+            q0 = *(const float4 *)qp;
+            q1 = *(const float4 *)(qp + 4);
+        }
+        qv[h][0] = q0.x; qv[h][1] = q0.y; qv[h][2] = q0.z; qv[h][3] = q0.w;
+        qv[h][4] = q1.x; qv[h][5] = q1.y; qv[h][6] = q1.z; qv[h][7] = q1.w;
+        l[h] = 0.0f;
+        m[h] = LNG_NEG_INF;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
+    }
+    for (uint64_t pb = c0 + 8u * wave; pb < c1; pb += 32u) {
+        const uint64_t p = pb + u;
+        const bool seen = p >= first && p < c1;
+        const uint64_t pc = p < first ? first : (p > last ? last : p); // a row that exists, whatever p is
+        const uint64_t r = pc % it.slots;
+        const float4 k0 = *(const float4 *)(kb + r * row_floats), k1 = *(const float4 *)(kb + r * row_floats + 4);
+        const float4 v0 = *(const float4 *)(vb + r * row_floats), v1 = *(const float4 *)(vb + r * row_floats + 4);
+        const float kx[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+        const float vx[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+            if ((uint32_t)h >= group) break; // the same for every lane
+            float part = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) part += qv[h][e] * kx[e];
+            const float sc = seen ? sum_over_dim_lanes(part) * a.scale : LNG_NEG_INF;
+            const float next = fmaxf(m[h], over_position_lanes<true>(sc));
+            if (next == LNG_NEG_INF) continue;   // nothing seen yet (the same for every lane)
+            const float keep = m[h] == LNG_NEG_INF ? 0.0f : expf(m[h] - next);
+            const float w = sc == LNG_NEG_INF ? 0.0f : expf(sc - next);
+            l[h] = l[h] * keep + w;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] = acc[h][e] * keep + w * vx[e];
+            m[h] = next;
+        }
+    }
+    // ---- over the positions of the wavefront, then over the four wavefronts -----------------------
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+        if ((uint32_t)h >= group) break;
+        const float lsum = over_position_lanes<false>(l[h]);
+        if (lane == 0) {
+            s_m[wave][h] = m[h];
+            s_l[wave][h] = lsum;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float o = over_position_lanes<false>(acc[h][e]);
+            if (u == 0) s_o[wave][h][8u * d8 + e] = o;
+        }
+    }
+    __syncthreads();
+    for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
+        const uint32_t h = idx >> 6;
+        const uint32_t d = idx & 63u;
+        float top = LNG_NEG_INF;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) top = fmaxf(top, s_m[w][h]);
+        float sum = 0.0f, o = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : expf(s_m[w][h] - top);
+            sum += s_l[w][h] * wt;
+            o += s_o[w][h][d] * wt;
+        }
+        if (row_chunks == 1) {
+            const uint32_t head = g * group + h;
+            const float sink = it.sinks_offset != LNG_NO_SINKS ? ((const float *)(a.sinks + it.sinks_offset))[head] : LNG_NEG_INF;
+            const float all = fmaxf(top, sink);
+            const float keep = top == LNG_NEG_INF ? 0.0f : expf(top - all);
+            const float z = sum * keep + (sink == LNG_NEG_INF ? 0.0f : expf(sink - all));
+            ((float *)(a.out + it.out_offset))[(uint64_t)head * 64u + d] = o * keep / z;
+        } else { // lng_decode_merge follows; it works in the log2 domain
+            const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
+            a.partial_o[slot * 64u + d] = o;
+            if (d == 0) {
+                a.partial_ml[slot * 2u] = top * LNG_LOG2E;
+                a.partial_ml[slot * 2u + 1u] = sum;
+            }
+        }
+    }
 }
 
 // The same merge as its own dispatch, for large grids: there a workgroup that waits for its
@@ -1651,6 +1795,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     a.partial_o = p.partial_o;
     a.partial_ml = p.partial_ml;
     a.n_chunks = p.splits;
+    a.dtype = LNG_BF16;
     lng_k_row it{};
     it.out_offset = (uint64_t)row * p.heads * 64u * 2u;
     it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;

@@ -488,3 +488,36 @@ def test_decode_bf16_one_long_row(gpu, start, window, slots):
     # the oracle reads position p from row p % slots of the same ring
     want = oracle.attention_bf16(q, kr, vr, sinks, start, window=window, slots=slots, scale=0.125, threads=THREADS)
     assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
+# ---- f32 caches (the reference's own element type) at the gpt-oss head width: lng_decode_f32_d64 ----
+@pytest.mark.parametrize("t,start,window,slots,heads,kv_heads", [
+    (1, 0, FULL, 1, 64, 8), (1, 36, FULL, 37, 64, 8), (1, 4095, FULL, 4096, 64, 8), (1, 5000, 128, 200, 64, 8),
+    (1, 70000, FULL, 70001, 64, 8), (1, 200000, 100000, 150016, 16, 2), (3, 2000, FULL, 2003, 8, 8), (7, 900, 33, 41, 6, 2),
+    (31, 100, FULL, 131, 5, 1), (2, 9000, 1, 3, 64, 8), (5, 260, 300, 305, 24, 8),
+])
+def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_heads, monkeypatch):
+    """The row-by-row operator on f32 caches: every grouping up to 8 heads per kv head, one chunk and many
+    (merged by a second dispatch), rings that have wrapped, windows that start inside a tile, with and without
+    sinks; rows the operator must not read hold NaN (attention_grouped.rs:57). Within 1e-5 (relative to
+    1 + |x|) of the CPU reference, and the generic kernel (LNG_F32_GENERIC) agrees."""
+    end = start + t
+    rng = np.random.default_rng(start + t)
+    q = (rng.standard_normal((t, heads, 64)) * 0.7).astype(np.float32)
+    first = 0 if window == FULL else max(0, start + 1 - window)
+    kept = max(first, end - slots)
+    k = np.full((end, kv_heads, 64), np.nan, np.float32)
+    v = np.full((end, kv_heads, 64), np.nan, np.float32)
+    k[kept:] = (rng.standard_normal((end - kept, kv_heads, 64)) * 0.7).astype(np.float32)
+    v[kept:] = rng.standard_normal((end - kept, kv_heads, 64)).astype(np.float32)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    kr, vr = ring_layout(k, t, start, slots, False), ring_layout(v, t, start, slots, False)
+    kz, vz = np.nan_to_num(k), np.nan_to_num(v)     # the oracle multiplies unseen rows by zero weights
+    for sinks in (rng.standard_normal(heads).astype(np.float32), None):
+        want = oracle.attention_f32(q, kz, vz, sinks, start, window=window, slots=None, scale=0.125, threads=THREADS)
+        got = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
+        assert rel_error(got, want) <= F32_RTOL
+        monkeypatch.setenv("LNG_F32_GENERIC", "1")
+        generic = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
+        monkeypatch.delenv("LNG_F32_GENERIC")
+        assert rel_error(generic, want) <= F32_RTOL
