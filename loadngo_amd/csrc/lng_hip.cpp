@@ -474,6 +474,8 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         q_rows = (s.t + 31) / 32 * 32; // apple.rs:1386-1395
         kv_rows = s.slots < end ? s.slots : (end + 31) / 32 * 32;
     }
+    // (slots and rows x heads fit in u32; a row of all heads below 2^32 bytes keeps the byte counts inside 64 bits)
+    if (!fits_u32(s.heads * s.dim * es)) return fail(LNG_ERR_DISPATCH, "rows of %llu bytes do not fit in u32", (unsigned long long)(s.heads * s.dim * es));
     Operand oq, ok, ov, oo, os{};
     if (int rc = check_slice(b, "q", q, q_rows * s.heads * s.dim * es, es, &oq)) return rc;
     if (int rc = check_slice(b, "k", k, kv_rows * s.kv_heads * s.dim * es, es, &ok)) return rc;
@@ -1001,6 +1003,7 @@ extern "C" int lng_hip_attention_decode_batched(lng_batch *b, uint64_t q_buffer,
     if (!bq || !bk || !bv || !bo) return fail(LNG_ERR_DISPATCH, "no such buffer (batch has %zu)", b->buffers.size() + b->residents.size());
     if (out_buffer >= b->buffers.size()) return fail(LNG_ERR_DISPATCH, "output is in read-only resident memory");
     const uint64_t es = elem_size(dtype);
+    if (!fits_u32(heads) || !fits_u32(heads * dim * es)) return fail(LNG_ERR_DISPATCH, "rows of %llu x %llu elements do not fit in u32", (unsigned long long)heads, (unsigned long long)dim);
     bool any_sinks = false, aligned16 = true;
     for (size_t i = 0; i < n_items; ++i) {
         const lng_decode_item &it = items[i];
