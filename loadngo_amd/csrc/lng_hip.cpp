@@ -86,7 +86,7 @@ struct lng_gpu {
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, decode_f32_d64 = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
+                  decode_merge = nullptr, decode_f32_d64 = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
                   add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
                   q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr, q8_tiled_bf16 = nullptr, rmsnorm_rows = nullptr;
     std::string name;
@@ -495,8 +495,11 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     // Measured break-even on 64/8 heads: rows x visible keys of about 32 K (16 rows over 2,048 keys, 4 over 8,192).
     const uint64_t seen = std::min<uint64_t>(end, s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t);
     const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && s.t * seen >= 32768 && !getenv("LNG_PLAIN_ROW_BY_ROW");
-    if ((tiled || several_rows) && dtype == LNG_BF16 && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16) {
+    if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 &&
+        (dtype == LNG_BF16 || !getenv("LNG_F32_GENERIC"))) {
+        const bool f32 = dtype == LNG_F32;
         lng_k_prefill p{};
+        p.dtype = (uint32_t)dtype;
         p.q = (const char *)oq.buf->ptr + q.offset;
         p.k = (const char *)ok.buf->ptr + k.offset;
         p.v = (const char *)ov.buf->ptr + v.offset;
@@ -512,8 +515,9 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         // Two heads per wavefront (64 query rows per workgroup) for long causal runs; one head
         // per wavefront (32 rows, two workgroups per compute unit) when each query sees few keys
         // and the pass is bound by latency, not by the matrix pipe.
-        const bool narrow = p.window != LNG_WINDOW_FULL && p.window <= 1024;
-        const unsigned rows_per_wg = narrow ? 32 : 64;
+        // (the f32 kernel has one form: 32 rows, one head per wavefront; it is bound by the f32 matrix rate)
+        const bool narrow = !f32 && p.window != LNG_WINDOW_FULL && p.window <= 1024;
+        const unsigned rows_per_wg = narrow || f32 ? 32 : 64;
         p.q_tiles = (uint32_t)((s.t + rows_per_wg - 1) / rows_per_wg);
         p.scale = s.scale;
         // Few query tiles over many keys (a chunk of a long prompt, a handful of rows late in a long
@@ -539,8 +543,8 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             p.partial_ml = g->scratch_ml;
         }
         Cmd c;
-        c.fn = narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
-        c.name = narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
+        c.fn = f32 ? g->prefill_f32_d64 : narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
+        c.name = f32 ? "lng_prefill_f32_d64" : narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
         c.grid[0] = p.q_tiles * (unsigned)s.kv_heads * p.splits; // kv head fastest: one XCD's L2 per kv head
         c.block = 512;
         set_args(c, p);
@@ -633,6 +637,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_f32_d64", &g->decode_f32_d64, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
+        {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
         {"lng_prefill_merge", &g->prefill_merge, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},

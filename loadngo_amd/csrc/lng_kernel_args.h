@@ -56,6 +56,7 @@ typedef struct lng_k_prefill {
     uint32_t q_tiles;   /* ceil(t / rows per workgroup) */
     float scale;
     uint32_t splits;    /* workgroups that share one (query tile, kv head), each with a run of its key tiles; 1: none */
+    uint32_t dtype;     /* LNG_F32 / LNG_BF16: element type of q, k, v and out */
     float *partial_o;   /* splits > 1: [row][kv_head][split][group][dim] f32, unnormalised */
     float *partial_ml;  /* splits > 1: [row][kv_head][split][group][2] f32 (max in the log2 domain, sum) */
 } lng_k_prefill;

@@ -1737,6 +1737,215 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     prefill_body<1>(a);
 }
 
+// =============================================================================================
+// Prompt-pass kernel, f32 (the reference's own element type), head width 64, up to 8 query heads
+// per kv head: the bf16 kernel's plan on the f32 matrix instruction.
+//
+// A workgroup (8 wavefronts) takes 32 consecutive query positions and all query heads of one kv
+// head, one head per wavefront; K/V tiles of 64 keys go through LDS as f32. Per 32-key block
+//   S^T[key][query] = K . Q^T    32 x v_mfma_f32_32x32x2_f32: lane (query n, half hh) feeds dims
+//                                8j + 4hh + e of its key row (ds_read_b128) and of its query (registers)
+//   O^T[dim][query] += V^T . P^T 32 x the same instruction: lane (n, hh) holds the weights of keys
+//                                8a + 4hh + e, which is how the first product left them, and reads
+//                                V[that key][dim 32db + n] with ds_read_b32
+// so softmax state and output column are lane-local exactly as in the bf16 kernel, and the
+// arithmetic is f32 throughout (products are not rounded to a narrower type anywhere). The kernel
+// is bound by the f32 matrix rate (64 FLOP per clock and SIMD, a sixteenth of bf16).
+// =============================================================================================
+#define PF32_BM 32u
+#define PF32_KSTRIDE 68 // floats per LDS row of K: 16-byte reads of 16 consecutive rows cover all 64 banks
+#define PF32_VSTRIDE 72 // of V: the rows 4 apart that the two halves of a wavefront read fall 32 banks apart
+
+extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_f32_d64(lng_k_prefill a) {
+    __shared__ __attribute__((aligned(16))) float s_k[2][PF_BN * PF32_KSTRIDE];
+    __shared__ __attribute__((aligned(16))) float s_v[2][PF_BN * PF32_VSTRIDE];
+
+    const uint32_t g = blockIdx.x % a.kv_heads;
+    const uint32_t split = (blockIdx.x / a.kv_heads) % a.splits;
+    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads / a.splits;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n = lane & 31u; // query within the workgroup's block
+    const uint32_t hh = lane >> 5; // which of the two k slots of the matrix instruction
+
+    const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
+    const uint32_t q0 = qtile * PF32_BM;
+    const uint32_t rows_here = t - q0 < PF32_BM ? t - q0 : PF32_BM;
+    const uint32_t end = start + t;
+    const uint32_t pos_first = start + q0;
+    const uint32_t pos_last = pos_first + rows_here - 1;
+    const bool windowed = a.window != LNG_WINDOW_FULL;
+    const uint32_t window = windowed ? (uint32_t)a.window : 0u;
+    const uint32_t kfirst = (windowed && pos_first + 1 > window) ? pos_first + 1 - window : 0u;
+    const uint32_t tile0 = kfirst & ~(uint32_t)(PF_BN - 1);
+    const uint32_t all_tiles = (pos_last - tile0) / PF_BN + 1;
+    const bool partial = a.splits > 1u;
+    const uint32_t first_tile = (uint32_t)((uint64_t)all_tiles * split / a.splits);
+    const uint32_t n_tiles = (uint32_t)((uint64_t)all_tiles * (split + 1u) / a.splits);
+    const bool ring = a.slots < end;
+    const uint32_t slots = (uint32_t)a.slots;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * 256u;
+
+    const uint32_t my_row = q0 + n;
+    const uint32_t my_pos = start + my_row;
+    const bool row_ok = my_row < t;
+    const bool wave_active = wave < group; // the others only help loading tiles
+    const uint32_t head = g * group + (wave_active ? wave : 0u);
+    float4 qreg[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        qreg[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (row_ok) qreg[j] = *(const float4 *)(a.q + (((uint64_t)my_row * a.heads + head) * 64u + 8u * j + 4u * hh) * 4u);
+    }
+    const float sl2 = a.scale * LNG_LOG2E;
+    const bool sink_here = a.sinks && !partial;
+    float m = sink_here ? a.sinks[head] * LNG_LOG2E : LNG_NEG_INF;
+    float l = (sink_here && hh == 0) ? 1.0f : 0.0f;
+    floatx16 ot[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ot[db][i] = 0.0f;
+    }
+
+    // ---- tile loader: two 16-byte chunks of K and of V per thread (keys ld_key and ld_key + 32) ----
+    const uint32_t ld_key = tid >> 4;  // 0..31
+    const uint32_t ld_chunk = tid & 15u;
+    const char *kbase = a.k + (uint64_t)g * 256u + ld_chunk * 16u;
+    const char *vbase = a.v + (uint64_t)g * 256u + ld_chunk * 16u;
+    uint4 kr0, kr1, vr0, vr1; // plain scalars: arrays indexed inside the lambdas end up in scratch memory
+    auto fetch_row = [&](uint32_t p, uint4 &kr, uint4 &vr) {
+        p = p > pos_last ? pos_last : p; // rows outside [first visible, last] are masked, and may not exist
+        p = p < kfirst ? kfirst : p;
+        const uint32_t row = ring ? p % slots : p;
+        kr = *(const uint4 *)(kbase + (uint64_t)row * row_bytes);
+        vr = *(const uint4 *)(vbase + (uint64_t)row * row_bytes);
+    };
+    auto fetch = [&](uint32_t tile) {
+        fetch_row(tile0 + tile * PF_BN + ld_key, kr0, vr0);
+        fetch_row(tile0 + tile * PF_BN + 32u + ld_key, kr1, vr1);
+    };
+    auto stash = [&](uint32_t buf) {
+        *(uint4 *)(&s_k[buf][ld_key * PF32_KSTRIDE + ld_chunk * 4u]) = kr0;
+        *(uint4 *)(&s_v[buf][ld_key * PF32_VSTRIDE + ld_chunk * 4u]) = vr0;
+        *(uint4 *)(&s_k[buf][(32u + ld_key) * PF32_KSTRIDE + ld_chunk * 4u]) = kr1;
+        *(uint4 *)(&s_v[buf][(32u + ld_key) * PF32_VSTRIDE + ld_chunk * 4u]) = vr1;
+    };
+    if (first_tile < n_tiles) {
+        fetch(first_tile);
+        stash(first_tile & 1u);
+    }
+    __syncthreads();
+
+    const uint32_t k_lane_off = n * PF32_KSTRIDE + 4u * hh; // + kb*32*KSTRIDE + 8j
+    const uint32_t v_lane_off = 4u * hh * PF32_VSTRIDE + n; // + (kb*32 + 8a + e)*VSTRIDE + 32db
+
+    auto step = [&](auto mask_tag, uint32_t tile) {
+        constexpr bool MASK = decltype(mask_tag)::value;
+        const uint32_t buf = tile & 1u;
+        if (tile + 1 < n_tiles) fetch(tile + 1);
+        if (wave_active) {
+            const uint32_t kt0 = tile0 + tile * PF_BN;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if constexpr (MASK) { // a block no query of the workgroup sees
+                    const uint32_t b0 = kt0 + 32u * kb;
+                    if (b0 > pos_last || b0 + 31u < kfirst) continue;
+                }
+                floatx16 st;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) st[i] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float4 ka = *(const float4 *)(&s_k[buf][k_lane_off + kb * 32 * PF32_KSTRIDE + 8 * j]);
+                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.x, qreg[j].x, st, 0, 0, 0);
+                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.y, qreg[j].y, st, 0, 0, 0);
+                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.z, qreg[j].z, st, 0, 0, 0);
+                    st = __builtin_amdgcn_mfma_f32_32x32x2f32(ka.w, qreg[j].w, st, 0, 0, 0);
+                }
+                if constexpr (MASK) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const uint32_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
+                        const bool vis = kp <= my_pos && (!windowed || kp + window > my_pos);
+                        st[i] = vis ? st[i] : LNG_NEG_INF;
+                    }
+                }
+                // online softmax, one query per lane; the maximum moves only when it grows by PF_TAU
+                float tmax = LNG_NEG_INF;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[i]);
+                tmax = other_half_max(tmax) * sl2;
+                const float m_new = tmax > m + PF_TAU ? tmax : m;
+                const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+                    const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+                    l *= alpha;
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) ot[db][i] *= alpha;
+                    }
+                    m = m_new;
+                }
+                float psum = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    st[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[i], sl2, -m_safe));
+                    psum += st[i];
+                }
+                l += psum;
+                // O^T += V^T . P^T: step i of the 16 multiplies keys 8(i>>2) + 4hh + (i&3)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float *vp = &s_v[buf][v_lane_off + (kb * 32 + 8 * (i >> 2) + (i & 3)) * PF32_VSTRIDE];
+                    ot[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[0], st[i], ot[0], 0, 0, 0);
+                    ot[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(vp[32], st[i], ot[1], 0, 0, 0);
+                }
+            }
+        }
+        if (tile + 1 < n_tiles) stash(buf ^ 1u);
+        __syncthreads();
+    };
+    auto edge = [&](uint32_t tile) {
+        const uint32_t kt0 = tile0 + tile * PF_BN;
+        return kt0 + (PF_BN - 1) > pos_first || (windowed && kt0 + window < pos_first + PF32_BM);
+    };
+    uint32_t tile = first_tile;
+    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tile);   // window edge
+    for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tile); // interior
+    for (; tile < n_tiles; ++tile) step(std::true_type{}, tile);                 // diagonal
+
+    if (!wave_active || !row_ok) return;
+    const float total = l + __shfl_xor(l, 32, 64);
+    if (partial) { // (max, sum, unnormalised output) for lng_prefill_merge, which also adds the sink
+        const uint64_t slot = (((uint64_t)my_row * a.kv_heads + g) * a.splits + split) * group + (head - g * group);
+        float *po = a.partial_o + slot * 64u;
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                *(float4 *)(po + 32 * db + 8 * blk + 4 * hh) = make_float4(ot[db][4 * blk + 0], ot[db][4 * blk + 1],
+                                                                           ot[db][4 * blk + 2], ot[db][4 * blk + 3]);
+            }
+        }
+        if (hh == 0) *(float2 *)(a.partial_ml + slot * 2u) = make_float2(m, total);
+        return;
+    }
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    float *op = (float *)a.out + ((uint64_t)my_row * a.heads + head) * 64u;
+#pragma unroll
+    for (int db = 0; db < 2; ++db) {
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            *(float4 *)(op + 32 * db + 8 * blk + 4 * hh) = make_float4(ot[db][4 * blk + 0] * inv, ot[db][4 * blk + 1] * inv,
+                                                                       ot[db][4 * blk + 2] * inv, ot[db][4 * blk + 3] * inv);
+        }
+    }
+}
+
 // Combines the splits of a prompt pass; the sink joins here. Up to eight splits (the usual case: one
 // workgroup per compute unit needs few): a thread per (row, head, four dims) requests its splits' partial
 // outputs at once, works out the weights from the (max, sum) pairs itself - the 16 threads of a head all
@@ -1779,6 +1988,10 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
                 sum.w += o[c].w * w;
             }
         }
+        if (p.dtype == LNG_F32) {
+            *(float4 *)((float *)p.out + pair * 64u + d4) = make_float4(sum.x / z, sum.y / z, sum.z / z, sum.w / z);
+            return;
+        }
         ushort4 r;
         r.x = f32_to_bf16_bits(sum.x / z);
         r.y = f32_to_bf16_bits(sum.y / z);
@@ -1795,9 +2008,9 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     a.partial_o = p.partial_o;
     a.partial_ml = p.partial_ml;
     a.n_chunks = p.splits;
-    a.dtype = LNG_BF16;
+    a.dtype = p.dtype;
     lng_k_row it{};
-    it.out_offset = (uint64_t)row * p.heads * 64u * 2u;
+    it.out_offset = (uint64_t)row * p.heads * 64u * (p.dtype == LNG_F32 ? 4u : 2u);
     it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;
     merge_chunks<false>(a, it, g, group, p.splits);
 }

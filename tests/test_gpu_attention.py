@@ -521,3 +521,55 @@ def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_hea
         generic = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
         monkeypatch.delenv("LNG_F32_GENERIC")
         assert rel_error(generic, want) <= F32_RTOL
+
+
+# ---- prompt passes in f32 (f32 matrix-instruction kernel) -------------------------------------
+@pytest.mark.parametrize("t,start,window,slots,heads,kv_heads,forced", [
+    (64, 0, FULL, 64, 64, 8, None), (33, 5, FULL, 64, 64, 8, None), (100, 37, FULL, 160, 16, 2, None), (65, 0, 1, 96, 64, 8, None),
+    (128, 64, 64, 192, 64, 8, None), (200, 1400, 1024, 1536, 16, 2, None), (512, 2600, 128, 640, 8, 8, None),
+    (97, 31, 40, 128, 16, 4, None), (130, 1000, 128, 320, 6, 2, None), (77, 700, FULL, 4096, 10, 2, None),
+    (40, 97, 7, 64, 4, 1, None), (256, 0, 100, 256, 32, 8, None), (128, 3968, FULL, 4096, 64, 8, None),
+    (96, 1952, FULL, 2048, 64, 8, "7"), (64, 960, FULL, 1024, 24, 8, "64"), (96, 0, FULL, 96, 64, 8, "5"),
+    (160, 2000, 1500, 2176, 16, 2, "3"),
+])
+def test_prefill_f32_matches_the_cpu_reference(gpu, t, start, window, slots, heads, kv_heads, forced, monkeypatch):
+    """The tiled operator on f32 operands at head width 64 (the reference's own prompt pass, gpu.rs:760-806):
+    within 1e-5 (relative to 1 + |x|) of the CPU reference, with and without sinks, rings, windows, ragged
+    last tiles, groupings from 1 to 8, keys split between workgroups (by the library's own choice and forced
+    through LNG_PREFILL_SPLITS); the generic kernel (LNG_F32_GENERIC) agrees."""
+    if forced:
+        monkeypatch.setenv("LNG_PREFILL_SPLITS", forced)
+    end = start + t
+    q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    kr, vr = ring_layout(k, t, start, slots, True), ring_layout(v, t, start, slots, True)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    for sk in (sinks, None):
+        want = oracle.attention_f32(q, k, v, sk, start, window=window, slots=None, scale=0.125, threads=THREADS)
+        got = run_attention(gpu, q, kr, vr, sk, shape, True, C.F32)
+        assert rel_error(got, want) <= F32_RTOL
+    monkeypatch.setenv("LNG_F32_GENERIC", "1")
+    generic = run_attention(gpu, q, kr, vr, None, shape, True, C.F32)
+    assert rel_error(generic, want) <= F32_RTOL
+
+
+@pytest.mark.parametrize("t,start,window,slots", [(8, 5000, FULL, 5008), (31, 3000, 2000, 2031), (16, 2100, FULL, 2116),
+                                                  (5, 7000, 6999, 7004)])
+def test_several_f32_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, monkeypatch):
+    """attention_grouped on f32 caches with a handful of rows over thousands of keys goes through the f32
+    prompt-pass kernel; same results as row by row (LNG_PLAIN_ROW_BY_ROW) and as the CPU reference; cache rows
+    outside [first visible, last] hold NaN, and rings need not be multiples of 32 rows."""
+    heads, kv_heads = 64, 8
+    end = start + t
+    q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    kr, vr = ring_layout(k, t, start, slots, False), ring_layout(v, t, start, slots, False)
+    first = 0 if window == FULL else max(0, start + 1 - window)
+    if slots >= end:
+        kr[:first] = np.nan
+        vr[:first] = np.nan
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    want = oracle.attention_f32(q, k, v, sinks, start, window=window, slots=None, scale=0.125, threads=THREADS)
+    got = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
+    assert rel_error(got, want) <= F32_RTOL
+    monkeypatch.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
+    rows = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
+    assert rel_error(rows, want) <= F32_RTOL
