@@ -37,6 +37,7 @@ ROW = G * D * 2          # bytes of one cached position of K (or V) in bf16
 QO = H * D * 2           # bytes of one query (or output) row
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X f32 matrix
 # HBM bytes per launch of the decode kernel on the default stack workload, from rocprofv3 FETCH_SIZE
 # and WRITE_SIZE scaled by a 1 GiB copy (profiles/decode_stack_c5_hbm_traffic.md).
 STACK_TRAFFIC_PER_LAUNCH = 2155619789
@@ -313,6 +314,32 @@ def run_prefill(gpu, steps, warmup, t=8192):
     res["full_in_chunks_of_512"] = {"calls": t // chunk, "gpu_ms": g * 1e3, "tflops": 4 * D * H * pairs / g / 1e12,
                                     "mfma_frac": 4 * D * H * pairs / g / 1e12 / MFMA_BF16_PEAK_TFLOPS}
     for b in bufs:
+        b.free()
+    # the same pass on f32 operands (the reference's element type): lng_prefill_f32_d64, bound by the f32 matrix rate
+    q, out = gpu.buffer(t * QO * 2), gpu.buffer(t * QO * 2)
+    k, v = gpu.buffer(t * ROW * 2), gpu.buffer(t * ROW * 2)
+    for i, b in enumerate((q, k, v)):
+        batch = gpu.batch([b])
+        batch.fill_synthetic(C.Slice(0, 0, b.len), C.F32, 30 + i, 0.5, 0)
+        batch.run()
+        batch.drop()
+    shape = C.GroupedShape(t, 0, H, G, D, C.FULL, t, SCALE)
+    sinks = gpu.upload(np.random.default_rng(4).standard_normal(H).astype(np.float32))
+
+    def go32():
+        batch = gpu.batch([q, k, v, out, sinks])
+        batch.attention_grouped_tiled_with_sinks((C.Slice(0, 0, q.len), C.Slice(1, 0, k.len), C.Slice(2, 0, v.len)),
+                                                 C.Slice(4, 0, H * 4), C.Slice(3, 0, out.len), shape, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    go32()
+    runs = sorted(go32() for _ in range(5))
+    g = runs[len(runs) // 2]
+    res["full_f32"] = {"gpu_ms": g * 1e3, "tflops": 4 * D * H * pairs / g / 1e12,
+                       "mfma_f32_frac": 4 * D * H * pairs / g / 1e12 / MFMA_F32_PEAK_TFLOPS}
+    for b in (q, out, k, v, sinks):
         b.free()
     res["workload"] = "C4 causal prefill, 8192 positions, 64 q / 8 kv heads, head_dim 64, bf16"
     return res
