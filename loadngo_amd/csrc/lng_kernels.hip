@@ -550,7 +550,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
 // positions per turn: lane = (position l / 8, dims 8 * (l % 8) ..): two 16-byte loads of the K
 // row and two of the V row, every head's partial dot product over the lane's 8 dims, summed over
 // the 8 lanes of a position with data-parallel primitives; block maximum over the 8 positions
-// (row rotation by 8, the two lane swaps); accurate expf; the lane keeps its own position stream's
+// (row rotation by 8, the two lane swaps); exponentials in the log2 domain (v_exp_f32, whose error
+// of one unit in the last place is far inside the 1e-5 bar); the lane keeps its own position stream's
 // sum and 8 heads x 8 dims of output, reduced over positions once at the end. K and V rows are
 // read once for all heads of the group, as in the bf16 kernel; the generic kernel reads them once
 // per head, a row per turn.
@@ -594,6 +595,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn 
     const float *kb = (const float *)(a.k + it.k_offset) + (uint64_t)g * 64u + 8u * d8;
     const float *vb = (const float *)(a.v + it.v_offset) + (uint64_t)g * 64u + 8u * d8;
 
+    const float sl2 = a.scale * LNG_LOG2E; // scores and maxima live in the log2 domain
     float qv[8][8], acc[8][8], l[8], m[8];
 #pragma unroll
     for (int h = 0; h < 8; ++h) {
@@ -610,13 +612,23 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn 
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
     }
+    // the rows of the next turn are requested before the arithmetic of this one
+    float4 k0, k1, v0, v1, nk0, nk1, nv0, nv1;
+    auto fetch = [&](uint64_t pb, float4 &a0, float4 &a1, float4 &b0, float4 &b1) {
+        const uint64_t p = pb + u;
+        const uint64_t pc = p < first ? first : (p > last ? last : p); // a row that exists, whatever p is
+        const uint64_t r = pc % it.slots;
+        a0 = *(const float4 *)(kb + r * row_floats);
+        a1 = *(const float4 *)(kb + r * row_floats + 4);
+        b0 = *(const float4 *)(vb + r * row_floats);
+        b1 = *(const float4 *)(vb + r * row_floats + 4);
+    };
+    if (c0 + 8u * wave < c1) fetch(c0 + 8u * wave, nk0, nk1, nv0, nv1);
     for (uint64_t pb = c0 + 8u * wave; pb < c1; pb += 32u) {
         const uint64_t p = pb + u;
         const bool seen = p >= first && p < c1;
-        const uint64_t pc = p < first ? first : (p > last ? last : p); // a row that exists, whatever p is
-        const uint64_t r = pc % it.slots;
-        const float4 k0 = *(const float4 *)(kb + r * row_floats), k1 = *(const float4 *)(kb + r * row_floats + 4);
-        const float4 v0 = *(const float4 *)(vb + r * row_floats), v1 = *(const float4 *)(vb + r * row_floats + 4);
+        k0 = nk0; k1 = nk1; v0 = nv0; v1 = nv1;
+        if (pb + 32u < c1) fetch(pb + 32u, nk0, nk1, nv0, nv1);
         const float kx[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
         const float vx[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
@@ -625,15 +637,20 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn 
             float part = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) part += qv[h][e] * kx[e];
-            const float sc = seen ? sum_over_dim_lanes(part) * a.scale : LNG_NEG_INF;
+            const float sc = seen ? sum_over_dim_lanes(part) * sl2 : LNG_NEG_INF; // log2 domain
             const float next = fmaxf(m[h], over_position_lanes<true>(sc));
             if (next == LNG_NEG_INF) continue;   // nothing seen yet (the same for every lane)
-            const float keep = m[h] == LNG_NEG_INF ? 0.0f : expf(m[h] - next);
-            const float w = sc == LNG_NEG_INF ? 0.0f : expf(sc - next);
-            l[h] = l[h] * keep + w;
+            if (next != m[h]) {                  // the maximum moved (the same for every lane): rescale
+                const float keep = m[h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(m[h] - next);
+                l[h] *= keep;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] = acc[h][e] * keep + w * vx[e];
-            m[h] = next;
+                for (int e = 0; e < 8; ++e) acc[h][e] *= keep;
+                m[h] = next;
+            }
+            const float w = sc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sc - next);
+            l[h] += w;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e] += w * vx[e];
         }
     }
     // ---- over the positions of the wavefront, then over the four wavefronts -----------------------
@@ -661,22 +678,24 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn 
         float sum = 0.0f, o = 0.0f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : expf(s_m[w][h] - top);
+            const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(s_m[w][h] - top);
             sum += s_l[w][h] * wt;
             o += s_o[w][h][d] * wt;
         }
         if (row_chunks == 1) {
             const uint32_t head = g * group + h;
-            const float sink = it.sinks_offset != LNG_NO_SINKS ? ((const float *)(a.sinks + it.sinks_offset))[head] : LNG_NEG_INF;
+            const float sink = it.sinks_offset != LNG_NO_SINKS
+                                   ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                   : LNG_NEG_INF;
             const float all = fmaxf(top, sink);
-            const float keep = top == LNG_NEG_INF ? 0.0f : expf(top - all);
-            const float z = sum * keep + (sink == LNG_NEG_INF ? 0.0f : expf(sink - all));
+            const float keep = top == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(top - all);
+            const float z = sum * keep + (sink == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink - all));
             ((float *)(a.out + it.out_offset))[(uint64_t)head * 64u + d] = o * keep / z;
-        } else { // lng_decode_merge follows; it works in the log2 domain
+        } else { // lng_decode_merge follows
             const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
             a.partial_o[slot * 64u + d] = o;
             if (d == 0) {
-                a.partial_ml[slot * 2u] = top * LNG_LOG2E;
+                a.partial_ml[slot * 2u] = top;
                 a.partial_ml[slot * 2u + 1u] = sum;
             }
         }
