@@ -413,8 +413,12 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     lng_gpu *g = b->gpu;
     const uint32_t group = a.heads / a.kv_heads;
     const bool fast = a.dtype == LNG_BF16 && a.dim == 64 && group <= 16 && aligned16;
-    // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the VALU
-    const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 8 && aligned16 && !getenv("LNG_F32_GENERIC");
+    // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the f32 matrix instruction
+    // (that kernel counts positions in 32 bits and looks up to 63 past the last one)
+    uint64_t latest = t_uniform ? host_rows[0].start + t_uniform - 1 : 0;
+    for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
+    const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 16 && aligned16 && latest < 0xffffff00ull &&
+                          !getenv("LNG_F32_GENERIC");
     if (!fast && !fast_f32) {
         Cmd c;
         c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;

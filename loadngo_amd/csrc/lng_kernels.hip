@@ -545,127 +545,173 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
 }
 
 // =============================================================================================
-// Decode kernel, f32 (the reference's own element type), head width 64, up to 8 query heads per
-// kv head: the bf16 kernel's grid, chunks and partials, on the VALU. A wavefront takes 8
-// positions per turn: lane = (position l / 8, dims 8 * (l % 8) ..): two 16-byte loads of the K
-// row and two of the V row, every head's partial dot product over the lane's 8 dims, summed over
-// the 8 lanes of a position with data-parallel primitives; block maximum over the 8 positions
-// (row rotation by 8, the two lane swaps); exponentials in the log2 domain (v_exp_f32, whose error
-// of one unit in the last place is far inside the 1e-5 bar); the lane keeps its own position stream's
-// sum and 8 heads x 8 dims of output, reduced over positions once at the end. K and V rows are
-// read once for all heads of the group, as in the bf16 kernel; the generic kernel reads them once
-// per head, a row per turn.
+// Decode kernel, f32 (the reference's own element type), head width 64, up to 16 query heads per
+// kv head: the bf16 kernel's grid, chunks, partials and lane roles on the f32 matrix instruction
+// v_mfma_f32_16x16x4_f32 (A: lane (n, j) gives row n, k-slot j; B: k-slot j, column n; the lane
+// receives rows 4j + i of column n).
+//
+//   S^T[tok][head] = K[tok][:] . Q[head][:]   16 instructions per 16 positions: lane (n, j) loads the
+//       four floats at dims 16s + 4j of position n's K row (16 bytes, the four lanes of a position
+//       read 64 contiguous bytes) and of head n's query; step (s, e) contracts dim 16s + 4j + e.
+//   O^T[dim][head] += V^T[dim][tok] . P^T[tok][head]   16 per 16 positions: step i of block mm takes the
+//       lane's own weight of position 4j + i as B and V[position 4j + i][dim 16mm + n] as A, a
+//       4-byte load whose 16 lanes read 64 contiguous bytes of one V row: V arrives transposed
+//       straight from memory, every byte read once.
+// 64 cycles of the matrix pipe per position and wavefront, a third of what reading the rows takes
+// at full memory rate, so the kernel is bound by memory like the bf16 one; nothing is rounded below
+// f32. Rows of a ring are found without a division per lane: the tile's first row is uniform.
 // =============================================================================================
-template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
-    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), CTRL, 0xf, 0xf, true));
-}
-__device__ __forceinline__ float sum_over_dim_lanes(float x) { // lanes that differ in bits 0..2
-    x += dpp_f32<0xB1>(x);  // quad_perm [1,0,3,2]
-    x += dpp_f32<0x4E>(x);  // quad_perm [2,3,0,1]
-    x += dpp_f32<0x141>(x); // row_half_mirror: the other quad of the 8 (every lane of a quad holds its sum)
-    return x;
-}
-template <bool MAX> __device__ __forceinline__ float over_position_lanes(float x) { // lanes that differ in bits 3..5
-    const float r = dpp_f32<0x128>(x); // row_ror:8
-    x = MAX ? fmaxf(x, r) : x + r;
-    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    x = MAX ? fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1])) : __uint_as_float(a[0]) + __uint_as_float(a[1]);
-    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return MAX ? fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1])) : __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
+struct kv_tile_f32 {
+    float4 k[2][4];  // [position half][dim step]
+    float v[2][16];  // [position half][4 * i + mm]: position 4j + i, dim 16mm + n
+};
 
-extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_d64(lng_k_attn a) {
-    __shared__ float s_m[4][8];
-    __shared__ float s_l[4][8];
-    __shared__ float s_o[4][8][64];
+extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_attn a) {
+    __shared__ float s_m[4][16];
+    __shared__ float s_l[4][16];
+    __shared__ float s_o[4][16][65];
+
     const uint32_t row = blockIdx.y / a.kv_heads;
     const uint32_t g = blockIdx.y % a.kv_heads;
     const lng_k_row it = row_of(a, row);
-    const uint64_t last = it.start;
-    const uint64_t first = first_visible(last, it.window);
-    const uint64_t base = first & ~(uint64_t)31;
-    const uint64_t c0 = base + (uint64_t)blockIdx.x * a.chunk;
-    if (c0 > last) return; // this row has fewer chunks than the longest one
-    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
-    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
-    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    const uint32_t u = lane >> 3, d8 = lane & 7u;
-    const uint32_t group = a.heads / a.kv_heads;
-    const uint64_t row_floats = (uint64_t)a.kv_heads * 64u;
-    const float *kb = (const float *)(a.k + it.k_offset) + (uint64_t)g * 64u + 8u * d8;
-    const float *vb = (const float *)(a.v + it.v_offset) + (uint64_t)g * 64u + 8u * d8;
+    // positions and slots fit 32 bits (the host refuses shapes whose counts do not)
+    const uint32_t last = (uint32_t)it.start;
+    const uint32_t first = (uint32_t)first_visible(it.start, it.window);
+    const uint32_t base = first & ~31u;
+    const uint64_t c0w = (uint64_t)base + (uint64_t)blockIdx.x * a.chunk;
+    if (c0w > last) return; // this row has fewer chunks than the longest one
+    const uint32_t c0 = (uint32_t)c0w;
+    const uint32_t c1 = (c0w + a.chunk < (uint64_t)last + 1u) ? (uint32_t)(c0w + a.chunk) : last + 1u; // last + 1 fits: last < 2^32 - 1 here or the chunk ends earlier
+    const uint32_t row_chunks = (uint32_t)(((uint64_t)last + 1u - base + a.chunk - 1u) / a.chunk);
 
-    const float sl2 = a.scale * LNG_LOG2E; // scores and maxima live in the log2 domain
-    float qv[8][8], acc[8][8], l[8], m[8];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n = lane & 15u;
+    const uint32_t j = lane >> 4;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t slots = (uint32_t)(it.slots > 0xffffffffull ? 0xffffffffull : it.slots);
+    const bool wraps = it.slots <= last;
+    const bool small_ring = slots < 32u;
+    const uint64_t row_floats = (uint64_t)a.kv_heads * 64u;
+    const float *kb = (const float *)(a.k + it.k_offset) + (uint64_t)g * 64u + 4u * j;
+    const float *vb = (const float *)(a.v + it.v_offset) + (uint64_t)g * 64u + n;
+
+    float4 qv[4];
 #pragma unroll
-    for (int h = 0; h < 8; ++h) {
-        const float *qp = (const float *)(a.q + it.q_offset) + ((uint64_t)g * group + h) * 64u + 8u * d8;
-        float4 q0 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), q1 = q0;
-        if ((uint32_t)h < group) {
-            q0 = *(const float4 *)qp;
-            q1 = *(const float4 *)(qp + 4);
-        }
-        qv[h][0] = q0.x; qv[h][1] = q0.y; qv[h][2] = q0.z; qv[h][3] = q0.w;
-        qv[h][4] = q1.x; qv[h][5] = q1.y; qv[h][6] = q1.z; qv[h][7] = q1.w;
-        l[h] = 0.0f;
-        m[h] = LNG_NEG_INF;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
+    for (int s = 0; s < 4; ++s) {
+        qv[s] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (n < group) qv[s] = *(const float4 *)((const float *)(a.q + it.q_offset) + ((uint64_t)g * group + n) * 64u + 16u * s + 4u * j);
     }
-    // the rows of the next turn are requested before the arithmetic of this one
-    float4 k0, k1, v0, v1, nk0, nk1, nv0, nv1;
-    auto fetch = [&](uint64_t pb, float4 &a0, float4 &a1, float4 &b0, float4 &b1) {
-        const uint64_t p = pb + u;
-        const uint64_t pc = p < first ? first : (p > last ? last : p); // a row that exists, whatever p is
-        const uint64_t r = pc % it.slots;
-        a0 = *(const float4 *)(kb + r * row_floats);
-        a1 = *(const float4 *)(kb + r * row_floats + 4);
-        b0 = *(const float4 *)(vb + r * row_floats);
-        b1 = *(const float4 *)(vb + r * row_floats + 4);
+
+    // cache row of position tp + off (off < 32), clamped into [first, last] so that it exists and is finite
+    auto row_of_pos = [&](uint32_t tp, uint32_t rbase, uint32_t off) -> uint64_t {
+        uint32_t p = tp + off;
+        p = p < first ? first : p;
+        p = p > last ? last : p;
+        uint32_t r = rbase + (p - tp);
+        if (small_ring) {
+            r %= slots;
+        } else {
+            r = r >= slots ? r - slots : r;
+        }
+        return (uint64_t)r * row_floats;
     };
-    if (c0 + 8u * wave < c1) fetch(c0 + 8u * wave, nk0, nk1, nv0, nv1);
-    for (uint64_t pb = c0 + 8u * wave; pb < c1; pb += 32u) {
-        const uint64_t p = pb + u;
-        const bool seen = p >= first && p < c1;
-        k0 = nk0; k1 = nk1; v0 = nv0; v1 = nv1;
-        if (pb + 32u < c1) fetch(pb + 32u, nk0, nk1, nv0, nv1);
-        const float kx[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
-        const float vx[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+    auto load_tile = [&](uint32_t tp, kv_tile_f32 &t) {
+        const uint32_t rbase = wraps ? tp % slots : tp; // uniform over the wavefront
 #pragma unroll
-        for (int h = 0; h < 8; ++h) {
-            if ((uint32_t)h >= group) break; // the same for every lane
-            float part = 0.0f;
+        for (int half = 0; half < 2; ++half) {
+            const float *kp = kb + row_of_pos(tp, rbase, 16u * half + n);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) part += qv[h][e] * kx[e];
-            const float sc = seen ? sum_over_dim_lanes(part) * sl2 : LNG_NEG_INF; // log2 domain
-            const float next = fmaxf(m[h], over_position_lanes<true>(sc));
-            if (next == LNG_NEG_INF) continue;   // nothing seen yet (the same for every lane)
-            if (next != m[h]) {                  // the maximum moved (the same for every lane): rescale
-                const float keep = m[h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(m[h] - next);
-                l[h] *= keep;
+            for (int s = 0; s < 4; ++s) t.k[half][s] = *(const float4 *)(kp + 16 * s);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[h][e] *= keep;
-                m[h] = next;
+            for (int i = 0; i < 4; ++i) {
+                const float *vp = vb + row_of_pos(tp, rbase, 16u * half + 4u * j + i);
+#pragma unroll
+                for (int mm = 0; mm < 4; ++mm) t.v[half][4 * i + mm] = vp[16 * mm];
             }
-            const float w = sc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sc - next);
-            l[h] += w;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) acc[h][e] += w * vx[e];
         }
+    };
+
+    const float sl2 = a.scale * LNG_LOG2E;
+    float m = LNG_NEG_INF; // running max of head n, log2 domain
+    float l = 0.0f;        // this lane's share of the running sum
+    floatx4 ot[4];         // O^T[16mm + 4j + i][head n]
+#pragma unroll
+    for (int mm = 0; mm < 4; ++mm) ot[mm] = (floatx4){0.f, 0.f, 0.f, 0.f};
+
+    kv_tile_f32 cur, nxt;
+    uint32_t tp = c0 + wave * 32u;
+    if (tp < c1) load_tile(tp, cur);
+    for (; tp < c1; tp += 128u) {
+        if (c1 - tp > 128u) load_tile(tp + 128u, nxt);
+
+        floatx4 st[2];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            st[half] = (floatx4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].x, qv[s].x, st[half], 0, 0, 0);
+                st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].y, qv[s].y, st[half], 0, 0, 0);
+                st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].z, qv[s].z, st[half], 0, 0, 0);
+                st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].w, qv[s].w, st[half], 0, 0, 0);
+            }
+        }
+        float tmax = LNG_NEG_INF;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t off = (uint32_t)(half * 16 + i) + 4u * j;
+                const bool seen = off < c1 - tp && tp + off >= first; // c1 <= last + 1
+                const float x = seen ? st[half][i] * sl2 : LNG_NEG_INF;
+                st[half][i] = x;
+                tmax = fmaxf(tmax, x);
+            }
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m, tmax);
+        const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+        float psum = 0.0f;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float pw = __builtin_amdgcn_exp2f(st[half][i] - m_safe);
+                st[half][i] = pw;
+                psum += pw;
+            }
+        }
+        l = l * alpha + psum;
+        m = m_new;
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {
+            ot[mm] = ot[mm] * alpha;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    ot[mm] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.v[half][4 * i + mm], st[half][i], ot[mm], 0, 0, 0);
+                }
+            }
+        }
+        cur = nxt;
     }
-    // ---- over the positions of the wavefront, then over the four wavefronts -----------------------
-#pragma unroll
-    for (int h = 0; h < 8; ++h) {
-        if ((uint32_t)h >= group) break;
-        const float lsum = over_position_lanes<false>(l[h]);
-        if (lane == 0) {
-            s_m[wave][h] = m[h];
-            s_l[wave][h] = lsum;
+
+    // ---- merge the four wavefronts ---------------------------------------------------------
+    {
+        float lt = l + __shfl_xor(l, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (j == 0) {
+            s_m[wave][n] = m;
+            s_l[wave][n] = lt;
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float o = over_position_lanes<false>(acc[h][e]);
-            if (u == 0) s_o[wave][h][8u * d8 + e] = o;
+        for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_o[wave][n][16 * mm + 4 * j + i] = ot[mm][i];
         }
     }
     __syncthreads();

@@ -494,10 +494,11 @@ def test_decode_bf16_one_long_row(gpu, start, window, slots):
 @pytest.mark.parametrize("t,start,window,slots,heads,kv_heads", [
     (1, 0, FULL, 1, 64, 8), (1, 36, FULL, 37, 64, 8), (1, 4095, FULL, 4096, 64, 8), (1, 5000, 128, 200, 64, 8),
     (1, 70000, FULL, 70001, 64, 8), (1, 200000, 100000, 150016, 16, 2), (3, 2000, FULL, 2003, 8, 8), (7, 900, 33, 41, 6, 2),
-    (31, 100, FULL, 131, 5, 1), (2, 9000, 1, 3, 64, 8), (5, 260, 300, 305, 24, 8),
+    (31, 100, FULL, 131, 5, 1), (2, 9000, 1, 3, 64, 8), (5, 260, 300, 305, 24, 8), (1, 5000, FULL, 5001, 32, 2),
+    (3, 700, 100, 128, 12, 1), (2, 40, 17, 19, 16, 1), (1, 31, FULL, 32, 64, 8), (1, 0, FULL, 1, 64, 8),
 ])
 def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_heads, monkeypatch):
-    """The row-by-row operator on f32 caches: every grouping up to 8 heads per kv head, one chunk and many
+    """The row-by-row operator on f32 caches: groupings up to 16 heads per kv head, one chunk and many
     (merged by a second dispatch), rings that have wrapped, windows that start inside a tile, with and without
     sinks; rows the operator must not read hold NaN (attention_grouped.rs:57). Within 1e-5 (relative to
     1 + |x|) of the CPU reference, and the generic kernel (LNG_F32_GENERIC) agrees."""
