@@ -194,6 +194,31 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
     for _ in range(5):
         go32()
     f32_us = sorted(go32() for _ in range(max(steps, 20)))[max(steps, 20) // 2] * 1e6
+    for b in (qf, of, kf, vf):
+        b.free()
+    # one f32 layer of a decoding step: 16 sequences at a 32,768-token context (4.3 GB of cache rows)
+    n_seq, long_ctx = 16, 32768
+    qf, of = gpu.buffer(n_seq * 2 * QO), gpu.buffer(n_seq * 2 * QO)
+    kf, vf = gpu.buffer(n_seq * long_ctx * 2 * ROW), gpu.buffer(n_seq * long_ctx * 2 * ROW)
+    for i, b in enumerate((qf, kf, vf)):
+        bb = gpu.batch([b])
+        bb.fill_synthetic(C.Slice(0, 0, b.len), C.F32, 20 + i, 0.5, 0)
+        bb.run()
+        bb.drop()
+    items = C.decode_items([C.DecodeItem(i * 2 * QO, i * 2 * QO, i * long_ctx * 2 * ROW, i * long_ctx * 2 * ROW, 0,
+                                         long_ctx - 1, C.FULL, long_ctx) for i in range(n_seq)])
+
+    def go32b():
+        batch = gpu.batch([qf, kf, vf, of, sinks32])
+        batch.attention_decode_batched(0, 1, 2, 3, 4, items, H, G, D, SCALE, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(3):
+        go32b()
+    f32_batch = sorted(go32b() for _ in range(9))[4]
+    f32_batch_bytes = n_seq * (long_ctx * 2 * ROW * 2 + 4 * QO + H * 4)
     for b in (qf, of, kf, vf, sinks32):
         b.free()
     nbytes = decode_bytes(ctx, C.FULL)
@@ -201,6 +226,9 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
     gb, wb = many[len(many) // 2]
     return {"workload": "C2 decode, 1 query, 4096 cached positions, full-causal", "bytes": nbytes,
             "f32_caches_single_launch_gpu_us": f32_us,
+            "f32_caches_16_sequences_32768": {"gpu_us": f32_batch * 1e6, "bytes": f32_batch_bytes,
+                                              "gbs": f32_batch_bytes / f32_batch / 1e9,
+                                              "hbm_frac": f32_batch_bytes / f32_batch / 1e9 / HBM_PEAK_GBS},
             "single_launch_gpu_us": g1 * 1e6, "single_launch_wall_us": w1 * 1e6,
             "single_launch_gbs": nbytes / g1 / 1e9 if g1 > 0 else None,
             "burst": burst, "burst_gpu_us_per_launch": gb / burst * 1e6,
