@@ -418,7 +418,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     uint64_t latest = t_uniform ? host_rows[0].start + t_uniform - 1 : 0;
     for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
     const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 16 && aligned16 && latest < 0xffffff00ull &&
-                          !getenv("LNG_F32_GENERIC");
+                          a.scale > 0.0f && a.scale <= 3.0e38f && !getenv("LNG_F32_GENERIC");
     if (!fast && !fast_f32) {
         Cmd c;
         c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;
@@ -499,7 +499,10 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     // Measured break-even on 64/8 heads: rows x visible keys of about 32 K (16 rows over 2,048 keys, 4 over 8,192).
     const uint64_t seen = std::min<uint64_t>(end, s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t);
     const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && s.t * seen >= 32768 && !getenv("LNG_PLAIN_ROW_BY_ROW");
-    if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 &&
+    // (the matrix kernels take the maximum of the raw products and scale it afterwards: scale > 0; any other
+    // scale goes to the kernels that scale first)
+    const bool scale_positive = s.scale > 0.0f && s.scale <= 3.0e38f;
+    if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 && scale_positive &&
         (dtype == LNG_BF16 || !getenv("LNG_F32_GENERIC"))) {
         const bool f32 = dtype == LNG_F32;
         lng_k_prefill p{};

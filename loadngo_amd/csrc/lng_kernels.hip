@@ -664,14 +664,14 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
             for (int i = 0; i < 4; ++i) {
                 const uint32_t off = (uint32_t)(half * 16 + i) + 4u * j;
                 const bool seen = off < c1 - tp && tp + off >= first; // c1 <= last + 1
-                const float x = seen ? st[half][i] * sl2 : LNG_NEG_INF;
+                const float x = seen ? st[half][i] : LNG_NEG_INF;
                 st[half][i] = x;
                 tmax = fmaxf(tmax, x);
             }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m, tmax);
+        const float m_new = fmaxf(m, tmax * sl2); // scale > 0: the maximum commutes with it
         const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
         float psum = 0.0f;
@@ -679,7 +679,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
         for (int half = 0; half < 2; ++half) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float pw = __builtin_amdgcn_exp2f(st[half][i] - m_safe);
+                // one rounding, of the small difference (not of the scaled score and then of the difference)
+                const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(st[half][i], sl2, -m_safe));
                 st[half][i] = pw;
                 psum += pw;
             }

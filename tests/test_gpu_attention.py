@@ -574,3 +574,25 @@ def test_several_f32_rows_through_the_row_by_row_operator_over_long_caches(gpu, 
     monkeypatch.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
     rows = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
     assert rel_error(rows, want) <= F32_RTOL
+
+
+@pytest.mark.parametrize("scale", [-0.125, 0.0])
+def test_scales_that_are_not_positive(gpu, scale):
+    """GroupedShape.scale is 1/sqrt(dim) in every caller, but the operator takes any float: a negative or zero
+    scale (which the matrix kernels, taking maxima of unscaled products, do not handle) still gives the CPU
+    reference's result, in both element types, prompt pass and decode."""
+    heads, kv_heads = 16, 2
+    for t, start in ((96, 32), (1, 700)):
+        end = start + t
+        q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
+        tiled = t >= 32
+        slots = (end + 31) // 32 * 32
+        kr, vr = ring_layout(k, t, start, slots, tiled), ring_layout(v, t, start, slots, tiled)
+        shape = C.GroupedShape(t, start, heads, kv_heads, 64, FULL, slots, scale)
+        want = oracle.attention_f32(q, k, v, sinks, start, window=FULL, slots=None, scale=scale, threads=THREADS)
+        assert rel_error(run_attention(gpu, q, kr, vr, sinks, shape, tiled, C.F32), want) <= F32_RTOL
+        qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+        krb, vrb = ring_layout(kb, t, start, slots, tiled), ring_layout(vb, t, start, slots, tiled)
+        wantb = oracle.attention_bf16(qb, kb, vb, sinks, start, window=FULL, scale=scale, threads=THREADS)
+        gotb = run_attention(gpu, qb, krb, vrb, sinks, shape, tiled, C.BF16)
+        assert max_error(from_bf16_bits(gotb), from_bf16_bits(wantb)) < BF16_TOL
