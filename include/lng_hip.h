@@ -128,8 +128,10 @@ int lng_hip_batch_barrier(lng_batch *batch);
 /* apple.rs:2202 Batch::commit(proactor, on_done) — submits without blocking. `on_done` runs
  * once on a library thread when the GPU has finished (the Rust shim re-posts it to the
  * caller's proactor, as apple.rs:2231-2232 does); it may be NULL. The batch handle stays
- * valid for lng_hip_batch_wait / lng_hip_batch_drop, neither of which may be called from
- * inside `on_done` (they wait for the thread that is running it). Batches may be recorded on
+ * valid for lng_hip_batch_wait / lng_hip_batch_drop. lng_hip_batch_wait may not be called from
+ * inside `on_done` (it waits for the thread that is running it); lng_hip_batch_drop may: the
+ * handle is then freed when the callback returns, which is how a binding whose commit consumes
+ * the batch (apple.rs:2202 takes `self`) lets go of it. Batches may be recorded on
  * different threads at once; their submissions are serialised, and the dispatches of one batch
  * run back to back on the device. */
 int lng_hip_batch_commit(lng_batch *batch, lng_on_done on_done, void *user);

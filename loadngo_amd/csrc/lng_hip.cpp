@@ -133,6 +133,7 @@ struct lng_batch {
     std::mutex mu;
     std::condition_variable cv;
     bool released = false;
+    bool drop_when_done = false; // lng_hip_batch_drop was called from inside on_done
 };
 
 namespace {
@@ -341,6 +342,13 @@ void finish(lng_batch *b) {
     release(b);
 }
 
+void destroy(lng_batch *b) {
+    if (b->ev0) hipEventDestroy(b->ev0);
+    if (b->ev1) hipEventDestroy(b->ev1);
+    for (hipEvent_t mark : b->marks) hipEventDestroy(mark);
+    delete b;
+}
+
 void worker_loop(lng_gpu *g) {
     for (;;) {
         lng_batch *b = nullptr;
@@ -356,13 +364,16 @@ void worker_loop(lng_gpu *g) {
             lng_completed done{b->status, b->seconds, b->message.c_str()};
             b->on_done(&done, b->user);
         }
+        bool drop = false;
         {
             // Notified under the lock: a waiter may delete the batch as soon as it sees Done, and
             // it cannot see it before this thread has let go of the batch for good.
             std::lock_guard<std::mutex> lock(b->mu);
             b->state = lng_batch::Done;
+            drop = b->drop_when_done;
             b->cv.notify_all();
         }
+        if (drop) destroy(b); // the callback dropped its own batch: nobody else holds the handle
     }
 }
 
@@ -879,11 +890,12 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
         b->message = hip_text(e);
         release(b);
         b->state = lng_batch::Done;
+        const std::string message = b->message; // on_done may drop the batch
         if (on_done) {
-            lng_completed done{b->status, 0.0, b->message.c_str()};
+            lng_completed done{LNG_ERR_GPU, 0.0, message.c_str()};
             on_done(&done, user);
         }
-        return fail(LNG_ERR_GPU, "submission failed: %s", b->message.c_str());
+        return fail(LNG_ERR_GPU, "submission failed: %s", message.c_str());
     }
     if (on_done) {
         std::lock_guard<std::mutex> lock(g->qmu);
@@ -911,15 +923,23 @@ extern "C" int lng_hip_batch_wait(lng_batch *b, double *gpu_seconds) {
 
 extern "C" void lng_hip_batch_drop(lng_batch *b) {
     if (!b) return;
+    if (b->state == lng_batch::Committed && b->on_done) {
+        bool on_completion_thread;
+        {
+            std::lock_guard<std::mutex> lock(b->gpu->qmu); // commit starts the thread under this lock
+            on_completion_thread = b->gpu->worker.get_id() == std::this_thread::get_id();
+        }
+        if (on_completion_thread) { // inside its own on_done: freed when the callback returns
+            b->drop_when_done = true;
+            return;
+        }
+    }
     if (b->state == lng_batch::Recording) {
         release(b);
     } else {
         lng_hip_batch_wait(b, nullptr);
     }
-    if (b->ev0) hipEventDestroy(b->ev0);
-    if (b->ev1) hipEventDestroy(b->ev1);
-    for (hipEvent_t mark : b->marks) hipEventDestroy(mark);
-    delete b;
+    destroy(b);
 }
 
 extern "C" int lng_hip_batch_set_timing(lng_batch *b, int enabled) {
