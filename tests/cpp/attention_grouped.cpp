@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "lng_compute.hpp"
+#include "test_support.hpp"
 
 using lng::Batch;
 using lng::Buffer;
@@ -24,33 +25,9 @@ using lng::Slice;
 
 namespace {
 
-int failures = 0;
-
-void expect(bool ok, const std::string &what) {
-    if (!ok) {
-        ++failures;
-        std::printf("FAILED %s\n", what.c_str());
-    }
-}
-
-// attention_grouped.rs:25-36: xorshift values in [-1, 1)
-std::vector<float> values(uint64_t seed, size_t n) {
-    std::vector<float> out(n);
-    uint64_t s = seed | 1;
-    for (size_t i = 0; i < n; ++i) {
-        s ^= s << 13;
-        s ^= s >> 7;
-        s ^= s << 17;
-        out[i] = (float)(s >> 40) / (float)(1ull << 23) - 1.0f;
-    }
-    return out;
-}
-
-Buffer upload(const Gpu &gpu, const std::vector<float> &v) {
-    Buffer b = gpu.buffer((v.empty() ? 1 : v.size()) * 4);
-    b.copy_from_f32(v);
-    return b;
-}
+using support::expect;
+using support::upload;
+using support::values;
 
 size_t up32(size_t n) { return (n + 31) / 32 * 32; }
 
@@ -330,6 +307,6 @@ int main() {
         std::printf("FAILED with %s\n", e.what());
         return 100;
     }
-    std::printf("%d failures\n", failures);
-    return failures;
+    std::printf("%d failures\n", support::failures);
+    return support::failures;
 }
