@@ -85,10 +85,14 @@ struct lng_gpu {
     int device = 0;
     hipStream_t stream = nullptr;
     hipModule_t module = nullptr;
-    hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr, decode_bf16_d64 = nullptr,
-                  decode_merge = nullptr, decode_f32_d64 = nullptr, prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_merge = nullptr, copy_rows = nullptr, fill_synthetic = nullptr,
-                  add_rows = nullptr, rotate_halves = nullptr, prepare_v4 = nullptr, prepare_v1 = nullptr,
-                  q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr, q8_tiled_bf16 = nullptr, rmsnorm_rows = nullptr;
+    // kernels of the embedded code object
+    hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
+    hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr;
+    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_merge = nullptr;
+    hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr;
+    hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
+    hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
+                  q8_tiled_bf16 = nullptr;
     std::string name;
     unsigned cus = 256;
 
