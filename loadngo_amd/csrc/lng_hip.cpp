@@ -511,9 +511,10 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     // tokens at once late in a context) reads the cache once per row in the decode kernel; the prompt-pass
     // kernel reads it once per call and gives the same rows (it touches no row outside
     // [first visible position, last position], which is all the row-by-row operator promises to be there).
-    // Measured break-even on 64/8 heads: rows x visible keys of about 32 K (16 rows over 2,048 keys, 4 over 8,192).
+    // Measured break-even on 64/8 heads: rows x visible keys of about 32 K at 2,048 keys (16 rows), 16 K from 4,096 keys on.
     const uint64_t seen = std::min<uint64_t>(end, s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t);
-    const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && s.t * seen >= 32768 && !getenv("LNG_PLAIN_ROW_BY_ROW");
+    const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && (s.t * seen >= 32768 || (seen >= 4096 && s.t * seen >= 16384)) &&
+                              !getenv("LNG_PLAIN_ROW_BY_ROW");
     // (the matrix kernels take the maximum of the raw products and scale it afterwards: scale > 0; any other
     // scale goes to the kernels that scale first)
     const bool scale_positive = s.scale > 0.0f && s.scale <= 3.0e38f;
@@ -538,7 +539,10 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         // per wavefront (32 rows, two workgroups per compute unit) when each query sees few keys
         // and the pass is bound by latency, not by the matrix pipe.
         // (the f32 kernel has one form: 32 rows, one head per wavefront; it is bound by the f32 matrix rate)
-        const bool narrow = !f32 && p.window != LNG_WINDOW_FULL && p.window <= 1024;
+        // Up to 32 rows (the tail of a prompt, a few tokens at once) would leave half of a 64-row tile empty: the
+        // 32-row form again (measured 10-30 % faster there; from 64 rows on the two-head form wins at long contexts).
+        const bool few_rows = s.t <= 32;
+        const bool narrow = !f32 && ((p.window != LNG_WINDOW_FULL && p.window <= 1024) || few_rows);
         const unsigned rows_per_wg = narrow || f32 ? 32 : 64;
         p.q_tiles = (uint32_t)((s.t + rows_per_wg - 1) / rows_per_wg);
         p.scale = s.scale;
@@ -551,7 +555,7 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const uint64_t visible = p.window == LNG_WINDOW_FULL ? end : std::min<uint64_t>(end, p.window + rows_per_wg);
         const uint64_t key_tiles = (visible + 63) / 64;
         const uint64_t plain_wgs = (uint64_t)p.q_tiles * s.kv_heads;
-        if (!narrow && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
+        if ((!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
             uint64_t want = g->cus / plain_wgs;
             want = std::min<uint64_t>(want, key_tiles / 4);
             want = std::min<uint64_t>(want, 64);
