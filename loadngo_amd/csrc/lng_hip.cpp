@@ -393,7 +393,7 @@ uint64_t visible_from_tile(const lng_k_row &r) { // positions from the tile-alig
     return last + 1 - (first & ~(uint64_t)31);
 }
 
-DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_uniform, uint32_t kv_heads) {
+DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_uniform, uint32_t kv_heads, unsigned wgs_per_cu) {
     // rows == the table, or one row standing for t_uniform consecutive queries of one cache
     uint64_t total = 0, longest = 0;
     if (t_uniform) {
@@ -415,7 +415,13 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     const uint64_t per_wg = (total * kv_heads + g->decode_wgs - 1) / g->decode_wgs;
     uint64_t chunk = (per_wg + 127) / 128 * 128;
     chunk = std::max<uint64_t>(chunk, 128);
-    // no row may have more than LNG_MAX_CHUNKS chunks (the merge keeps one weight per chunk in LDS)
+    // The merge of a row walks its chunks one after another: no more than 32 chunks per row, unless so few rows
+    // are in the dispatch that this would leave compute units without a workgroup (bf16; two workgroups for the
+    // f32 kernel, which has twice the bytes per position and a merge of its own dispatch anyway: measured);
+    // never more than LNG_MAX_CHUNKS (the merge keeps one weight per chunk in LDS).
+    const uint64_t pairs = (t_uniform ? t_uniform : (uint64_t)n) * kv_heads;
+    const uint64_t most = std::min<uint64_t>(LNG_MAX_CHUNKS, std::max<uint64_t>(32, (wgs_per_cu * g->cus + pairs - 1) / pairs));
+    chunk = std::max<uint64_t>(chunk, ((longest + most - 1) / most + 127) / 128 * 128);
     chunk = std::max<uint64_t>(chunk, ((longest + LNG_MAX_CHUNKS - 1) / LNG_MAX_CHUNKS + 127) / 128 * 128);
     p.chunk = (uint32_t)chunk;
     p.n_chunks = (uint32_t)((longest + chunk - 1) / chunk);
@@ -444,7 +450,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         b->cmds.push_back(std::move(c));
         return LNG_OK;
     }
-    const DecodePlan plan = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads);
+    const DecodePlan plan = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads, fast ? 1u : 2u);
     a.chunk = plan.chunk;
     a.n_chunks = plan.n_chunks;
     if (plan.n_chunks > 1) {
