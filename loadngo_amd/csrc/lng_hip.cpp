@@ -415,12 +415,16 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     const uint64_t per_wg = (total * kv_heads + g->decode_wgs - 1) / g->decode_wgs;
     uint64_t chunk = (per_wg + 127) / 128 * 128;
     chunk = std::max<uint64_t>(chunk, 128);
-    // The merge of a row walks its chunks one after another: no more than 32 chunks per row, unless so few rows
-    // are in the dispatch that this would leave compute units without a workgroup (bf16; two workgroups for the
-    // f32 kernel, which has twice the bytes per position and a merge of its own dispatch anyway: measured);
-    // never more than LNG_MAX_CHUNKS (the merge keeps one weight per chunk in LDS).
+    // The merge of a row walks its chunks one after another: no more than 32 chunks per row (16 up to 8,192
+    // positions when the dispatch has one or two sequences: with many rows the merges run side by side and
+    // larger chunks only unbalance the workgroups), unless so few rows are in the dispatch that this would leave compute units without
+    // a workgroup (bf16; two workgroups for the f32 kernel, which has twice the bytes per position and a merge
+    // of its own dispatch anyway) and the chunks would stay at 512 positions or more (all measured on one
+    // sequence: 4,096 keys 13.9 -> 12.3 us, 131,072 keys 76 -> 50 us); never more than LNG_MAX_CHUNKS (the merge
+    // keeps one weight per chunk in LDS).
     const uint64_t pairs = (t_uniform ? t_uniform : (uint64_t)n) * kv_heads;
-    const uint64_t most = std::min<uint64_t>(LNG_MAX_CHUNKS, std::max<uint64_t>(32, (wgs_per_cu * g->cus + pairs - 1) / pairs));
+    const uint64_t fill = std::min<uint64_t>((wgs_per_cu * g->cus + pairs - 1) / pairs, longest / 512);
+    const uint64_t most = std::min<uint64_t>(LNG_MAX_CHUNKS, std::max<uint64_t>(longest <= 8192 && pairs <= 16 ? 16 : 32, fill));
     chunk = std::max<uint64_t>(chunk, ((longest + most - 1) / most + 127) / 128 * 128);
     chunk = std::max<uint64_t>(chunk, ((longest + LNG_MAX_CHUNKS - 1) / LNG_MAX_CHUNKS + 127) / 128 * 128);
     p.chunk = (uint32_t)chunk;
