@@ -196,6 +196,28 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
     f32_us = sorted(go32() for _ in range(max(steps, 20)))[max(steps, 20) // 2] * 1e6
     for b in (qf, of, kf, vf):
         b.free()
+    # one sequence late in a long context (the reference's interactive case): bf16, 131,072 cached positions
+    far = 131072
+    qs, os_ = gpu.buffer(QO), gpu.buffer(QO)
+    ks, vs = gpu.buffer(far * ROW), gpu.buffer(far * ROW)
+    for i, b in enumerate((qs, ks, vs)):
+        fill(gpu, b, 40 + i)
+    far_shape = C.GroupedShape(1, far - 1, H, G, D, C.FULL, far, SCALE)
+
+    def go_far():
+        batch = gpu.batch([qs, ks, vs, os_, sinks32])
+        batch.attention_grouped_with_sinks((C.Slice(0, 0, QO), C.Slice(1, 0, far * ROW), C.Slice(2, 0, far * ROW)),
+                                           C.Slice(4, 0, H * 4), C.Slice(3, 0, QO), far_shape, C.BF16)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(3):
+        go_far()
+    far_s = sorted(go_far() for _ in range(15))[7]
+    far_bytes = decode_bytes(far, C.FULL)
+    for b in (qs, os_, ks, vs):
+        b.free()
     # one f32 layer of a decoding step: 16 sequences at a 32,768-token context (4.3 GB of cache rows)
     n_seq, long_ctx = 16, 32768
     qf, of = gpu.buffer(n_seq * 2 * QO), gpu.buffer(n_seq * 2 * QO)
@@ -226,6 +248,8 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
     gb, wb = many[len(many) // 2]
     return {"workload": "C2 decode, 1 query, 4096 cached positions, full-causal", "bytes": nbytes,
             "f32_caches_single_launch_gpu_us": f32_us,
+            "one_sequence_131072": {"gpu_us": far_s * 1e6, "bytes": far_bytes, "gbs": far_bytes / far_s / 1e9,
+                                    "hbm_frac": far_bytes / far_s / 1e9 / HBM_PEAK_GBS},
             "f32_caches_16_sequences_32768": {"gpu_us": f32_batch * 1e6, "bytes": f32_batch_bytes,
                                               "gbs": f32_batch_bytes / f32_batch / 1e9,
                                               "hbm_frac": f32_batch_bytes / f32_batch / 1e9 / HBM_PEAK_GBS},
