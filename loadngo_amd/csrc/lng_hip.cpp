@@ -88,7 +88,7 @@ struct lng_gpu {
     // kernels of the embedded code object
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr;
-    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_merge = nullptr;
+    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
     hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
@@ -579,9 +579,11 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             p.partial_ml = g->scratch_ml;
         }
         Cmd c;
-        c.fn = f32 ? g->prefill_f32_d64 : narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
-        c.name = f32 ? "lng_prefill_f32_d64" : narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
         c.grid[0] = p.q_tiles * (unsigned)s.kv_heads * p.splits; // kv head fastest: one XCD's L2 per kv head
+        // f32: two workgroups per compute unit only when there are four rounds of them or more (see the kernels)
+        const bool f32_two = f32 && c.grid[0] >= 4u * g->cus;
+        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
+        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
         c.block = 512;
         set_args(c, p);
         b->cmds.push_back(std::move(c));
@@ -674,6 +676,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
+        {"lng_prefill_f32_d64_w4", &g->prefill_f32_d64_w4, true},
         {"lng_prefill_merge", &g->prefill_merge, true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},

@@ -1822,7 +1822,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
 #define PF32_KSTRIDE 68 // floats per LDS row of K: 16-byte reads of 16 consecutive rows cover all 64 banks
 #define PF32_VSTRIDE 72 // of V: the rows 4 apart that the two halves of a wavefront read fall 32 banks apart
 
-extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_f32_d64(lng_k_prefill a) {
+__device__ __forceinline__ void prefill_f32_body(const lng_k_prefill &a) {
     __shared__ __attribute__((aligned(16))) float s_k[2][PF_BN * PF32_KSTRIDE];
     __shared__ __attribute__((aligned(16))) float s_v[2][PF_BN * PF32_VSTRIDE];
 
@@ -2011,6 +2011,15 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_f32_d64(lng
         }
     }
 }
+
+// One workgroup per compute unit (146 registers): passes with few workgroups, which then go to the compute units
+// longest first, one at a time, and stay balanced.
+extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_f32_d64(lng_k_prefill a) { prefill_f32_body(a); }
+
+// Two workgroups per compute unit (128 registers, 4 of them spilled): one's softmax and LDS traffic under the
+// other's matrix instructions. For passes with many workgroups (the long causal pass +3-6 %, the windowed one +19 %);
+// with two rounds of workgroups or fewer, co-resident pairs of unequal length leave units idle (2,048 positions -25 %).
+extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_f32_d64_w4(lng_k_prefill a) { prefill_f32_body(a); }
 
 // Combines the splits of a prompt pass; the sink joins here. Up to eight splits (the usual case: one
 // workgroup per compute unit needs few): a thread per (row, head, four dims) requests its splits' partial
