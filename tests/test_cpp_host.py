@@ -1,7 +1,8 @@
 """The C++ host side (include/lng_compute.hpp: the reference's Gpu / Buffer / Resident / Slice / Batch /
 GroupedShape / Completed / Error over the C ABI) under the reference's own operator tests, restated in
 tests/cpp/ (metal-compute/tests/attention_grouped.rs, q8_0_and_gpt_oss_glue.rs, glue.rs: same shapes,
-generator, float64 definitions and bounds). Without a GPU the programs must compile, link and refuse to run
+generator, float64 definitions and bounds), and the entry points without a counterpart there against the
+sequences of reference operators they stand for (tests/cpp/additions.cpp). Without a GPU the programs must compile, link and refuse to run
 with NoDevice; with one they must pass."""
 import os
 import subprocess
@@ -11,6 +12,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_DIR = os.path.join(ROOT, "loadngo_amd")
 PROGRAMS = {
+    "additions": ("batched_decode_is_one_plain_call_per_sequence", "prepare_attention_is_the_reference_sequence_of_dispatches",
+                  "q8_product_of_bf16_positions_is_the_f32_product"),
     "attention_grouped": ("matches_the_float64_definition", "tiled_matches_the_float64_definition",
                           "sinks_take_probability_without_value_on_gpt_oss_shapes", "rejects_shapes_it_cannot_run",
                           "ownership_residents_and_bf16"),
