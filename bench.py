@@ -470,6 +470,38 @@ def run_q8(gpu, steps, warmup):
                       "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS, "tflops": flops / g / 1e12}
         x.free()
         y.free()
+    # the q, k and v projections of one decoding position (4096, 512 and 512 rows): three products as the reference
+    # records them (gpu.rs:724-732), and as one dispatch
+    kv_rows = 512
+    k_codes = gpu.resident(rng.integers(-127, 128, kv_rows * cols, dtype=np.int8))
+    k_scales = gpu.resident((rng.random(kv_rows * cols // 32, dtype=np.float32) * 0.01 + 0.001).astype(np.float16).view(np.uint16))
+    x, y = gpu.buffer(cols * 4), gpu.buffer((rows + 2 * kv_rows) * 4)
+    b = gpu.batch([x])
+    b.fill_synthetic(C.Slice(0, 0, x.len), C.F32, 79, 0.5, 0)
+    b.run()
+    b.drop()
+    for label, together in (("qkv_one_position_three_dispatches", False), ("qkv_one_position_one_dispatch", True)):
+        def go3():
+            batch = gpu.batch([x, y])
+            mq, mk = (batch.attach(codes), batch.attach(scales)), (batch.attach(k_codes), batch.attach(k_scales))
+            xs = C.Slice(0, 0, x.len)
+            ys = [C.Slice(1, 0, rows * 4), C.Slice(1, rows * 4, kv_rows * 4), C.Slice(1, (rows + kv_rows) * 4, kv_rows * 4)]
+            if together:
+                batch.gemm_q8_0_many([(mq, ys[0], rows), (mk, ys[1], kv_rows), (mk, ys[2], kv_rows)], xs, cols, 1, cols)
+            else:
+                batch.gemv_q8_0(mq, xs, ys[0], rows, cols)
+                batch.gemv_q8_0(mk, xs, ys[1], kv_rows, cols)
+                batch.gemv_q8_0(mk, xs, ys[2], kv_rows, cols)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        for _ in range(warmup):
+            go3()
+        runs = sorted(go3() for _ in range(max(steps, 9)))
+        out[label] = {"gpu_us": runs[len(runs) // 2] * 1e6}
+    x.free()
+    y.free()
     # the same matrix on bf16 positions (what a bf16 attention leaves for the output projection): one operand
     # plane instead of two, no split of x
     for label, n in (("decode_16_sequences_bf16_positions", 16), ("prompt_8192_bf16_positions", 8192)):

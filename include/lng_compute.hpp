@@ -275,6 +275,18 @@ class Batch {
         detail::check(lng_hip_gemm_q8_0_bf16(h_, matrix.first.c(), matrix.second.c(), x.c(), y.c(), rows_cols.first,
                                              rows_cols.second, n, strides.first, strides.second));
     }
+    // No counterpart in the reference (three gemv/gemm calls per layer, gpu.rs:724-732): up to four matrices
+    // times the same positions, each y dense [n][rows]; one dispatch below 32 positions.
+    struct Q8Matrix {
+        std::pair<Slice, Slice> matrix; // (codes, scales)
+        Slice y;
+        std::size_t rows;
+    };
+    void gemm_q8_0_many(const std::vector<Q8Matrix> &matrices, Slice x, std::size_t cols, std::size_t n, std::size_t x_stride) {
+        std::vector<lng_q8_matrix> raw;
+        for (const Q8Matrix &m : matrices) raw.push_back(lng_q8_matrix{m.matrix.first.c(), m.matrix.second.c(), m.y.c(), m.rows});
+        detail::check(lng_hip_gemm_q8_0_many(h_, raw.data(), raw.size(), x.c(), cols, n, x_stride));
+    }
     // No counterpart in the reference: one decoding query per item, many sequences in one dispatch.
     void attention_decode_batched(std::size_t q_buffer, std::size_t k_buffer, std::size_t v_buffer, std::size_t out_buffer,
                                   std::size_t sinks_buffer, const std::vector<DecodeItem> &items, std::size_t heads,

@@ -290,6 +290,21 @@ int lng_hip_gemm_q8_0_tiled(lng_batch *batch, lng_slice codes, lng_slice scales,
 int lng_hip_gemm_q8_0_bf16(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
                            uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride);
 
+/* No counterpart in the reference, which records one product per matrix (the q, k and v projections of a
+ * layer are three gemv/gemm calls, gpt-oss/src/gpu.rs:724-732): up to four Q8_0 matrices of the same number of
+ * columns multiplied by the same positions. Matrix i gives y_i[p] = W_i x[p], y_i dense ([n][rows_i] f32);
+ * each product is exactly lng_hip_gemm_q8_0(codes_i, scales_i, x, y_i, rows_i, cols, n, x_stride, rows_i), with
+ * its refusals, plus: outputs may not overlap one another or any matrix. Below 32 positions (decoding), where
+ * a product is bound by launches and by reading its matrix once, all of them run as one dispatch. */
+typedef struct lng_q8_matrix {
+    lng_slice codes;
+    lng_slice scales;
+    lng_slice y;
+    uint64_t rows;
+} lng_q8_matrix;
+int lng_hip_gemm_q8_0_many(lng_batch *batch, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
+                           uint64_t cols, uint64_t n, uint64_t x_stride);
+
 /* Deterministic synthetic data written on the device (benchmarks and full-size tests):
  * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
  * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The

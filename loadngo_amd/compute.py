@@ -79,6 +79,10 @@ class _PrepareBuffers(ctypes.Structure):
                [(n, ctypes.POINTER(_Slice)) for n in ("q_bias", "k_bias", "v_bias")]
 
 
+class _Q8Matrix(ctypes.Structure):
+    _fields_ = [("codes", _Slice), ("scales", _Slice), ("y", _Slice), ("rows", ctypes.c_uint64)]
+
+
 class _Completed(ctypes.Structure):
     _fields_ = [("status", ctypes.c_int), ("gpu_seconds", ctypes.c_double), ("message", ctypes.c_char_p)]
 
@@ -128,6 +132,7 @@ SYMBOLS = {
     "lng_hip_gemm_q8_0": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_gemm_q8_0_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_gemm_q8_0_bf16": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
+    "lng_hip_gemm_q8_0_many": (ctypes.c_int, [_P, ctypes.POINTER(_Q8Matrix), ctypes.c_size_t, _Slice, _U64, _U64, _U64]),
     "lng_hip_prepare_attention": (ctypes.c_int, [_P, ctypes.POINTER(_PrepareBuffers), ctypes.POINTER(_PrepareItem),
                                                  ctypes.c_size_t, _U64, _U64, _U64, _U64, ctypes.c_int]),
 }
@@ -471,6 +476,15 @@ class Batch:
         codes, scales = matrix
         _check(library().lng_hip_gemm_q8_0_bf16(self._h, codes._c(), scales._c(), x._c(), y._c(), rows, cols, n,
                                                 strides[0], strides[1]))
+
+    def gemm_q8_0_many(self, matrices, x, cols, n, x_stride):
+        """Up to four Q8_0 products of the same positions (no counterpart in the reference, which records one
+        per matrix: gpu.rs:724-732): ``matrices`` is a list of ``((codes, scales), y, rows)``, each y dense
+        [n][rows]; one dispatch below 32 positions."""
+        arr = (_Q8Matrix * len(matrices))()
+        for slot, ((codes, scales), y, rows) in zip(arr, matrices):
+            slot.codes, slot.scales, slot.y, slot.rows = codes._c(), scales._c(), y._c(), rows
+        _check(library().lng_hip_gemm_q8_0_many(self._h, arr, len(matrices), x._c(), cols, n, x_stride))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))

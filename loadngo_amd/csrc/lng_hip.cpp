@@ -1365,11 +1365,16 @@ int reserve_x(lng_gpu *g, size_t bytes, char **out) {
     return LNG_OK;
 }
 
-// The three Q8_0 products share their checks (apple.rs:1792-1883) and their kernels.
+// The Q8_0 products share their checks (apple.rs:1792-1883) and their kernels.
 // x_bf16: the positions are bf16 (exact as one operand plane: no split, one matrix instruction per block).
-int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, const lng_slice &x, const lng_slice &y,
-               uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled,
-               bool x_bf16 = false) {
+struct Q8Checked {
+    lng_k_q8 a{};
+    Operand codes{}, scales{}, x{}, y{};
+};
+
+int q8_check(lng_batch *b, const lng_slice &codes, const lng_slice &scales, const lng_slice &x, const lng_slice &y,
+             uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled,
+             bool x_bf16, Q8Checked *out) {
     if (int rc = need_recording(b)) return rc;
     if (tiled && (rows % 64 != 0 || cols % 32 != 0 || n % 32 != 0)) { // apple.rs:1868-1872
         return fail(LNG_ERR_DISPATCH, "tiled Q8_0 product needs rows %% 64, cols %% 32 and n %% 32 == 0: %llu x %llu, n %llu",
@@ -1387,53 +1392,67 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
         if (!fits_u32(v)) return fail(LNG_ERR_DISPATCH, "too large");
     }
     if (cols % 32 != 0) return fail(LNG_ERR_DISPATCH, "Q8_0 rows of %llu are not whole blocks", (unsigned long long)cols); // apple.rs:1799-1803
-    Operand oc, os, ox, oy;
-    if (int rc = check_slice(b, "codes", codes, rows * cols, 16, &oc)) return rc;
-    if (int rc = check_slice(b, "scales", scales, rows * cols / 32 * 2, 2, &os)) return rc;
-    if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * (x_bf16 ? 2 : 4), 16, &ox)) return rc;
-    if (int rc = check_slice(b, "y", y, ((n - 1) * y_stride + rows) * 4, 4, &oy)) return rc;
-    if (int rc = check_output(b, oy, {&oc, &os, &ox})) return rc;
-    lng_k_q8 a{};
-    a.codes = (const int8_t *)((const char *)oc.buf->ptr + codes.offset);
-    a.scales = (const uint16_t *)((const char *)os.buf->ptr + scales.offset);
-    a.x = (const float *)((const char *)ox.buf->ptr + x.offset);
-    a.y = (float *)((char *)oy.buf->ptr + y.offset);
+    Q8Checked &q = *out;
+    if (int rc = check_slice(b, "codes", codes, rows * cols, 16, &q.codes)) return rc;
+    if (int rc = check_slice(b, "scales", scales, rows * cols / 32 * 2, 2, &q.scales)) return rc;
+    if (int rc = check_slice(b, "x", x, ((n - 1) * x_stride + cols) * (x_bf16 ? 2 : 4), 16, &q.x)) return rc;
+    if (int rc = check_slice(b, "y", y, ((n - 1) * y_stride + rows) * 4, 4, &q.y)) return rc;
+    if (int rc = check_output(b, q.y, {&q.codes, &q.scales, &q.x})) return rc;
+    lng_k_q8 &a = q.a;
+    a.codes = (const int8_t *)((const char *)q.codes.buf->ptr + codes.offset);
+    a.scales = (const uint16_t *)((const char *)q.scales.buf->ptr + scales.offset);
+    a.x = (const float *)((const char *)q.x.buf->ptr + x.offset);
+    a.y = (float *)((char *)q.y.buf->ptr + y.offset);
     a.rows = (uint32_t)rows;
     a.cols = (uint32_t)cols;
     a.n = (uint32_t)n;
     a.x_stride = (uint32_t)x_stride;
     a.y_stride = (uint32_t)y_stride;
-    Cmd c1;
     if (x_bf16) {
+        a.x_hi = (const uint16_t *)a.x;
         a.x = nullptr;
-        a.x_hi = (const uint16_t *)((const char *)ox.buf->ptr + x.offset);
         a.plane_stride = (uint32_t)x_stride;
     }
-    if (n < 32) {
-        // bound by reading the matrix: one pass over it per 16 positions, x split in registers
-        const bool one = n == 1 && cols <= 12288 && !x_bf16; // x of a single position is held in LDS (Q8S_X1 floats)
-        c1.fn = x_bf16 ? b->gpu->q8_stream_bf16 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
-        c1.name = x_bf16 ? "lng_q8_stream_bf16" : one ? "lng_q8_stream_one" : "lng_q8_stream";
-        c1.grid[0] = (unsigned)((rows + 15) / 16);
-        c1.grid[1] = (unsigned)((n + 15) / 16);
-        c1.block = 1024;
-    } else if (x_bf16) {
-        const uint64_t n_pad = (n + 127) / 128 * 128;
-        if (n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
+    return LNG_OK;
+}
+
+// Few positions (n < 32): bound by reading the matrix, one pass over it per 16 positions, x split in registers.
+// `a` may name further matrices of the same dispatch (a.more); row_tiles counts the tiles of all of them.
+void q8_record_stream(lng_batch *b, const lng_k_q8 &a, uint64_t row_tiles, bool x_bf16) {
+    const bool one = a.n == 1 && a.cols <= 12288 && !x_bf16; // x of a single position is held in LDS (Q8S_X1 floats)
+    Cmd c;
+    c.fn = x_bf16 ? b->gpu->q8_stream_bf16 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
+    c.name = x_bf16 ? "lng_q8_stream_bf16" : one ? "lng_q8_stream_one" : "lng_q8_stream";
+    c.grid[0] = (unsigned)row_tiles;
+    c.grid[1] = (unsigned)((a.n + 15) / 16);
+    c.block = 1024;
+    set_args(c, a);
+    b->cmds.push_back(std::move(c));
+    b->dispatches += 1;
+}
+
+// Many positions: bound by the matrix unit.
+int q8_record_tiled(lng_batch *b, lng_k_q8 a, bool x_bf16) {
+    const uint64_t n = a.n, cols = a.cols, rows = a.rows;
+    const uint64_t n_pad = (n + 127) / 128 * 128;
+    if (n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
+    // one-dimensional grid; the kernel maps ids to tiles (XCD-aware from eight position tiles on,
+    // rounded up to blocks of 8 row tiles x 4 position tiles per XCD)
+    const uint64_t row_tiles = (rows + 255) / 256, pos_tiles = n_pad / 128;
+    uint64_t ids = row_tiles * pos_tiles;
+    if (pos_tiles >= 8) {
+        const uint64_t per_xcd = (pos_tiles + 7) / 8;
+        ids = 8 * ((per_xcd + 3) / 4) * ((row_tiles + 7) / 8) * 32;
+    }
+    if (ids > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
+    Cmd c1;
+    c1.grid[0] = (unsigned)ids;
+    c1.block = 512;
+    if (x_bf16) {
         c1.fn = b->gpu->q8_tiled_bf16;
         c1.name = "lng_q8_tiled_bf16";
-        const uint64_t row_tiles = (rows + 255) / 256, pos_tiles = n_pad / 128;
-        uint64_t ids = row_tiles * pos_tiles;
-        if (pos_tiles >= 8) {
-            const uint64_t per_xcd = (pos_tiles + 7) / 8;
-            ids = 8 * ((per_xcd + 3) / 4) * ((row_tiles + 7) / 8) * 32;
-        }
-        if (ids > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
-        c1.grid[0] = (unsigned)ids;
-        c1.block = 512;
     } else {
-        const uint64_t n_pad = (n + 127) / 128 * 128;
-        if (!fits_u32(n_pad * cols) || n_pad / 128 > 65535) return fail(LNG_ERR_DISPATCH, "too large");
+        if (!fits_u32(n_pad * cols)) return fail(LNG_ERR_DISPATCH, "too large");
         char *planes = nullptr;
         if (int rc = reserve_x(b->gpu, 2 * n_pad * cols * 2, &planes)) return rc;
         lng_k_q8_split sp{};
@@ -1443,7 +1462,7 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
         sp.n = (uint32_t)n;
         sp.n_pad = (uint32_t)n_pad;
         sp.cols = (uint32_t)cols;
-        sp.x_stride = (uint32_t)x_stride;
+        sp.x_stride = a.x_stride;
         Cmd c0;
         c0.fn = b->gpu->q8_split_x;
         c0.name = "lng_q8_split_x";
@@ -1456,22 +1475,23 @@ int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, co
         a.plane_stride = (uint32_t)cols;
         c1.fn = b->gpu->q8_tiled;
         c1.name = "lng_q8_tiled";
-        // one-dimensional grid; the kernel maps ids to tiles (XCD-aware from eight position tiles on,
-        // rounded up to blocks of 8 row tiles x 4 position tiles per XCD)
-        const uint64_t row_tiles = (rows + 255) / 256, pos_tiles = n_pad / 128;
-        uint64_t ids = row_tiles * pos_tiles;
-        if (pos_tiles >= 8) {
-            const uint64_t per_xcd = (pos_tiles + 7) / 8;
-            ids = 8 * ((per_xcd + 3) / 4) * ((row_tiles + 7) / 8) * 32;
-        }
-        if (ids > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
-        c1.grid[0] = (unsigned)ids;
-        c1.block = 512;
     }
     set_args(c1, a);
     b->cmds.push_back(std::move(c1));
     b->dispatches += 1;
     return LNG_OK;
+}
+
+int q8_product(lng_batch *b, const lng_slice &codes, const lng_slice &scales, const lng_slice &x, const lng_slice &y,
+               uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride, bool gemm, bool tiled,
+               bool x_bf16 = false) {
+    Q8Checked q;
+    if (int rc = q8_check(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, gemm, tiled, x_bf16, &q)) return rc;
+    if (n < 32) {
+        q8_record_stream(b, q.a, (rows + 15) / 16, x_bf16);
+        return LNG_OK;
+    }
+    return q8_record_tiled(b, q.a, x_bf16);
 }
 
 } // namespace
@@ -1495,6 +1515,55 @@ extern "C" int lng_hip_gemm_q8_0_tiled(lng_batch *b, lng_slice codes, lng_slice 
 extern "C" int lng_hip_gemm_q8_0_bf16(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, lng_slice y,
                                       uint64_t rows, uint64_t cols, uint64_t n, uint64_t x_stride, uint64_t y_stride) {
     return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, false, true);
+}
+
+extern "C" int lng_hip_gemm_q8_0_many(lng_batch *b, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
+                                      uint64_t cols, uint64_t n, uint64_t x_stride) {
+    if (int rc = need_recording(b)) return rc;
+    if (!matrices || n_matrices == 0 || n_matrices > 1 + LNG_Q8_MORE) {
+        return fail(LNG_ERR_DISPATCH, "%zu matrices: one dispatch takes 1 to %d", n_matrices, 1 + LNG_Q8_MORE);
+    }
+    Q8Checked q[1 + LNG_Q8_MORE];
+    for (size_t i = 0; i < n_matrices; ++i) {
+        const lng_q8_matrix &m = matrices[i];
+        if (int rc = q8_check(b, m.codes, m.scales, x, m.y, m.rows, cols, n, x_stride, m.rows, true, false, false, &q[i])) {
+            return fail(rc, "matrix %zu: %s", i, std::string(g_error).c_str());
+        }
+    }
+    for (size_t i = 0; i < n_matrices; ++i) { // no product's output may share bytes with another's output or inputs
+        for (size_t j = 0; j < n_matrices; ++j) {
+            if (i == j) continue;
+            if (overlaps(q[i].y, q[j].y)) return fail(LNG_ERR_DISPATCH, "outputs of matrices %zu and %zu overlap", i, j);
+            if (overlaps(q[i].y, q[j].codes) || overlaps(q[i].y, q[j].scales)) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+        }
+    }
+    if (n >= 32) { // the matrix unit is the bound there, not the launches: one product after the other
+        const size_t cmds = b->cmds.size(), dispatches = b->dispatches;
+        for (size_t i = 0; i < n_matrices; ++i) {
+            if (int rc = q8_record_tiled(b, q[i].a, false)) {
+                b->cmds.resize(cmds); // a refused dispatch leaves nothing behind
+                b->dispatches = dispatches;
+                return rc;
+            }
+        }
+        return LNG_OK;
+    }
+    lng_k_q8 a = q[0].a;
+    uint64_t tiles = (a.rows + 15) / 16;
+    a.n_more = (uint32_t)(n_matrices - 1);
+    for (size_t i = 1; i < n_matrices; ++i) {
+        auto &m = a.more[i - 1];
+        m.codes = q[i].a.codes;
+        m.scales = q[i].a.scales;
+        m.y = q[i].a.y;
+        m.rows = q[i].a.rows;
+        m.y_stride = q[i].a.y_stride;
+        m.first_tile = (uint32_t)tiles;
+        tiles += (q[i].a.rows + 15) / 16;
+    }
+    if (!fits_u32(tiles) || tiles > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
+    q8_record_stream(b, a, tiles, false);
+    return LNG_OK;
 }
 
 extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, uint64_t seed, float scale,

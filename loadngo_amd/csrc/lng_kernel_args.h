@@ -156,7 +156,21 @@ typedef struct lng_k_q8 {
     uint32_t y_stride;
     uint32_t plane_stride;   /* elements between positions of x_hi / x_lo: cols for the split planes; x's own stride
                                 when the positions are bf16 already (x_hi = x, no x_lo, n rows only) */
+    /* Few positions only: further matrices of the same dispatch, multiplied by the same x (same cols, n).
+     * Workgroups from `first_tile` (in units of 16 rows) on belong to matrix more[i]; first_tile ascends. */
+    uint32_t n_more;         /* 0..LNG_Q8_MORE */
+    uint32_t pad_;
+    struct lng_k_q8_more {
+        const int8_t *codes;
+        const uint16_t *scales;
+        float *y;
+        uint32_t rows;
+        uint32_t y_stride;
+        uint32_t first_tile;
+        uint32_t pad_;
+    } more[3];
 } lng_k_q8;
+#define LNG_Q8_MORE 3
 
 /* Synthetic element i: z = splitmix64 finaliser of (i' + seed * 0x9E3779B97F4A7C15) with
  * i' = period ? i % period : i; s = sum of the four 16-bit fields of z; value =

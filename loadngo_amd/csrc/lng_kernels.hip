@@ -1037,14 +1037,31 @@ __device__ __forceinline__ void q8_split8(const float (&x)[8], bf16x8 &hi, bf16x
 #define Q8S_UNROLL 8 // blocks in flight per wavefront: 128 blocks (4096 columns) in one turn
 #define Q8S_X1 12288 // floats of x held in LDS by the one-position form (48 KB)
 #define Q8S_SC_BLOCKS 512 // rows of up to this many blocks (16,384 columns) have their scales staged through LDS
-template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a) {
+// The matrix a workgroup of a several-matrix dispatch works on becomes the one `a` names; returns its row tile.
+__device__ __forceinline__ uint32_t q8_select_matrix(lng_k_q8 &a) {
+    uint32_t tile = blockIdx.x;
+#pragma unroll
+    for (int i = 0; i < LNG_Q8_MORE; ++i) {
+        if ((uint32_t)i < a.n_more && blockIdx.x >= a.more[i].first_tile) { // uniform: scalar selects
+            a.codes = a.more[i].codes;
+            a.scales = a.more[i].scales;
+            a.y = a.more[i].y;
+            a.rows = a.more[i].rows;
+            a.y_stride = a.more[i].y_stride;
+            tile = blockIdx.x - a.more[i].first_tile;
+        }
+    }
+    return tile;
+}
+
+template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a, uint32_t tile) {
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
     __shared__ __attribute__((aligned(16))) float s_x1[ONE ? Q8S_X1 : 4];
     __shared__ __attribute__((aligned(4))) uint16_t s_sc[16 * Q8S_SC_BLOCKS];
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
-    const uint32_t r0 = blockIdx.x * 16u, p0 = blockIdx.y * 16u;
+    const uint32_t r0 = tile * 16u, p0 = blockIdx.y * 16u;
     const uint32_t row = r0 + j < a.rows ? r0 + j : a.rows - 1u;
     const uint32_t pos = p0 + j < a.n ? p0 + j : a.n - 1u; // rows of the product past n are not stored
     const uint32_t blocks = a.cols / 32u;
@@ -1134,16 +1151,19 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
 }
 
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k_q8 a) {
-    q8_stream_body<false>(a);
+    const uint32_t tile = q8_select_matrix(a);
+    q8_stream_body<false>(a, tile);
 }
 
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_one(lng_k_q8 a) {
-    q8_stream_body<true>(a);
+    const uint32_t tile = q8_select_matrix(a);
+    q8_stream_body<true>(a, tile);
 }
 
 // positions already in bf16 (the output of a bf16 attention): one matrix instruction per block
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_bf16(lng_k_q8 a) {
-    q8_stream_body<false, true>(a);
+    const uint32_t tile = q8_select_matrix(a);
+    q8_stream_body<false, true>(a, tile);
 }
 
 // Many positions (bound by the matrix unit): a workgroup of eight wavefronts takes 256 rows x 128

@@ -2,7 +2,7 @@
 // against the sequence of reference operators it stands for:
 //   * attention_decode_batched == one attention_grouped_with_sinks (t = 1) per sequence (gpt-oss/src/gpu.rs:794-805);
 //   * prepare_attention == add_rows x 3, rotate_halves x 2 and copy_rows into the ring (gpu.rs:733-759), bit for bit in f32;
-//   * gemm_q8_0_bf16 == gemm_q8_0 on positions that are exact in bf16.
+//   * gemm_q8_0_bf16 == gemm_q8_0 on positions that are exact in bf16; gemm_q8_0_many == one gemm_q8_0 per matrix.
 //
 // Prints one line per test and exits with the number of failures.
 #include <cmath>
@@ -171,13 +171,27 @@ void q8_product_of_bf16_positions_is_the_f32_product(const Gpu &gpu) {
         buffers.push_back(std::move(narrow));
         buffers.push_back(gpu.buffer(n * rows * 4));
         buffers.push_back(gpu.buffer(n * rows * 4));
+        buffers.push_back(gpu.buffer(n * rows * 4)); // 6: the two halves
         Batch batch = gpu.batch(std::move(buffers));
         const std::pair<Slice, Slice> matrix{Slice(0, 0, codes.size()), Slice(1, 0, scales.size())};
         batch.gemm_q8_0(matrix, f32s(2, x.size()), f32s(4, n * rows), {rows, cols}, n, {cols, rows});
         batch.gemm_q8_0_bf16(matrix, Slice(3, 0, xb.size() * 2), f32s(5, n * rows), {rows, cols}, n, {cols, rows});
+        // the same matrix as two matrices of 160 rows each through the several-matrices form: the same bits
+        const size_t h = rows / 2;
+        batch.gemm_q8_0_many({{{Slice(0, 0, h * cols), Slice(1, 0, h * cols / 16)}, Slice(6, 0, n * h * 4), h},
+                              {{Slice(0, h * cols, h * cols), Slice(1, h * cols / 16, h * cols / 16)}, Slice(6, n * h * 4, n * h * 4), h}},
+                             f32s(2, x.size()), cols, n, cols);
         Completed done = std::move(batch).run();
         done.gpu_time();
-        const std::vector<float> wide = done.buffers[4].to_f32(), narrow_y = done.buffers[5].to_f32();
+        const std::vector<float> wide = done.buffers[4].to_f32(), narrow_y = done.buffers[5].to_f32(), halves = done.buffers[6].to_f32();
+        bool same_bits = true;
+        for (size_t p = 0; p < n; ++p) {
+            for (size_t r = 0; r < rows; ++r) {
+                const float split = r < h ? halves[p * h + r] : halves[n * h + p * h + (r - h)];
+                same_bits = same_bits && std::memcmp(&split, &wide[p * rows + r], 4) == 0;
+            }
+        }
+        expect(same_bits, std::to_string(n) + " positions: two half matrices in one call give the bits of the whole product");
         double worst = 0.0, largest = 0.0;
         for (size_t i = 0; i < wide.size(); ++i) {
             largest = std::max(largest, (double)std::fabs(wide[i]));

@@ -236,3 +236,50 @@ def test_tiny_model_golden_with_device_projections(gpu, chunk):
             codes.free()
             scales.free()
     assert np.abs(got - want).max() < TOLERANCE
+
+
+@pytest.mark.parametrize("n", [1, 5, 16, 17, 31, 40])
+def test_several_matrices_in_one_dispatch_give_the_separate_products(gpu, n):
+    """The q, k and v projections of a layer (gpu.rs:724-732 records three products) as one call: bit for bit
+    the three separate gemm_q8_0 products, in one dispatch below 32 positions (three from 32 on); rows that are
+    not a multiple of 16, a fourth matrix, and the refusals."""
+    cols = 2880
+    shapes = [(4096, 21), (512, 22), (37, 23), (528, 24)]
+    mats = [q8_test_matrix(rows, cols, seed)[:2] for rows, seed in shapes]
+    x = xorshift_values(31 + n, n * cols).reshape(n, cols)
+    bufs = [gpu.upload(x)]
+    for codes, bits in mats:
+        bufs += [gpu.upload(codes), gpu.upload(bits)]
+    y_lens = [n * rows * 4 for rows, _ in shapes]
+    bufs += [gpu.buffer(2 * sum(y_lens))]                   # all outputs, once per way of computing them
+    bufs[-1].fill(0xFF)
+    batch = gpu.batch(bufs)
+    xs = C.Slice(0, 0, x.nbytes)
+    many, offset = [], 0
+    for i, ((rows, _), (codes, bits)) in enumerate(zip(shapes, mats)):
+        m = (C.Slice(1 + 2 * i, 0, codes.nbytes), C.Slice(2 + 2 * i, 0, bits.nbytes))
+        many.append((m, C.Slice(9, offset, y_lens[i]), rows))
+        batch.gemm_q8_0(m, xs, C.Slice(9, sum(y_lens) + offset, y_lens[i]), rows, cols, n, (cols, rows))
+        offset += y_lens[i]
+    before = batch.dispatches()
+    batch.gemm_q8_0_many(many, xs, cols, n, cols)
+    assert batch.dispatches() - before == (1 if n < 32 else 4)
+    # refusals: nothing is recorded
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many(many + many[:1], xs, cols, n, cols)                       # five matrices
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many([], xs, cols, n, cols)
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many([many[0], (many[1][0], many[0][1], many[0][2])], xs, cols, n, cols)   # same output twice
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many([many[0], (many[1][0], many[1][1], 513)], xs, cols, n, cols)          # rows do not fit the slices
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many([(many[0][0], C.Slice(1, 0, y_lens[0]), 4096)], xs, cols, n, cols)     # output over a matrix
+    assert batch.dispatches() - before == (1 if n < 32 else 4)
+    batch.run()
+    raw = bufs[-1].read(np.float32)
+    batch.drop()
+    for b in bufs:
+        b.free()
+    together, apart = raw[:raw.size // 2], raw[raw.size // 2:]
+    assert not np.isnan(together).any() and np.array_equal(together, apart)
