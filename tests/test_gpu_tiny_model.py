@@ -155,9 +155,9 @@ class DeviceBlocks:
     output projection, its bias, the residual add into H. The host only uploads H and the rotary table and reads
     H back (the experts stay in numpy)."""
 
-    def __init__(self, gpu, model, chunk, tiled):
+    def __init__(self, gpu, model, chunk, tiled, qkv_together=False):
         m = self.m = model
-        self.gpu, self.chunk, self.tiled = gpu, chunk, tiled
+        self.gpu, self.chunk, self.tiled, self.qkv_together = gpu, chunk, tiled, qkv_together
         self.qw, self.kw = m.heads * m.dim, m.kv_heads * m.dim
         self.pad = pad = (chunk + 31) // 32 * 32
         self.slots = [((m.window + chunk + 31) // 32 * 32) if m.is_sliding(l) else 64 for l in range(m.layers_n)]
@@ -210,9 +210,16 @@ class DeviceBlocks:
 
         batch.copy_rows((rows_of(H, hidden), hidden), (rows_of(X, hidden), hidden), n, hidden)
         batch.rmsnorm_rows((rows_of(X, hidden), batch.attach(r["attn_norm"])), n, (hidden, hidden), m.eps)
-        mul("q", X, Q)
-        mul("k", X, K)
-        mul("v", X, V)
+        if self.qkv_together:  # the three projections as one call (one dispatch below 32 positions)
+            mats = []
+            for part, y in (("q", Q), ("k", K), ("v", V)):
+                codes, scales, rows, cols = r[part]
+                mats.append(((batch.attach(codes), batch.attach(scales)), rows_of(y, rows, n_run), rows))
+            batch.gemm_q8_0_many(mats, rows_of(X, cols, n_run), cols, n_run, cols)
+        else:
+            mul("q", X, Q)
+            mul("k", X, K)
+            mul("v", X, V)
         item = C.PrepareItem(n=n, start=start, slots=self.slots[l])
         batch.prepare_attention(dict(q=Q, k=K, v=V, table=TABLE, q_out=QR, k_cache=KC, v_cache=VC), [item], m.heads,
                                 m.kv_heads, m.dim, m.dim, C.F32, batch.attach(r["q_bias"]), batch.attach(r["k_bias"]),
@@ -247,10 +254,11 @@ class DeviceBlocks:
                     b.free()
 
 
-@pytest.mark.parametrize("chunk,tiled", [(1, False), (9, False), (40, False), (40, True)])
-def test_whole_attention_blocks_on_the_device_match_transformers(gpu, model, chunk, tiled):
+@pytest.mark.parametrize("chunk,tiled,qkv_together", [(1, False, False), (9, False, False), (40, False, False), (40, True, False),
+                                                      (1, False, True), (9, False, True), (40, True, True)])
+def test_whole_attention_blocks_on_the_device_match_transformers(gpu, model, chunk, tiled, qkv_together):
     ids, want = tm.load_fixture(FIXTURE)
-    s = DeviceBlocks(gpu, model, chunk, tiled)
+    s = DeviceBlocks(gpu, model, chunk, tiled, qkv_together)
     try:
         got = model.forward(ids, None, None, chunk=chunk, block=s.block)
     finally:
