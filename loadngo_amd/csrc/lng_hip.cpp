@@ -89,7 +89,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr;
     hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
-    hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr;
+    hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
     hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
                   q8_tiled_bf16 = nullptr;
@@ -691,6 +691,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_q8_tiled_bf16", &g->q8_tiled_bf16, true},
         {"lng_q8_stream_bf16", &g->q8_stream_bf16, true},
         {"lng_rmsnorm_rows", &g->rmsnorm_rows, true},
+        {"lng_rmsnorm_row_wg", &g->rmsnorm_row_wg, true},
     };
     for (auto &w : wanted) {
         e = hipModuleGetFunction(w.fn, g->module, w.name);
@@ -1136,9 +1137,10 @@ extern "C" int lng_hip_rmsnorm_rows(lng_batch *b, lng_slice v, lng_slice w, uint
     a.stride = (uint32_t)stride;
     a.eps = eps;
     Cmd c;
-    c.fn = b->gpu->rmsnorm_rows;
-    c.name = "lng_rmsnorm_rows";
-    c.grid[0] = (unsigned)((rows + 3) / 4);
+    const bool wide = d > 256 && d <= 4096; // a workgroup per row, elements held in registers; else a wavefront per row
+    c.fn = wide ? b->gpu->rmsnorm_row_wg : b->gpu->rmsnorm_rows;
+    c.name = wide ? "lng_rmsnorm_row_wg" : "lng_rmsnorm_rows";
+    c.grid[0] = wide ? (unsigned)rows : (unsigned)((rows + 3) / 4);
     c.block = 256;
     set_args(c, a);
     b->cmds.push_back(std::move(c));

@@ -819,6 +819,36 @@ extern "C" __global__ __launch_bounds__(256) void lng_rmsnorm_rows(lng_k_rmsnorm
     for (i = lane; i < a.d; i += 64u) x[i] = x[i] * scale * a.w[i];
 }
 
+// The same operator with a workgroup per row, for rows of 257..4096 floats: every thread requests its (up to 16)
+// elements and weights at once and keeps the elements in registers between the sum and the scaling, so a row
+// costs two memory round trips instead of one per 64 elements (one decoding row of 2,880 floats: 14 -> 7 us).
+extern "C" __global__ __launch_bounds__(256) void lng_rmsnorm_row_wg(lng_k_rmsnorm a) {
+#pragma clang fp contract(off)
+    __shared__ float s_part[4];
+    float *x = a.v + (uint64_t)blockIdx.x * a.stride;
+    float v[16], w[16];
+    float ss = 0.0f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const uint32_t i = threadIdx.x + 256u * u;
+        v[u] = i < a.d ? x[i] : 0.0f;
+        w[u] = i < a.d ? a.w[i] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) ss += v[u] * v[u];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((threadIdx.x & 63u) == 0) s_part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+    const float scale = 1.0f / sqrtf(ss / (float)a.d + a.eps);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const uint32_t i = threadIdx.x + 256u * u;
+        if (i < a.d) x[i] = v[u] * scale * w[u];
+    }
+}
+
 // Batch::add_rows (apple.rs:1886-1911; kernels.metal:1648-1660). One thread per element.
 extern "C" __global__ __launch_bounds__(256) void lng_add_rows(lng_k_add a) {
     const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
