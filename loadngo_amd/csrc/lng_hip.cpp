@@ -478,6 +478,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         Cmd m;
         m.fn = g->decode_merge;
         m.name = "lng_decode_merge";
+        m.grid[0] = group; // a workgroup per (row, kv head, query head)
         m.grid[1] = (unsigned)(n_rows * a.kv_heads);
         m.block = 256;
         set_args(m, a);

@@ -749,9 +749,15 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
     }
 }
 
-// The same merge as its own dispatch, for large grids: there a workgroup that waits for its
-// coherent stores and its ticket holds a compute unit's slot that another chunk could use.
+// The merge as its own dispatch, for large grids (there a workgroup that waits for its coherent stores and
+// its ticket holds a compute unit's slot that another chunk could use) and for the f32 kernel. One workgroup
+// per (row, kv head, query head): thread c turns chunk c's (max, sum) into a weight, then thread (dim, quarter)
+// adds every fourth chunk's partial output and the quarters meet in LDS: eight times the workgroups of a
+// merge per (row, kv head) and a quarter of the chain of loads per thread.
 extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a) {
+    __shared__ float s_w[LNG_MAX_CHUNKS];
+    __shared__ float s_red[2][4];
+    __shared__ float s_acc[4][64];
     const uint32_t row = blockIdx.y / a.kv_heads;
     const uint32_t g = blockIdx.y % a.kv_heads;
     const lng_k_row it = row_of(a, row);
@@ -759,7 +765,55 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a)
     const uint64_t base = first_visible(last, it.window) & ~(uint64_t)31;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
     if (row_chunks == 1) return; // the decode kernel already wrote this row
-    merge_chunks<false>(a, it, g, a.heads / a.kv_heads, row_chunks);
+    const uint32_t group = a.heads / a.kv_heads, h = blockIdx.x, head = g * group + h;
+    const uint32_t tid = threadIdx.x, wave = tid >> 6;
+    const uint64_t slot0 = ((uint64_t)blockIdx.y * a.n_chunks) * group + h;
+    const float sink2 = it.sinks_offset != LNG_NO_SINKS ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                                         : LNG_NEG_INF;
+    float mc = LNG_NEG_INF, lc = 0.0f;
+    if (tid < row_chunks) {
+        const float2 ml = *(const float2 *)(a.partial_ml + (slot0 + (uint64_t)tid * group) * 2u);
+        mc = ml.x;
+        lc = ml.y;
+    }
+    float top = fmaxf(mc, sink2);
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) top = fmaxf(top, __shfl_xor(top, s, 64));
+    if ((tid & 63u) == 0) s_red[0][wave] = top;
+    __syncthreads();
+    top = fmaxf(fmaxf(s_red[0][0], s_red[0][1]), fmaxf(s_red[0][2], s_red[0][3]));
+    const float wt = mc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(mc - top);
+    if (tid < row_chunks) s_w[tid] = wt;
+    float z = lc * wt;
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) z += __shfl_xor(z, s, 64);
+    if ((tid & 63u) == 0) s_red[1][wave] = z;
+    __syncthreads();
+    z = (s_red[1][0] + s_red[1][1]) + (s_red[1][2] + s_red[1][3]) +
+        (sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top));
+    const uint32_t d = tid & 63u;
+    const float *po = a.partial_o + slot0 * 64u + d;
+    const uint64_t step = (uint64_t)group * 64u;
+    float o = 0.0f;
+    uint32_t c = wave;
+    for (; c + 28u < row_chunks; c += 32u) { // eight loads in flight per turn
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = po[(c + 4u * u) * step];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o += x[u] * s_w[c + 4u * u];
+    }
+    for (; c < row_chunks; c += 4u) o += po[c * step] * s_w[c];
+    s_acc[wave][d] = o;
+    __syncthreads();
+    if (wave != 0) return;
+    const float res = ((s_acc[0][d] + s_acc[1][d]) + (s_acc[2][d] + s_acc[3][d])) / z;
+    const uint64_t at = (uint64_t)head * 64u + d;
+    if (a.dtype == LNG_F32) {
+        ((float *)(a.out + it.out_offset))[at] = res;
+    } else {
+        ((uint16_t *)(a.out + it.out_offset))[at] = f32_to_bf16_bits(res);
+    }
 }
 
 // =============================================================================================
