@@ -1,5 +1,5 @@
 """The C ABI from plain C: tests/c_abi/decode_once.c includes only include/lng_hip.h, links only
-liblng_hip.so, and is what a foreign-function binding (the Rust crate sketched in INTEGRATION.md)
+liblng_hip.so, and is what a foreign-function binding (a Rust crate over this C ABI)
 would do. Without a GPU it must compile and link; with one it must run and agree with itself."""
 import os
 import subprocess
