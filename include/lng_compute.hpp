@@ -287,6 +287,23 @@ class Batch {
         for (const Q8Matrix &m : matrices) raw.push_back(lng_q8_matrix{m.matrix.first.c(), m.matrix.second.c(), m.y.c(), m.rows});
         detail::check(lng_hip_gemm_q8_0_many(h_, raw.data(), raw.size(), x.c(), cols, n, x_stride));
     }
+    // gemm_q8_0_many of RMS-normalised positions (x itself is left alone): copy_rows + rmsnorm_rows + the products
+    // of gpu.rs:712-732 in one dispatch; fewer than 32 positions.
+    void gemm_q8_0_many_normed(const std::vector<Q8Matrix> &matrices, Slice x, std::pair<Slice, float> norm, std::size_t cols,
+                               std::size_t n, std::size_t x_stride) {
+        std::vector<lng_q8_matrix> raw;
+        for (const Q8Matrix &m : matrices) raw.push_back(lng_q8_matrix{m.matrix.first.c(), m.matrix.second.c(), m.y.c(), m.rows});
+        detail::check(lng_hip_gemm_q8_0_many_normed(h_, raw.data(), raw.size(), x.c(), norm.first.c(), norm.second, cols, n, x_stride));
+    }
+    // h += W x + bias: the product, add_rows of the bias and add_rows into the hidden state (gpu.rs:807-827) in one
+    // dispatch and with their bits; fewer than 32 positions; strides = (x_stride, h_stride).
+    void gemm_q8_0_residual(std::pair<Slice, Slice> matrix, Slice x, const Slice *bias, Slice h, std::pair<std::size_t, std::size_t> rows_cols,
+                            std::size_t n, std::pair<std::size_t, std::size_t> strides, DType x_dtype = DType::F32) {
+        lng_slice b{};
+        if (bias) b = bias->c();
+        detail::check(lng_hip_gemm_q8_0_residual(h_, matrix.first.c(), matrix.second.c(), x.c(), (int)x_dtype, bias ? &b : nullptr, h.c(),
+                                                 rows_cols.first, rows_cols.second, n, strides.first, strides.second));
+    }
     // No counterpart in the reference: one decoding query per item, many sequences in one dispatch.
     void attention_decode_batched(std::size_t q_buffer, std::size_t k_buffer, std::size_t v_buffer, std::size_t out_buffer,
                                   std::size_t sinks_buffer, const std::vector<DecodeItem> &items, std::size_t heads,

@@ -305,6 +305,23 @@ typedef struct lng_q8_matrix {
 int lng_hip_gemm_q8_0_many(lng_batch *batch, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
                            uint64_t cols, uint64_t n, uint64_t x_stride);
 
+/* The same with the RMS norm of the positions folded in (no counterpart in the reference, which copies the
+ * hidden state, normalises the copy in place and then multiplies: gpu.rs:712-732): y_i[p] = W_i x'[p] with
+ * x'[p][c] = (x[p][c] / sqrt(mean_c(x[p]^2) + eps)) * norm_w[c], the arithmetic of lng_hip_rmsnorm_rows; x is
+ * left as it is. norm_w holds cols f32 on a 16-byte boundary. For decoding only: fewer than 32 positions of up
+ * to 12288 columns (refused otherwise: prompt passes are bound by the matrix unit and take the separate calls). */
+int lng_hip_gemm_q8_0_many_normed(lng_batch *batch, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
+                                  lng_slice norm_w, float eps, uint64_t cols, uint64_t n, uint64_t x_stride);
+
+/* The output projection with its bias and the residual add folded in (no counterpart in the reference, which
+ * records the product, add_rows of the bias and add_rows into the hidden state: gpu.rs:807-827):
+ * h[p] = h[p] + ((W x[p]) + bias), every sum rounded as those three dispatches round it, so the result is theirs
+ * bit for bit. x is f32 or bf16 (x_dtype; strides as in lng_hip_gemm_q8_0 / _bf16), bias rows f32 or NULL, h f32
+ * with h_stride >= rows. For decoding only: fewer than 32 positions (refused otherwise). */
+int lng_hip_gemm_q8_0_residual(lng_batch *batch, lng_slice codes, lng_slice scales, lng_slice x, int x_dtype,
+                               const lng_slice *bias, lng_slice h, uint64_t rows, uint64_t cols, uint64_t n,
+                               uint64_t x_stride, uint64_t h_stride);
+
 /* Deterministic synthetic data written on the device (benchmarks and full-size tests):
  * element i of the slice gets g((seed, i mod period)) * scale, g a fixed integer hash mapped
  * to a centred sum of four uniforms (variance 1); period == 0 means no repetition. The

@@ -133,6 +133,10 @@ SYMBOLS = {
     "lng_hip_gemm_q8_0_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_gemm_q8_0_bf16": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_gemm_q8_0_many": (ctypes.c_int, [_P, ctypes.POINTER(_Q8Matrix), ctypes.c_size_t, _Slice, _U64, _U64, _U64]),
+    "lng_hip_gemm_q8_0_many_normed": (ctypes.c_int, [_P, ctypes.POINTER(_Q8Matrix), ctypes.c_size_t, _Slice, _Slice,
+                                                     ctypes.c_float, _U64, _U64, _U64]),
+    "lng_hip_gemm_q8_0_residual": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, ctypes.c_int, ctypes.POINTER(_Slice), _Slice,
+                                                  _U64, _U64, _U64, _U64, _U64]),
     "lng_hip_prepare_attention": (ctypes.c_int, [_P, ctypes.POINTER(_PrepareBuffers), ctypes.POINTER(_PrepareItem),
                                                  ctypes.c_size_t, _U64, _U64, _U64, _U64, ctypes.c_int]),
 }
@@ -485,6 +489,24 @@ class Batch:
         for slot, ((codes, scales), y, rows) in zip(arr, matrices):
             slot.codes, slot.scales, slot.y, slot.rows = codes._c(), scales._c(), y._c(), rows
         _check(library().lng_hip_gemm_q8_0_many(self._h, arr, len(matrices), x._c(), cols, n, x_stride))
+
+    def gemm_q8_0_many_normed(self, matrices, x, norm, cols, n, x_stride):
+        """``gemm_q8_0_many`` of the RMS-normalised positions (``norm`` = (weights slice, eps)); x is not changed.
+        Replaces copy_rows + rmsnorm_rows + the products of gpu.rs:712-732; fewer than 32 positions."""
+        arr = (_Q8Matrix * len(matrices))()
+        for slot, ((codes, scales), y, rows) in zip(arr, matrices):
+            slot.codes, slot.scales, slot.y, slot.rows = codes._c(), scales._c(), y._c(), rows
+        w, eps = norm
+        _check(library().lng_hip_gemm_q8_0_many_normed(self._h, arr, len(matrices), x._c(), w._c(), eps, cols, n, x_stride))
+
+    def gemm_q8_0_residual(self, matrix, x, bias, h, rows, cols, n, strides, x_dtype=F32):
+        """h += W x + bias in one dispatch, bit for bit gemm_q8_0 + add_rows(bias) + add_rows(residual) of
+        gpu.rs:807-827; x f32 or bf16; fewer than 32 positions. ``strides`` = (x_stride, h_stride)."""
+        codes, scales = matrix
+        held = None if bias is None else bias._c()
+        _check(library().lng_hip_gemm_q8_0_residual(self._h, codes._c(), scales._c(), x._c(), x_dtype,
+                                                    None if held is None else ctypes.pointer(held), h._c(), rows, cols, n,
+                                                    strides[0], strides[1]))
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))

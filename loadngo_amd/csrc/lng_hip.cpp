@@ -1520,8 +1520,45 @@ extern "C" int lng_hip_gemm_q8_0_bf16(lng_batch *b, lng_slice codes, lng_slice s
     return q8_product(b, codes, scales, x, y, rows, cols, n, x_stride, y_stride, true, false, true);
 }
 
+namespace {
+int q8_many(lng_batch *b, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x, const lng_slice *norm_w, float eps,
+            uint64_t cols, uint64_t n, uint64_t x_stride);
+}
+
 extern "C" int lng_hip_gemm_q8_0_many(lng_batch *b, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
                                       uint64_t cols, uint64_t n, uint64_t x_stride) {
+    return q8_many(b, matrices, n_matrices, x, nullptr, 0.0f, cols, n, x_stride);
+}
+
+extern "C" int lng_hip_gemm_q8_0_many_normed(lng_batch *b, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x,
+                                             lng_slice norm_w, float eps, uint64_t cols, uint64_t n, uint64_t x_stride) {
+    return q8_many(b, matrices, n_matrices, x, &norm_w, eps, cols, n, x_stride);
+}
+
+extern "C" int lng_hip_gemm_q8_0_residual(lng_batch *b, lng_slice codes, lng_slice scales, lng_slice x, int x_dtype,
+                                          const lng_slice *bias, lng_slice h, uint64_t rows, uint64_t cols, uint64_t n,
+                                          uint64_t x_stride, uint64_t h_stride) {
+    if (x_dtype != LNG_F32 && x_dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", x_dtype);
+    Q8Checked q;
+    if (int rc = q8_check(b, codes, scales, x, h, rows, cols, n, x_stride, h_stride, true, false, x_dtype == LNG_BF16, &q)) return rc;
+    if (n >= 32) {
+        return fail(LNG_ERR_DISPATCH, "%llu positions: the product with bias and residual folded in is for fewer than 32 "
+                    "(use gemm_q8_0[_tiled] and add_rows)", (unsigned long long)n);
+    }
+    if (bias) {
+        Operand ob;
+        if (int rc = check_slice(b, "bias", *bias, rows * 4, 4, &ob)) return rc;
+        if (overlaps(q.y, ob)) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+        q.a.bias = (const float *)((const char *)ob.buf->ptr + bias->offset);
+    }
+    q.a.accumulate = 1;
+    q8_record_stream(b, q.a, (rows + 15) / 16, x_dtype == LNG_BF16);
+    return LNG_OK;
+}
+
+namespace {
+int q8_many(lng_batch *b, const lng_q8_matrix *matrices, size_t n_matrices, lng_slice x, const lng_slice *norm_w, float eps,
+            uint64_t cols, uint64_t n, uint64_t x_stride) {
     if (int rc = need_recording(b)) return rc;
     if (!matrices || n_matrices == 0 || n_matrices > 1 + LNG_Q8_MORE) {
         return fail(LNG_ERR_DISPATCH, "%zu matrices: one dispatch takes 1 to %d", n_matrices, 1 + LNG_Q8_MORE);
@@ -1538,6 +1575,18 @@ extern "C" int lng_hip_gemm_q8_0_many(lng_batch *b, const lng_q8_matrix *matrice
             if (i == j) continue;
             if (overlaps(q[i].y, q[j].y)) return fail(LNG_ERR_DISPATCH, "outputs of matrices %zu and %zu overlap", i, j);
             if (overlaps(q[i].y, q[j].codes) || overlaps(q[i].y, q[j].scales)) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+        }
+    }
+    Operand onw{};
+    if (norm_w) {
+        if (n >= 32 || cols > 12288) {
+            return fail(LNG_ERR_DISPATCH, "%llu positions of %llu columns: the product with the RMS norm folded in is for fewer "
+                        "than 32 positions of up to 12288 columns (use rmsnorm_rows and gemm_q8_0[_tiled])",
+                        (unsigned long long)n, (unsigned long long)cols);
+        }
+        if (int rc = check_slice(b, "norm_w", *norm_w, cols * 4, 16, &onw)) return rc;
+        for (size_t i = 0; i < n_matrices; ++i) {
+            if (overlaps(q[i].y, onw)) return fail(LNG_ERR_DISPATCH, "output overlaps an input");
         }
     }
     if (n >= 32) { // the matrix unit is the bound there, not the launches: one product after the other
@@ -1565,9 +1614,14 @@ extern "C" int lng_hip_gemm_q8_0_many(lng_batch *b, const lng_q8_matrix *matrice
         tiles += (q[i].a.rows + 15) / 16;
     }
     if (!fits_u32(tiles) || tiles > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "too large");
+    if (norm_w) {
+        a.norm_w = (const float *)((const char *)onw.buf->ptr + norm_w->offset);
+        a.eps = eps;
+    }
     q8_record_stream(b, a, tiles, false);
     return LNG_OK;
 }
+} // namespace
 
 extern "C" int lng_hip_fill_synthetic(lng_batch *b, lng_slice dst, int dtype, uint64_t seed, float scale,
                                       uint64_t period) {

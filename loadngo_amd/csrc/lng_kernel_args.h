@@ -159,6 +159,12 @@ typedef struct lng_k_q8 {
     /* Few positions only: further matrices of the same dispatch, multiplied by the same x (same cols, n).
      * Workgroups from `first_tile` (in units of 16 rows) on belong to matrix more[i]; first_tile ascends. */
     uint32_t n_more;         /* 0..LNG_Q8_MORE */
+    float eps;               /* of the RMS norm, when norm_w is set */
+    /* Few positions only. norm_w: x is RMS-normalised on the way in, x'[c] = (x[c] / sqrt(mean(x^2) + eps)) * norm_w[c]
+     * (cols <= 12288). bias: y gets bias[row] added. accumulate: the result is added to what y holds (a residual). */
+    const float *norm_w;
+    const float *bias;
+    uint32_t accumulate;
     uint32_t pad_;
     struct lng_k_q8_more {
         const int8_t *codes;

@@ -1140,8 +1140,11 @@ __device__ __forceinline__ uint32_t q8_select_matrix(lng_k_q8 &a) {
 
 template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a, uint32_t tile) {
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
-    __shared__ __attribute__((aligned(16))) float s_x1[ONE ? Q8S_X1 : 4];
+    // ONE: the position's x (normalised there, if asked); otherwise the weights of the RMS norm, if asked
+    __shared__ __attribute__((aligned(16))) float s_x1[(ONE || !XBF16) ? Q8S_X1 : 4];
     __shared__ __attribute__((aligned(4))) uint16_t s_sc[16 * Q8S_SC_BLOCKS];
+    __shared__ float s_norm[Q8S_WAVES]; // ONE: partial sums of squares; otherwise the 16 positions' scales
+    const bool normed = !XBF16 && a.norm_w != nullptr; // uniform
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t j = lane & 15u, kg = lane >> 4;
@@ -1158,6 +1161,18 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
     // The scales of the workgroup's 16 rows are one contiguous run (rows follow each other): copied to
     // LDS a dword per thread, instead of 2-byte loads from 16 different rows per block and wavefront.
     const bool sc_staged = blocks <= Q8S_SC_BLOCKS && r0 + 16u <= a.rows && ((uintptr_t)a.scales & 3u) == 0;
+    if (!ONE && normed) { // wavefront w works out the scale of position p0 + w (there are 16 of each)
+        const uint32_t pw = p0 + wave < a.n ? p0 + wave : a.n - 1u;
+        const float *xp = a.x + (uint64_t)pw * a.x_stride;
+        float ss = 0.0f;
+        for (uint32_t c = 4u * lane; c < a.cols; c += 256u) {
+            const float4 v = *(const float4 *)(xp + c);
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (lane == 0) s_norm[wave] = 1.0f / sqrtf(ss / (float)a.cols + a.eps);
+    }
     bool staged = false;
     for (uint32_t b0 = wave; b0 < blocks || !staged; b0 += Q8S_UNROLL * Q8S_WAVES) {
         uint2 raw[Q8S_UNROLL];
@@ -1182,8 +1197,34 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
         }
         if (!staged) { // every wavefront comes here exactly once, in its first turn
             if (ONE) {
+                float ss = 0.0f;
                 for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
-                    *(float4 *)(&s_x1[i]) = *(const float4 *)(a.x + i);
+                    const float4 v = *(const float4 *)(a.x + i);
+                    *(float4 *)(&s_x1[i]) = v;
+                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                }
+                if (normed) { // every thread normalises the elements it has just written
+#pragma unroll
+                    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+                    if (lane == 0) s_norm[wave] = ss;
+                    __syncthreads();
+                    float total = 0.0f;
+#pragma unroll
+                    for (int w = 0; w < Q8S_WAVES; ++w) total += s_norm[w];
+                    const float scale = 1.0f / sqrtf(total / (float)a.cols + a.eps);
+                    for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                        float4 v = *(const float4 *)(&s_x1[i]);
+                        const float4 nw = *(const float4 *)(a.norm_w + i);
+                        v.x = v.x * scale * nw.x;
+                        v.y = v.y * scale * nw.y;
+                        v.z = v.z * scale * nw.z;
+                        v.w = v.w * scale * nw.w;
+                        *(float4 *)(&s_x1[i]) = v;
+                    }
+                }
+            } else if (normed) {
+                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                    *(float4 *)(&s_x1[i]) = *(const float4 *)(a.norm_w + i);
                 }
             }
             if (sc_staged) { // 16 * blocks * 2 bytes from a 32-byte boundary
@@ -1206,7 +1247,15 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
                 if (XBF16) {
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, xa[u]), wb, zero4, 0, 0, 0);
                 } else {
-                    const float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                    float xs[8] = {xa[u].x, xa[u].y, xa[u].z, xa[u].w, xb[u].x, xb[u].y, xb[u].z, xb[u].w};
+                    if (!ONE && normed) {
+                        const float sp = s_norm[j];
+                        const float4 wa = *(const float4 *)(&s_x1[32u * b + 8u * kg]);
+                        const float4 wb2 = *(const float4 *)(&s_x1[32u * b + 8u * kg + 4u]);
+                        const float nw[8] = {wa.x, wa.y, wa.z, wa.w, wb2.x, wb2.y, wb2.z, wb2.w};
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) xs[e] = xs[e] * sp * nw[e];
+                    }
                     bf16x8 hi, lo;
                     q8_split8(xs, hi, lo);
                     acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hi, wb, zero4, 0, 0, 0);
@@ -1230,7 +1279,12 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
 #pragma unroll
         for (int w = 0; w < Q8S_WAVES - 1; ++w) sum += s_part[w][i][lane];
         const uint32_t p = p0 + 4u * kg + i; // accumulator row = position, column = matrix row
-        if (p < a.n && r0 + j < a.rows) a.y[(uint64_t)p * a.y_stride + r0 + j] = sum;
+        if (p < a.n && r0 + j < a.rows) {
+            float *yp = a.y + (uint64_t)p * a.y_stride + r0 + j;
+            if (a.bias) sum = sum + a.bias[r0 + j];
+            if (a.accumulate) sum = *yp + sum; // the residual: h + ((W x) + bias), each sum rounded as the separate dispatches round it
+            *yp = sum;
+        }
     }
 }
 

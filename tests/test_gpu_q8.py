@@ -283,3 +283,105 @@ def test_several_matrices_in_one_dispatch_give_the_separate_products(gpu, n):
         b.free()
     together, apart = raw[:raw.size // 2], raw[raw.size // 2:]
     assert not np.isnan(together).any() and np.array_equal(together, apart)
+
+
+@pytest.mark.parametrize("n", [1, 5, 16, 31])
+def test_products_of_rms_normalised_positions(gpu, n):
+    """gemm_q8_0_many_normed against the reference's sequence (gpu.rs:712-732): copy the hidden rows, normalise the
+    copy in place, three products. Within 1e-5 of the largest |y| (the sums of squares are added in another
+    order); the hidden rows themselves are not touched; refusals."""
+    cols, eps = 2880, 1e-5
+    shapes = [(4096, 41), (512, 42), (512, 43)]
+    mats = [q8_test_matrix(rows, cols, seed)[:2] for rows, seed in shapes]
+    h = (xorshift_values(51 + n, n * cols) * 3).reshape(n, cols)
+    w = 1 + 0.2 * xorshift_values(52, cols)
+    bufs = [gpu.upload(h), gpu.buffer(h.nbytes), gpu.upload(w)]
+    for codes, bits in mats:
+        bufs += [gpu.upload(codes), gpu.upload(bits)]
+    y_lens = [n * rows * 4 for rows, _ in shapes]
+    bufs += [gpu.buffer(2 * sum(y_lens))]
+    batch = gpu.batch(bufs)
+    hs, xs, ws = C.Slice(0, 0, h.nbytes), C.Slice(1, 0, h.nbytes), C.Slice(2, 0, w.nbytes)
+    batch.copy_rows((hs, cols), (xs, cols), n, cols)
+    batch.rmsnorm_rows((xs, ws), n, (cols, cols), eps)
+    many, offset = [], 0
+    for i, ((rows, _), (codes, bits)) in enumerate(zip(shapes, mats)):
+        m = (C.Slice(3 + 2 * i, 0, codes.nbytes), C.Slice(4 + 2 * i, 0, bits.nbytes))
+        many.append((m, C.Slice(9, offset, y_lens[i]), rows))
+        batch.gemm_q8_0(m, xs, C.Slice(9, sum(y_lens) + offset, y_lens[i]), rows, cols, n, (cols, rows))
+        offset += y_lens[i]
+    before = batch.dispatches()
+    batch.gemm_q8_0_many_normed(many, hs, (ws, eps), cols, n, cols)
+    assert batch.dispatches() == before + 1
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many_normed(many, hs, (C.Slice(2, 4, w.nbytes - 4), eps), cols, n, cols)    # weights too short
+    with pytest.raises(C.Dispatch):
+        batch.gemm_q8_0_many_normed([(many[0][0], C.Slice(2, 0, w.nbytes), 1)], hs, (ws, eps), cols, n, cols)
+    assert batch.dispatches() == before + 1
+    batch.run()
+    raw = bufs[-1].read(np.float32)
+    assert np.array_equal(bufs[0].read(np.float32).reshape(n, cols), h)
+    batch.drop()
+    for b in bufs:
+        b.free()
+    together, apart = raw[:raw.size // 2], raw[raw.size // 2:]
+    assert not np.isnan(together).any()
+    assert np.abs(together - apart).max() <= 1e-5 * np.abs(apart).max()
+
+
+def test_the_normalised_product_is_for_decoding(gpu):
+    cols = 64
+    codes, bits, _ = q8_test_matrix(64, cols, 3)
+    bufs = [gpu.buffer(32 * cols * 4), gpu.upload(np.ones(cols, np.float32)), gpu.upload(codes), gpu.upload(bits),
+            gpu.buffer(32 * 64 * 4)]
+    batch = gpu.batch(bufs)
+    m = [((C.Slice(2, 0, codes.nbytes), C.Slice(3, 0, bits.nbytes)), C.Slice(4, 0, 32 * 64 * 4), 64)]
+    with pytest.raises(C.Dispatch, match="fewer than 32"):
+        batch.gemm_q8_0_many_normed(m, C.Slice(0, 0, 32 * cols * 4), (C.Slice(1, 0, cols * 4), 1e-5), cols, 32, cols)
+    with pytest.raises(C.Dispatch, match="fewer than 32"):
+        batch.gemm_q8_0_residual(m[0][0], C.Slice(0, 0, 32 * cols * 4), None, C.Slice(4, 0, 32 * 64 * 4), 64, cols, 32, (cols, 64))
+    assert batch.dispatches() == 0
+    batch.drop()
+    for b in bufs:
+        b.free()
+
+
+@pytest.mark.parametrize("n,bf16", [(1, False), (7, False), (31, False), (1, True), (16, True)])
+def test_output_projection_with_bias_and_residual_folded_in(gpu, n, bf16):
+    """gemm_q8_0_residual against the reference's three dispatches (gpu.rs:807-827: the product, add_rows of the
+    bias, add_rows into the hidden state): the same bits, for f32 and bf16 positions, hidden rows wider than the
+    product, with and without a bias."""
+    from tests.helpers import to_bf16_bits
+    rows, cols, h_stride = 2880, 4096, 2912
+    codes, bits, _ = q8_test_matrix(rows, cols, 61)
+    x = xorshift_values(62 + n, n * cols).reshape(n, cols)
+    xin = to_bf16_bits(x) if bf16 else x
+    h = xorshift_values(63, n * h_stride).reshape(n, h_stride)
+    bias = xorshift_values(64, rows)
+    for with_bias in (True, False):
+        bufs = [gpu.upload(codes), gpu.upload(bits), gpu.upload(xin), gpu.upload(h), gpu.upload(h), gpu.upload(bias),
+                gpu.buffer(n * rows * 4)]
+        batch = gpu.batch(bufs)
+        m = (C.Slice(0, 0, codes.nbytes), C.Slice(1, 0, bits.nbytes))
+        xs = C.Slice(2, 0, xin.nbytes)
+        h_len = ((n - 1) * h_stride + rows) * 4
+        if bf16:
+            batch.gemm_q8_0_bf16(m, xs, C.Slice(6, 0, n * rows * 4), rows, cols, n, (cols, rows))
+        else:
+            batch.gemm_q8_0(m, xs, C.Slice(6, 0, n * rows * 4), rows, cols, n, (cols, rows))
+        if with_bias:
+            batch.add_rows(C.Slice(6, 0, n * rows * 4), (C.Slice(5, 0, rows * 4), 0), n, rows)
+        for p in range(n):  # add_rows writes dense rows: one call per row of the wider hidden state
+            batch.add_rows(C.Slice(3, p * h_stride * 4, rows * 4), (C.Slice(6, p * rows * 4, rows * 4), rows), 1, rows)
+        before = batch.dispatches()
+        batch.gemm_q8_0_residual(m, xs, C.Slice(5, 0, rows * 4) if with_bias else None, C.Slice(4, 0, h_len), rows, cols, n,
+                                 (cols, h_stride), C.BF16 if bf16 else C.F32)
+        assert batch.dispatches() == before + 1
+        batch.run()
+        apart, together = bufs[3].read(np.float32), bufs[4].read(np.float32)
+        batch.drop()
+        for b in bufs:
+            b.free()
+        assert not np.isnan(together).any() and np.array_equal(together, apart)
+        assert not np.array_equal(together.reshape(n, h_stride)[:, :rows], h[:, :rows])
+        assert np.array_equal(together.reshape(n, h_stride)[:, rows:], h[:, rows:])

@@ -208,9 +208,17 @@ class DeviceBlocks:
             else:
                 batch.gemm_q8_0(mat, xs, ys, rows, cols, n_run, (cols, rows))
 
-        batch.copy_rows((rows_of(H, hidden), hidden), (rows_of(X, hidden), hidden), n, hidden)
-        batch.rmsnorm_rows((rows_of(X, hidden), batch.attach(r["attn_norm"])), n, (hidden, hidden), m.eps)
-        if self.qkv_together:  # the three projections as one call (one dispatch below 32 positions)
+        fused = self.qkv_together == "fused"  # norm folded into the projections, bias and residual into the output projection
+        if not fused:
+            batch.copy_rows((rows_of(H, hidden), hidden), (rows_of(X, hidden), hidden), n, hidden)
+            batch.rmsnorm_rows((rows_of(X, hidden), batch.attach(r["attn_norm"])), n, (hidden, hidden), m.eps)
+        if fused:
+            mats = []
+            for part, y in (("q", Q), ("k", K), ("v", V)):
+                codes, scales, rows, cols = r[part]
+                mats.append(((batch.attach(codes), batch.attach(scales)), rows_of(y, rows), rows))
+            batch.gemm_q8_0_many_normed(mats, rows_of(H, hidden), (batch.attach(r["attn_norm"]), m.eps), hidden, n, hidden)
+        elif self.qkv_together:  # the three projections as one call (one dispatch below 32 positions)
             mats = []
             for part, y in (("q", Q), ("k", K), ("v", V)):
                 codes, scales, rows, cols = r[part]
@@ -236,9 +244,14 @@ class DeviceBlocks:
             rows = min(slots, end)
             batch.attention_grouped_with_sinks((rows_of(QR, qw), rows_of(KC, kw, rows), rows_of(VC, kw, rows)), sinks,
                                                rows_of(ATT, qw), shape, C.F32)
-        mul("output", ATT, TMP)
-        batch.add_rows(rows_of(TMP, hidden), (batch.attach(r["o_bias"]), 0), n, hidden)
-        batch.add_rows(rows_of(H, hidden), (rows_of(TMP, hidden), hidden), n, hidden)
+        if fused:
+            codes, scales, rows, cols = r["output"]
+            batch.gemm_q8_0_residual((batch.attach(codes), batch.attach(scales)), rows_of(ATT, cols), batch.attach(r["o_bias"]),
+                                     rows_of(H, hidden), rows, cols, n, (cols, hidden))
+        else:
+            mul("output", ATT, TMP)
+            batch.add_rows(rows_of(TMP, hidden), (batch.attach(r["o_bias"]), 0), n, hidden)
+            batch.add_rows(rows_of(H, hidden), (rows_of(TMP, hidden), hidden), n, hidden)
         done = batch.run()
         assert not isinstance(done.gpu_time, Exception), done.gpu_time
         batch.drop()
@@ -255,7 +268,8 @@ class DeviceBlocks:
 
 
 @pytest.mark.parametrize("chunk,tiled,qkv_together", [(1, False, False), (9, False, False), (40, False, False), (40, True, False),
-                                                      (1, False, True), (9, False, True), (40, True, True)])
+                                                      (1, False, True), (9, False, True), (40, True, True),
+                                                      (1, False, "fused"), (9, False, "fused")])
 def test_whole_attention_blocks_on_the_device_match_transformers(gpu, model, chunk, tiled, qkv_together):
     ids, want = tm.load_fixture(FIXTURE)
     s = DeviceBlocks(gpu, model, chunk, tiled, qkv_together)
