@@ -202,6 +202,56 @@ void q8_product_of_bf16_positions_is_the_f32_product(const Gpu &gpu) {
     std::printf("done q8_product_of_bf16_positions_is_the_f32_product\n");
 }
 
+void decoding_products_fold_their_neighbours_in(const Gpu &gpu) {
+    const size_t rows = 96, cols = 2880, n = 3;
+    std::vector<uint8_t> codes;
+    for (float x : values(71, rows * cols)) codes.push_back((uint8_t)(int8_t)(x * 127.9f));
+    std::vector<uint8_t> scales;
+    for (size_t i = 0; i < rows * cols / 32; ++i) {
+        scales.push_back(0x00);
+        scales.push_back((uint8_t)(0x20 + 4 * (i % 5))); // binary16 2^-7, 2^-6, ...
+    }
+    const std::vector<float> h = values(72, n * cols), w = values(73, cols), bias = values(74, rows), hidden = values(75, n * rows);
+    std::vector<Buffer> buffers;
+    buffers.push_back(upload_bytes(gpu, codes));   // 0
+    buffers.push_back(upload_bytes(gpu, scales));  // 1
+    buffers.push_back(upload(gpu, h));             // 2: positions
+    buffers.push_back(upload(gpu, h));             // 3: their copy, normalised in place
+    buffers.push_back(upload(gpu, w));             // 4
+    buffers.push_back(gpu.buffer(n * rows * 4));   // 5: product of the normalised copy
+    buffers.push_back(gpu.buffer(n * rows * 4));   // 6: the same in one dispatch
+    buffers.push_back(upload(gpu, bias));          // 7
+    buffers.push_back(upload(gpu, hidden));        // 8: hidden rows, three dispatches
+    buffers.push_back(upload(gpu, hidden));        // 9: hidden rows, one dispatch
+    Batch batch = gpu.batch(std::move(buffers));
+    const std::pair<Slice, Slice> matrix{Slice(0, 0, codes.size()), Slice(1, 0, scales.size())};
+    batch.rmsnorm_rows({f32s(3, n * cols), f32s(4, cols)}, n, {cols, cols}, 1e-5f);
+    batch.gemm_q8_0(matrix, f32s(3, n * cols), f32s(5, n * rows), {rows, cols}, n, {cols, rows});
+    batch.gemm_q8_0_many_normed({{matrix, f32s(6, n * rows), rows}}, f32s(2, n * cols), {f32s(4, cols), 1e-5f}, cols, n, cols);
+    // the output-projection pattern on the product in buffer 5: bias, then into the hidden rows
+    batch.add_rows(f32s(5, n * rows), {f32s(7, rows), 0}, n, rows);
+    batch.add_rows(f32s(8, n * rows), {f32s(5, n * rows), rows}, n, rows);
+    const Slice bias_slice = f32s(7, rows);
+    batch.gemm_q8_0_residual(matrix, f32s(3, n * cols), &bias_slice, f32s(9, n * rows), {rows, cols}, n, {cols, rows});
+    Completed done = std::move(batch).run();
+    done.gpu_time();
+    const std::vector<float> apart = done.buffers[5].to_f32(), together = done.buffers[6].to_f32();
+    // buffer 5 holds product + bias by now: take the bias off on the host for the comparison of the products
+    double worst = 0.0, largest = 0.0;
+    for (size_t p = 0; p < n; ++p) {
+        for (size_t r = 0; r < rows; ++r) {
+            const double product = (double)apart[p * rows + r] - (double)bias[r];
+            largest = std::max(largest, std::fabs(product));
+            worst = std::max(worst, std::fabs(product - (double)together[p * rows + r]));
+        }
+    }
+    expect(worst <= 2e-5 * largest, "the normalised product in one dispatch: relative " + std::to_string(worst / largest));
+    const std::vector<float> three = done.buffers[8].to_f32(), one = done.buffers[9].to_f32();
+    expect(std::memcmp(three.data(), one.data(), three.size() * 4) == 0, "bias and residual folded in give the bits of the three dispatches");
+    expect(done.buffers[2].to_f32() == h, "the positions of the normalised product are left alone");
+    std::printf("done decoding_products_fold_their_neighbours_in\n");
+}
+
 } // namespace
 
 int main() {
@@ -210,6 +260,7 @@ int main() {
         batched_decode_is_one_plain_call_per_sequence(gpu);
         prepare_attention_is_the_reference_sequence_of_dispatches(gpu);
         q8_product_of_bf16_positions_is_the_f32_product(gpu);
+        decoding_products_fold_their_neighbours_in(gpu);
     } catch (const lng::Error &e) {
         std::printf("FAILED with %s\n", e.what());
         return 100;
