@@ -650,6 +650,78 @@ def run_copy(gpu, steps, warmup, nbytes=1 << 30):
             "gpu_ms": g * 1e3, "gbs": 2 * nbytes / g / 1e9}
 
 
+def run_block(gpu, steps, warmup, ctx=4096, layers=24):
+    """One decoding token through the attention block of gpt-oss/src/gpu.rs:703-827 at gpt-oss-20b's sizes (hidden
+    2880, 64 q / 8 kv heads of 64, Q8_0 projections), `layers` times in one batch over a bf16 cache of `ctx` tokens:
+    as the reference records it (with prepare_attention for its seven pre-attention dispatches), with the q, k and v
+    projections as one call, and with the RMS norm, the bias and the residual folded into the products as well.
+    Launch-bound: microseconds per layer."""
+    hidden, qw, kw = 2880, H * D, G * D
+    rng = np.random.default_rng(21)
+
+    def q8(rows, cols):
+        return (gpu.resident(rng.integers(-127, 128, rows * cols, dtype=np.int8)),
+                gpu.resident((rng.random(rows * cols // 32, dtype=np.float32) * 0.01 + 0.001).astype(np.float16).view(np.uint16)))
+
+    wq, wk, wv, wo = q8(qw, hidden), q8(kw, hidden), q8(kw, hidden), q8(hidden, qw)
+    consts = {name: gpu.resident(arr) for name, arr in (
+        ("norm", np.ones(hidden, np.float32)), ("qb", np.zeros(qw, np.float32)), ("kb", np.zeros(kw, np.float32)),
+        ("vb", np.zeros(kw, np.float32)), ("ob", np.zeros(hidden, np.float32)), ("sinks", np.zeros(H, np.float32)))}
+    f32 = lambda n: gpu.buffer(n * 4)  # noqa: E731
+    bufs = [f32(hidden), f32(hidden), f32(qw), f32(kw), f32(kw), f32(D), gpu.buffer(qw * 2), gpu.buffer(ctx * kw * 2),
+            gpu.buffer(ctx * kw * 2), gpu.buffer(qw * 2), f32(hidden)]
+    iH, iX, iQ, iK, iV, iT, iQR, iKC, iVC, iATT, iTMP = range(11)
+    for i in (iH, iT):
+        bufs[i].write(np.full(bufs[i].len // 4, 0.1, np.float32))
+    for i in (iKC, iVC):
+        fill(gpu, bufs[i], 50 + i)
+    start = ctx - 1
+    S = lambda b, n, es=4: C.Slice(b, 0, n * es)  # noqa: E731
+
+    def go(mode):
+        batch = gpu.batch(bufs)
+        at = batch.attach
+        mats = [((at(w[0]), at(w[1])), S(y, rows), rows) for w, y, rows in ((wq, iQ, qw), (wk, iK, kw), (wv, iV, kw))]
+        for _ in range(layers):
+            if mode == "folded":
+                batch.gemm_q8_0_many_normed(mats, S(iH, hidden), (at(consts["norm"]), 1e-5), hidden, 1, hidden)
+            else:
+                batch.copy_rows((S(iH, hidden), hidden), (S(iX, hidden), hidden), 1, hidden)
+                batch.rmsnorm_rows((S(iX, hidden), at(consts["norm"])), 1, (hidden, hidden), 1e-5)
+                if mode == "one_qkv_call":
+                    batch.gemm_q8_0_many(mats, S(iX, hidden), hidden, 1, hidden)
+                else:
+                    for m, y, rows in mats:
+                        batch.gemv_q8_0(m, S(iX, hidden), y, rows, hidden)
+            batch.prepare_attention(dict(q=iQ, k=iK, v=iV, table=iT, q_out=iQR, k_cache=iKC, v_cache=iVC),
+                                    [C.PrepareItem(n=1, start=start, slots=ctx)], H, G, D, D, C.BF16, at(consts["qb"]),
+                                    at(consts["kb"]), at(consts["vb"]))
+            batch.attention_grouped_with_sinks((S(iQR, qw, 2), S(iKC, ctx * kw, 2), S(iVC, ctx * kw, 2)), at(consts["sinks"]),
+                                               S(iATT, qw, 2), C.GroupedShape(1, start, H, G, D, C.FULL, ctx, SCALE), C.BF16)
+            mo = (at(wo[0]), at(wo[1]))
+            if mode == "folded":
+                batch.gemm_q8_0_residual(mo, S(iATT, qw, 2), at(consts["ob"]), S(iH, hidden), hidden, qw, 1, (qw, hidden), C.BF16)
+            else:
+                batch.gemm_q8_0_bf16(mo, S(iATT, qw, 2), S(iTMP, hidden), hidden, qw, 1, (qw, hidden))
+                batch.add_rows(S(iTMP, hidden), (at(consts["ob"]), 0), 1, hidden)
+                batch.add_rows(S(iH, hidden), (S(iTMP, hidden), hidden), 1, hidden)
+        n = batch.dispatches()
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time, n
+
+    out = {"workload": "one decoding token through %d attention blocks (gpt-oss-20b sizes), bf16 cache of %d tokens" % (layers, ctx)}
+    for mode in ("as_the_reference_records_it", "one_qkv_call", "folded"):
+        for _ in range(warmup):
+            go(mode)
+        runs = sorted(go(mode) for _ in range(max(steps, 7)))
+        t, n = runs[len(runs) // 2]
+        out[mode] = {"dispatches_per_layer": n // layers, "gpu_us_per_layer": t * 1e6 / layers}
+    for b in bufs:
+        b.free()
+    return out
+
+
 def run_prepare(gpu, steps, warmup):
     """The step before attention (biases, rotation by halves, bf16 narrowing, ring append) at gpt-oss
     shapes: a prompt pass of 8192 rows into a flat cache, and one decoding step of 16 sequences (one
@@ -735,7 +807,7 @@ def main():
     ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
                     "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -746,7 +818,7 @@ def main():
     log("device:", gpu.name())
     extra = {}
     if args.only:
-        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare,
+        runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare, "block": run_block,
                 "c4act": run_prefill_activity, "q8": run_q8}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
@@ -763,6 +835,8 @@ def main():
         log("prep", extra["pre_attention_step"])
         extra["q8_0_projection"] = run_q8(gpu, args.steps, args.warmup)
         log("q8", extra["q8_0_projection"])
+        extra["decode_block_one_token"] = run_block(gpu, args.steps, args.warmup)
+        log("block", extra["decode_block_one_token"])
         extra["c1_fp32"] = run_config1(gpu, args.steps, args.warmup)
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)
     log("c5", r)
