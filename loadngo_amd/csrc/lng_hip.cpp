@@ -91,7 +91,7 @@ struct lng_gpu {
     hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
-    hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
+    hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_one_w8 = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
                   q8_tiled_bf16 = nullptr;
     std::string name;
     unsigned cus = 256;
@@ -688,6 +688,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_q8_split_x", &g->q8_split_x, true},
         {"lng_q8_stream", &g->q8_stream, true},
         {"lng_q8_stream_one", &g->q8_stream_one, true},
+        {"lng_q8_stream_one_w8", &g->q8_stream_one_w8, true},
         {"lng_q8_tiled", &g->q8_tiled, true},
         {"lng_q8_tiled_bf16", &g->q8_tiled_bf16, true},
         {"lng_q8_stream_bf16", &g->q8_stream_bf16, true},
@@ -1423,12 +1424,14 @@ int q8_check(lng_batch *b, const lng_slice &codes, const lng_slice &scales, cons
 // `a` may name further matrices of the same dispatch (a.more); row_tiles counts the tiles of all of them.
 void q8_record_stream(lng_batch *b, const lng_k_q8 &a, uint64_t row_tiles, bool x_bf16) {
     const bool one = a.n == 1 && a.cols <= 12288 && !x_bf16; // x of a single position is held in LDS (Q8S_X1 floats)
+    // more row tiles than compute units (several matrices): 8-wavefront workgroups, two per unit, one round
+    const bool w8 = one && row_tiles > b->gpu->cus && !getenv("LNG_Q8_W16");
     Cmd c;
-    c.fn = x_bf16 ? b->gpu->q8_stream_bf16 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
-    c.name = x_bf16 ? "lng_q8_stream_bf16" : one ? "lng_q8_stream_one" : "lng_q8_stream";
+    c.fn = x_bf16 ? b->gpu->q8_stream_bf16 : w8 ? b->gpu->q8_stream_one_w8 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
+    c.name = x_bf16 ? "lng_q8_stream_bf16" : w8 ? "lng_q8_stream_one_w8" : one ? "lng_q8_stream_one" : "lng_q8_stream";
     c.grid[0] = (unsigned)row_tiles;
     c.grid[1] = (unsigned)((a.n + 15) / 16);
-    c.block = 1024;
+    c.block = w8 ? 512 : 1024;
     set_args(c, a);
     b->cmds.push_back(std::move(c));
     b->dispatches += 1;

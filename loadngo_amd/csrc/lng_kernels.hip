@@ -1138,12 +1138,16 @@ __device__ __forceinline__ uint32_t q8_select_matrix(lng_k_q8 &a) {
     return tile;
 }
 
-template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a, uint32_t tile) {
+// WAVES wavefronts share the blocks of a row tile (16; 8 for the one-position form when two workgroups per compute
+// unit cover the row tiles in one round instead of two).
+template <bool ONE, bool XBF16 = false, int WAVES = Q8S_WAVES>
+__device__ __forceinline__ void q8_stream_body(const lng_k_q8 &a, uint32_t tile) {
+    static_assert(ONE || WAVES == 16, "the several-position forms map wavefront w to position w of 16");
     __shared__ float s_part[Q8S_WAVES - 1][4][64];
     // ONE: the position's x (normalised there, if asked); otherwise the weights of the RMS norm, if asked
     __shared__ __attribute__((aligned(16))) float s_x1[(ONE || !XBF16) ? Q8S_X1 : 4];
     __shared__ __attribute__((aligned(4))) uint16_t s_sc[16 * Q8S_SC_BLOCKS];
-    __shared__ float s_norm[Q8S_WAVES]; // ONE: partial sums of squares; otherwise the 16 positions' scales
+    __shared__ float s_norm[16]; // ONE: partial sums of squares; otherwise the 16 positions' scales
     const bool normed = !XBF16 && a.norm_w != nullptr; // uniform
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1174,7 +1178,10 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
         if (lane == 0) s_norm[wave] = 1.0f / sqrtf(ss / (float)a.cols + a.eps);
     }
     bool staged = false;
-    for (uint32_t b0 = wave; b0 < blocks || !staged; b0 += Q8S_UNROLL * Q8S_WAVES) {
+    floatx4 y0 = zero4; // stream 0's sum (wavefront 0)
+    for (uint32_t stream = wave; stream < Q8S_WAVES; stream += WAVES) {
+    y = zero4;
+    for (uint32_t b0 = stream; b0 < blocks || !staged; b0 += Q8S_UNROLL * Q8S_WAVES) {
         uint2 raw[Q8S_UNROLL];
         uint16_t scale[Q8S_UNROLL];
         float4 xa[Q8S_UNROLL], xb[Q8S_UNROLL];
@@ -1198,7 +1205,7 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
         if (!staged) { // every wavefront comes here exactly once, in its first turn
             if (ONE) {
                 float ss = 0.0f;
-                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * WAVES) {
                     const float4 v = *(const float4 *)(a.x + i);
                     *(float4 *)(&s_x1[i]) = v;
                     ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
@@ -1210,9 +1217,9 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
                     __syncthreads();
                     float total = 0.0f;
 #pragma unroll
-                    for (int w = 0; w < Q8S_WAVES; ++w) total += s_norm[w];
+                    for (int w = 0; w < WAVES; ++w) total += s_norm[w];
                     const float scale = 1.0f / sqrtf(total / (float)a.cols + a.eps);
-                    for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                    for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * WAVES) {
                         float4 v = *(const float4 *)(&s_x1[i]);
                         const float4 nw = *(const float4 *)(a.norm_w + i);
                         v.x = v.x * scale * nw.x;
@@ -1223,13 +1230,13 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
                     }
                 }
             } else if (normed) {
-                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * Q8S_WAVES) {
+                for (uint32_t i = 4u * threadIdx.x; i < a.cols; i += 4u * 64u * WAVES) {
                     *(float4 *)(&s_x1[i]) = *(const float4 *)(a.norm_w + i);
                 }
             }
             if (sc_staged) { // 16 * blocks * 2 bytes from a 32-byte boundary
                 const uint32_t *src = (const uint32_t *)(a.scales + (uint64_t)r0 * blocks);
-                for (uint32_t i = threadIdx.x; i < 8u * blocks; i += 64u * Q8S_WAVES) ((uint32_t *)s_sc)[i] = src[i];
+                for (uint32_t i = threadIdx.x; i < 8u * blocks; i += 64u * WAVES) ((uint32_t *)s_sc)[i] = src[i];
             }
             __syncthreads();
             staged = true;
@@ -1267,15 +1274,18 @@ template <bool ONE, bool XBF16 = false> __device__ __forceinline__ void q8_strea
             }
         }
     }
-    if (wave != 0) {
+    if (stream != 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) s_part[wave - 1][i][lane] = y[i];
+        for (int i = 0; i < 4; ++i) s_part[stream - 1][i][lane] = y[i];
+    } else {
+        y0 = y;
+    }
     }
     __syncthreads();
     if (wave != 0) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        float sum = y[i];
+        float sum = y0[i];
 #pragma unroll
         for (int w = 0; w < Q8S_WAVES - 1; ++w) sum += s_part[w][i][lane];
         const uint32_t p = p0 + 4u * kg + i; // accumulator row = position, column = matrix row
@@ -1296,6 +1306,12 @@ extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream(lng_k
 extern "C" __global__ __launch_bounds__(64 * Q8S_WAVES) void lng_q8_stream_one(lng_k_q8 a) {
     const uint32_t tile = q8_select_matrix(a);
     q8_stream_body<true>(a, tile);
+}
+
+// the same with 8 wavefronts: half the LDS partials and threads, two workgroups per compute unit
+extern "C" __global__ __launch_bounds__(512) void lng_q8_stream_one_w8(lng_k_q8 a) {
+    const uint32_t tile = q8_select_matrix(a);
+    q8_stream_body<true, false, 8>(a, tile);
 }
 
 // positions already in bf16 (the output of a bf16 attention): one matrix instruction per block
