@@ -532,6 +532,8 @@ def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_hea
     (40, 97, 7, 64, 4, 1, None), (256, 0, 100, 256, 32, 8, None), (128, 3968, FULL, 4096, 64, 8, None),
     (96, 1952, FULL, 2048, 64, 8, "7"), (64, 960, FULL, 1024, 24, 8, "64"), (96, 0, FULL, 96, 64, 8, "5"),
     (160, 2000, 1500, 2176, 16, 2, "3"),
+    # a thousand workgroups and more: the build of the kernel with two workgroups per compute unit
+    (4096, 0, 128, 4096, 8, 8, None), (4096, 0, FULL, 4096, 8, 8, None), (2080, 3000, 300, 2400, 32, 8, None),
 ])
 def test_prefill_f32_matches_the_cpu_reference(gpu, t, start, window, slots, heads, kv_heads, forced, monkeypatch):
     """The tiled operator on f32 operands at head width 64 (the reference's own prompt pass, gpu.rs:760-806):
