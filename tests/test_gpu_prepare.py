@@ -248,9 +248,10 @@ def test_strided_rmsnorm_and_row_copy_touch_only_their_columns(gpu):
     assert (np.abs(got - orc.rms_norm_rows(vv, w, d, 1e-5)) <= 2e-6 * (1 + np.abs(want))).all()
 
 
-def test_rmsnorm_at_the_model_width(gpu):
+@pytest.mark.parametrize("rows,d", [(37, 2880), (1, 2880), (5, 256), (5, 257), (3, 4096), (3, 4100), (2, 12288)])
+def test_rmsnorm_at_the_model_width(gpu, rows, d):
+    """Rows of 257..4096 floats take a workgroup each, other widths a wavefront: both sides of both limits."""
     rng = np.random.default_rng(8)
-    rows, d = 37, 2880
     v = (rng.standard_normal((rows, d)) * 4).astype(np.float32)
     w = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
     (got,) = _run(gpu, [v, w], lambda b: b.rmsnorm_rows((C.Slice(0, 0, v.nbytes), C.Slice(1, 0, w.nbytes)), rows,
