@@ -314,6 +314,8 @@ def test_prefill_bf16_matches_the_cpu_reference(gpu, t, start, window, slots, he
     (512, 3584, FULL, 4096, None), (64, 4000, FULL, 4096, None), (33, 5000, 2048, 5056, None), (100, 8000, FULL, 8128, None),
     (512, 1536, FULL, 2048, "7"), (64, 960, FULL, 1024, "64"), (96, 0, FULL, 96, "5"), (160, 2000, 1500, 2176, "3"),
     (64, 4000, 3000, 3072, None), (96, 6000, 4000, 4096, "6"),
+    # up to 32 rows: the 32-row form of the kernel, with splits
+    (32, 4064, FULL, 4096, None), (20, 5000, FULL, 5024, None), (7, 9000, 4000, 4032, "9"),
 ])
 def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots, forced, monkeypatch):
     """A chunk of a long prompt (the reference passes 512 rows at a time, engine.rs:51), or a few rows late
