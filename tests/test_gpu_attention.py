@@ -473,12 +473,15 @@ def test_config5_layer_at_full_size_periodic_identity(gpu):
         assert max_error(got[batch_size + b], from_bf16_bits(win[0])) < BF16_TOL, ("window", b)
 
 
-@pytest.mark.parametrize("start,window,slots", [(131148, FULL, 131149), (200000, 100000, 150016), (70000, FULL, 70001)])
-def test_decode_bf16_one_long_row(gpu, start, window, slots):
-    """A single query over a very long cache: the run is cut into the largest allowed number of
-    chunks (the chunk length grows to respect it) and merged by a second dispatch; with a ring that
-    has wrapped and a window that does not start on a tile boundary."""
-    heads, kv_heads, dim = 64, 8, 64
+@pytest.mark.parametrize("start,window,slots,heads,kv_heads", [
+    (131148, FULL, 131149, 64, 8), (200000, 100000, 150016, 64, 8), (70000, FULL, 70001, 64, 8),
+    # one kv head: the planner lets the row have more chunks (137 and 256) so that the compute units have work
+    (70000, FULL, 70001, 4, 1), (300000, FULL, 300001, 16, 1), (6000, FULL, 6001, 8, 1)])
+def test_decode_bf16_one_long_row(gpu, start, window, slots, heads, kv_heads):
+    """A single query over a very long cache: the run is cut into chunks (at most 32 unless fewer would leave
+    compute units idle, never more than 256: the chunk length grows to respect that) and merged in the kernel
+    or by a second dispatch; with a ring that has wrapped and a window that does not start on a tile boundary."""
+    dim = 64
     rows = min(slots, start + 1)
     rng = np.random.default_rng(start)
     q = to_bf16_bits(rng.standard_normal((1, heads, dim), dtype=np.float32) * 0.5)
@@ -496,6 +499,7 @@ def test_decode_bf16_one_long_row(gpu, start, window, slots):
 @pytest.mark.parametrize("t,start,window,slots,heads,kv_heads", [
     (1, 0, FULL, 1, 64, 8), (1, 36, FULL, 37, 64, 8), (1, 4095, FULL, 4096, 64, 8), (1, 5000, 128, 200, 64, 8),
     (1, 70000, FULL, 70001, 64, 8), (1, 200000, 100000, 150016, 16, 2), (3, 2000, FULL, 2003, 8, 8), (7, 900, 33, 41, 6, 2),
+    (1, 70000, FULL, 70001, 4, 1), (1, 300000, FULL, 300001, 16, 1),
     (31, 100, FULL, 131, 5, 1), (2, 9000, 1, 3, 64, 8), (5, 260, 300, 305, 24, 8), (1, 5000, FULL, 5001, 32, 2),
     (3, 700, 100, 128, 12, 1), (2, 40, 17, 19, 16, 1), (1, 31, FULL, 32, 64, 8), (1, 0, FULL, 1, 64, 8),
 ])
