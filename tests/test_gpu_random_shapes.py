@@ -14,13 +14,18 @@ from tests.helpers import FULL, from_bf16_bits, ring_layout, to_bf16_bits
 pytestmark = pytest.mark.gpu
 
 
+def _pick(rng, values):
+    """One of `values` as the Python object it is (numpy would turn a list holding 2**64 - 1 into floats)."""
+    return values[int(rng.integers(len(values)))]
+
+
 def _random_shape(rng, tiled):
     kv_heads = int(rng.choice([1, 2, 3, 8]))
     group = int(rng.choice([1, 2, 4, 5, 8, 16]))
     dim = int(rng.choice([32, 64, 64, 64, 96, 128, 256]))
     t = int(rng.choice([1, 1, 2, 7, 31, 32, 33, 64, 65, 100]))
     start = int(rng.choice([0, 0, 1, 5, 31, 32, 63, 200, 777]))
-    window = int(rng.choice([FULL, FULL, 1, 2, 7, 31, 32, 33, 128, 500]))
+    window = _pick(rng, [FULL, FULL, FULL, 1, 2, 7, 31, 32, 33, 128, 500, 0])   # a window of 0 is refused
     end = start + t
     kind = rng.integers(0, 3)
     if kind == 0:
@@ -71,7 +76,7 @@ def test_random_shapes_agree_with_the_oracle_or_are_refused(gpu, tiled, dtype):
                                                tiled, dtype))
             assert max_error(got, want) <= 2e-2, f"{what}: {max_error(got, want)}"
         ran += 1
-    assert ran >= 15 and refused >= 1, (ran, refused)
+    assert ran >= 25 and refused >= 1, (ran, refused)
 
 
 def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
@@ -85,7 +90,7 @@ def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
         heads = kv_heads * int(rng.choice([1, 2, 3, 5, 8]))
         t = int(rng.choice([32, 33, 64, 65, 96, 128, 200, 511, 512, 600]))
         start = int(rng.choice([0, 31, 500, 1000, 2047, 3000, 4097, 6000]))
-        window = int(rng.choice([FULL, FULL, FULL, 1025, 1500, 3000]))
+        window = _pick(rng, [FULL, FULL, FULL, 1025, 1500, 3000])
         end = start + t
         if rng.integers(0, 2):
             slots = end + int(rng.integers(0, 70))
@@ -109,4 +114,4 @@ def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
         what = f"t={t} start={start} H={heads} G={kv_heads} window={window} slots={slots} splits={forced}"
         assert not np.isnan(got).any() and max_error(got, want) <= 2e-2, f"{what}: {max_error(got, want)}"
         ran += 1
-    assert ran >= 15, ran
+    assert ran >= 25, ran
