@@ -167,6 +167,13 @@ def _check(rc):
         raise _ERRORS.get(rc, Error)(message)
 
 
+def _u64(name, value):
+    """ctypes wraps integers modulo 2**64 without a word (2**64 becomes 0): counts are checked here instead."""
+    if not isinstance(value, (int, np.integer)) or isinstance(value, bool) or not 0 <= int(value) < 2**64:
+        raise ValueError("%s = %r is not an integer in 0 .. 2**64 - 1" % (name, value))
+    return int(value)
+
+
 class Slice:
     """apple.rs:507-521: bytes ``offset..offset+len`` of the batch's buffer number ``buffer``."""
 
@@ -176,7 +183,7 @@ class Slice:
         self.buffer, self.offset, self.len = buffer, offset, len
 
     def _c(self):
-        return _Slice(self.buffer, self.offset, self.len)
+        return _Slice(*[_u64(n, getattr(self, n)) for n in self.__slots__])
 
     def __repr__(self):
         return "Slice(buffer=%d, offset=%d, len=%d)" % (self.buffer, self.offset, self.len)
@@ -195,7 +202,7 @@ class GroupedShape:
         self.dim, self.window, self.slots, self.scale = dim, window, slots, scale
 
     def _c(self):
-        return _Shape(self.t, self.start, self.heads, self.kv_heads, self.dim, self.window, self.slots, self.scale)
+        return _Shape(*[_u64(n, getattr(self, n)) for n in self.__slots__[:7]], self.scale)
 
     def __repr__(self):
         return "GroupedShape(%s)" % ", ".join("%s=%r" % (n, getattr(self, n)) for n in self.__slots__)
@@ -221,8 +228,7 @@ def decode_items(items):
     """A prepared table of ``DecodeItem`` for ``Batch.attention_decode_batched`` (built once,
     reused every step)."""
     return (_Item * len(items))(*[
-        _Item(i.q_offset, i.out_offset, i.k_offset, i.v_offset, i.sinks_offset, i.start, i.window, i.slots)
-        for i in items])
+        _Item(*[_u64(n, getattr(i, n)) for n in DecodeItem.__slots__]) for i in items])
 
 
 class PrepareItem:
@@ -241,7 +247,7 @@ class PrepareItem:
 
 def prepare_items(items):
     """A prepared table of ``PrepareItem`` (built once, reused while the offsets hold)."""
-    return (_PrepareItem * len(items))(*[_PrepareItem(*[getattr(i, n) for n in _PREPARE_FIELDS]) for i in items])
+    return (_PrepareItem * len(items))(*[_PrepareItem(*[_u64(n, getattr(i, n)) for n in _PREPARE_FIELDS]) for i in items])
 
 
 def split_q8_0_blocks(raw):

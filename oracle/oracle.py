@@ -111,6 +111,8 @@ def ring(all_rows, t, start, slots, tiled):
 
 def accepts(t, start, heads, kv_heads, dim, window, slots, tiled=False):
     """metal-compute/src/apple.rs:1243-1272 and 1356-1385."""
+    for value in (t, start, heads, kv_heads, dim, window, slots):  # ctypes would wrap 2**64 to 0 without a word
+        assert 0 <= int(value) < 2**64 and int(value) == value, value
     return bool(_lib.lng_oracle_accepts(t, start, heads, kv_heads, dim, window, slots, int(tiled)))
 
 
