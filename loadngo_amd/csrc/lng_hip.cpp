@@ -432,10 +432,18 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     return p;
 }
 
-// Records the kernels for a set of single-query rows (decode, and short passes row by row).
-int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n_rows, uint64_t t_uniform,
-                bool aligned16) {
-    lng_gpu *g = b->gpu;
+// What a set of single-query rows (decode, and short passes row by row) runs as.
+struct RowsPlan {
+    enum Kind { Generic, Bf16, F32 } kind = Generic;
+    DecodePlan chunks;
+    bool fused = false;          // split-K merged inside the decode kernel (tickets) instead of by lng_decode_merge
+    size_t partial_slots = 0;    // (row, kv head, chunk, query head of the group) slots of split-K partials; 0: none
+    size_t pairs = 0;            // rows x kv heads
+};
+
+RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, size_t n_rows, uint64_t t_uniform,
+                   bool aligned16) {
+    RowsPlan p;
     const uint32_t group = a.heads / a.kv_heads;
     const bool fast = a.dtype == LNG_BF16 && a.dim == 64 && group <= 16 && aligned16;
     // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the f32 matrix instruction
@@ -444,45 +452,104 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
     const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 16 && aligned16 && latest < 0xffffff00ull &&
                           a.scale > 0.0f && a.scale <= 3.0e38f && !getenv("LNG_F32_GENERIC");
-    if (!fast && !fast_f32) {
-        Cmd c;
-        c.fn = a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32;
-        c.name = a.dtype == LNG_BF16 ? "lng_attn_generic_bf16" : "lng_attn_generic_f32";
-        c.grid[0] = (unsigned)(n_rows * a.heads);
-        c.block = 256;
-        set_args(c, a);
-        b->cmds.push_back(std::move(c));
+    p.pairs = n_rows * (size_t)a.kv_heads;
+    if (!fast && !fast_f32) return p;
+    p.kind = fast ? RowsPlan::Bf16 : RowsPlan::F32;
+    p.chunks = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads, fast ? 1u : 2u);
+    if (p.chunks.n_chunks > 1) {
+        p.partial_slots = p.pairs * (size_t)p.chunks.n_chunks * group;
+        // Small grids merge inside the kernel; large ones with a second dispatch (the f32 kernel always).
+        p.fused = fast && (uint64_t)p.chunks.n_chunks * p.pairs <= 4ull * g->cus;
+    }
+    return p;
+}
+
+// The (at most two) launches of a planned set of rows.
+struct RowsLaunches {
+    int n = 0;
+    struct One {
+        hipFunction_t fn;
+        const char *name;
+        unsigned grid;
+        lng_k_attn args;
+    } l[2];
+};
+
+// `a` already names its scratch. With a table of rows of unequal length the decode kernel takes a list of
+// its live (pair, chunk) workgroups (`work_host` / `work_dev`, room for every live entry of 8 bytes, or NULL:
+// a rectangle of n_chunks workgroups per pair, those past a row's end returning at once).
+int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *host_rows, size_t n_rows,
+                  uint32_t *work_host, const uint32_t *work_dev, RowsLaunches *out) {
+    const uint32_t group = a.heads / a.kv_heads;
+    out->n = 0;
+    if (p.kind == RowsPlan::Generic) {
+        if (n_rows * (uint64_t)a.heads > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "%zu rows of %u heads are more workgroups than one dispatch holds", n_rows, a.heads);
+        out->l[out->n++] = {a.dtype == LNG_BF16 ? g->generic_bf16 : g->generic_f32,
+                            a.dtype == LNG_BF16 ? "lng_attn_generic_bf16" : "lng_attn_generic_f32",
+                            (unsigned)(n_rows * a.heads), a};
         return LNG_OK;
     }
-    const DecodePlan plan = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads, fast ? 1u : 2u);
-    a.chunk = plan.chunk;
-    a.n_chunks = plan.n_chunks;
-    if (plan.n_chunks > 1) {
-        const size_t slots = n_rows * a.kv_heads * (size_t)plan.n_chunks * group;
-        if (int rc = reserve_scratch(g, slots * 64, slots * 2, n_rows * (size_t)a.kv_heads)) return rc;
+    a.chunk = p.chunks.chunk;
+    a.n_chunks = p.chunks.n_chunks;
+    a.fused = p.fused ? 1u : 0u;
+    uint64_t wgs = (uint64_t)p.pairs * a.n_chunks;
+    if (wgs > 0x7fffffffull || (uint64_t)p.pairs * group > 0x7fffffffull) {
+        return fail(LNG_ERR_DISPATCH, "%zu rows of %u kv heads in %u chunks are more workgroups than one dispatch holds", n_rows, a.kv_heads, a.n_chunks);
+    }
+    a.work = nullptr;
+    if (work_host && a.n_chunks > 1) {
+        uint64_t n = 0;
+        for (size_t r = 0; r < n_rows; ++r) {
+            const uint64_t live = (visible_from_tile(host_rows[r]) + a.chunk - 1) / a.chunk;
+            for (uint32_t kv = 0; kv < a.kv_heads; ++kv) {
+                for (uint64_t c = 0; c < live; ++c) {
+                    work_host[2 * n] = (uint32_t)(r * a.kv_heads + kv);
+                    work_host[2 * n + 1] = (uint32_t)c;
+                    ++n;
+                }
+            }
+        }
+        a.work = work_dev;
+        wgs = n;
+    }
+    out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_d64 : g->decode_f32_d64,
+                        p.kind == RowsPlan::Bf16 ? "lng_decode_bf16_d64" : "lng_decode_f32_d64", (unsigned)wgs, a};
+    if (a.n_chunks > 1 && !a.fused) { // a workgroup per (row, kv head, query head)
+        out->l[out->n++] = {g->decode_merge, "lng_decode_merge", (unsigned)(p.pairs * group), a};
+    }
+    return LNG_OK;
+}
+
+// Records the kernels for a set of single-query rows (decode, and short passes row by row).
+int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n_rows, uint64_t t_uniform,
+                bool aligned16) {
+    lng_gpu *g = b->gpu;
+    const RowsPlan p = plan_rows(g, a, host_rows, n_rows, t_uniform, aligned16);
+    if (p.partial_slots) {
+        if (int rc = reserve_scratch(g, p.partial_slots * 64, p.partial_slots * 2, p.pairs)) return rc;
         a.partial_o = g->scratch_o;
         a.partial_ml = g->scratch_ml;
         a.tickets = g->tickets;
-        // Small grids merge inside the kernel; large ones with a second dispatch (the f32 kernel always).
-        a.fused = fast && (uint64_t)plan.n_chunks * n_rows * a.kv_heads <= 4ull * g->cus ? 1u : 0u;
     }
-    Cmd c;
-    c.fn = fast ? g->decode_bf16_d64 : g->decode_f32_d64;
-    c.name = fast ? "lng_decode_bf16_d64" : "lng_decode_f32_d64";
-    c.grid[0] = plan.n_chunks;
-    c.grid[1] = (unsigned)(n_rows * a.kv_heads);
-    c.block = 256;
-    set_args(c, a);
-    b->cmds.push_back(std::move(c));
-    if (plan.n_chunks > 1 && !a.fused) {
-        Cmd m;
-        m.fn = g->decode_merge;
-        m.name = "lng_decode_merge";
-        m.grid[0] = group; // a workgroup per (row, kv head, query head)
-        m.grid[1] = (unsigned)(n_rows * a.kv_heads);
-        m.block = 256;
-        set_args(m, a);
-        b->cmds.push_back(std::move(m));
+    // Rows of unequal length (a table of sequences): room for the list of live workgroups.
+    char *work_host = nullptr, *work_dev = nullptr;
+    if (!t_uniform && p.chunks.n_chunks > 1 && p.kind != RowsPlan::Generic) {
+        uint64_t live = 0;
+        for (size_t r = 0; r < n_rows; ++r) live += (visible_from_tile(host_rows[r]) + p.chunks.chunk - 1) / p.chunks.chunk;
+        if (live < (uint64_t)n_rows * p.chunks.n_chunks && live * a.kv_heads <= 0x7fffffffull) {
+            if (int rc = reserve_table(b, live * a.kv_heads * 8, &work_host, &work_dev)) return rc;
+        }
+    }
+    RowsLaunches launches;
+    if (int rc = rows_launches(g, a, p, host_rows, n_rows, (uint32_t *)work_host, (const uint32_t *)work_dev, &launches)) return rc;
+    for (int i = 0; i < launches.n; ++i) {
+        Cmd c;
+        c.fn = launches.l[i].fn;
+        c.name = launches.l[i].name;
+        c.grid[0] = launches.l[i].grid;
+        c.block = 256;
+        set_args(c, launches.l[i].args);
+        b->cmds.push_back(std::move(c));
     }
     return LNG_OK;
 }

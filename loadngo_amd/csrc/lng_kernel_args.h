@@ -24,13 +24,15 @@ typedef struct lng_k_attn {
     float *partial_o;         /* split-K scratch: [row][kv_head][chunk][group][dim] f32 */
     float *partial_ml;        /* split-K scratch: [row][kv_head][chunk][group][2] f32 (max, sum) */
     uint32_t *tickets;        /* split-K scratch: [row][kv_head] arrival counters, zero between dispatches */
+    const uint32_t *work;     /* device list of (row * kv_heads + kv head, chunk) pairs, one per workgroup of a decode
+                                 kernel, or NULL: workgroup w takes pair w / n_chunks, chunk w % n_chunks */
     lng_k_row first;          /* row 0 when rows == NULL; row i: q/out advance by one row, start by i */
     uint32_t n_rows;
     uint32_t heads;
     uint32_t kv_heads;
     uint32_t dim;
     uint32_t chunk;           /* positions per workgroup along the cache (multiple of 128) */
-    uint32_t n_chunks;        /* workgroups along the cache = ceil(longest visible run / chunk) */
+    uint32_t n_chunks;        /* chunks of the longest visible run = ceil(it / chunk): the partials keep this many slots per (row, kv head) */
     uint32_t dtype;           /* lng_dtype of q, k, v, out */
     uint32_t fused;           /* split-K: 1 = the last workgroup of a row merges, 0 = lng_decode_merge follows */
     float scale;

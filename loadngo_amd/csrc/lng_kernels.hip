@@ -61,6 +61,28 @@ __device__ __forceinline__ uint64_t first_visible(uint64_t last, uint64_t window
     return (window != LNG_WINDOW_FULL && last + 1 > window) ? last + 1 - window : 0;
 }
 
+// Which (row, kv head) pair and which chunk of its visible run a decode workgroup takes: from the
+// host's list of live (pair, chunk) items when there is one (rows of unequal length: no workgroup is
+// launched only to return), else from a rectangle of n_chunks per pair, chunks the fast index.
+struct work_item {
+    uint32_t pair;
+    uint32_t chunk;
+};
+__device__ __forceinline__ work_item work_of(const lng_k_attn &a) {
+    work_item w;
+    if (a.work) {
+        const uint2 x = ((const uint2 *)a.work)[blockIdx.x];
+        w.pair = x.x;
+        w.chunk = x.y;
+    } else {
+        w.pair = blockIdx.x / a.n_chunks;
+        w.chunk = blockIdx.x % a.n_chunks;
+    }
+    w.pair = __builtin_amdgcn_readfirstlane(w.pair);
+    w.chunk = __builtin_amdgcn_readfirstlane(w.chunk);
+    return w;
+}
+
 // Sum over the 64 lanes, in every lane: four steps inside each row of 16 lanes with data-parallel
 // primitives (neighbour, pair, mirrored half row, mirrored row), then the two lane-swap instructions
 // across rows. All VALU: the shuffle form goes through the LDS crossbar six times, one after the other.
@@ -214,7 +236,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_attn_generic_bf16(lng_k_at
 // =============================================================================================
 // Decode kernel, bf16, head width 64, up to 16 query heads per kv head.
 //
-// Grid: x = chunk of the cache (a.chunk positions), y = row * kv_heads + kv head. A workgroup
+// Grid: one workgroup per (row, kv head, chunk of a.chunk cached positions), see work_of. A workgroup
 // serves ALL query heads of its kv head at once, so each cached K and V row is read from HBM
 // once per group instead of once per query head. Its four wavefronts take interleaved tiles
 // of 32 positions. Everything is lane-local between the three MFMA stages:
@@ -266,15 +288,15 @@ template <bool COHERENT> __device__ __forceinline__ float load_partial(const flo
 }
 
 template <bool COHERENT>
-__device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_row &it, uint32_t g, uint32_t group,
-                                             uint32_t row_chunks) {
+__device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_row &it, uint32_t pair, uint32_t g,
+                                             uint32_t group, uint32_t row_chunks) {
     __shared__ float s_w[16][LNG_MAX_CHUNKS];
     __shared__ float s_z[16];
     {
         const uint32_t h = threadIdx.x >> 4, t16 = threadIdx.x & 15u;
         if (h < group) {
             const uint32_t head = g * group + h;
-            const uint64_t slot0 = ((uint64_t)blockIdx.y * a.n_chunks) * group + h;
+            const uint64_t slot0 = ((uint64_t)pair * a.n_chunks) * group + h;
             const float sink2 = it.sinks_offset != LNG_NO_SINKS
                                     ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
                                     : LNG_NEG_INF;
@@ -303,7 +325,7 @@ __device__ __forceinline__ void merge_chunks(const lng_k_attn &a, const lng_k_ro
     for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
         const uint32_t h = idx >> 6;
         const uint32_t d = idx & 63u;
-        const float *po = a.partial_o + (((uint64_t)blockIdx.y * a.n_chunks) * group + h) * 64u + d;
+        const float *po = a.partial_o + (((uint64_t)pair * a.n_chunks) * group + h) * 64u + d;
         const uint64_t step = (uint64_t)group * 64u;
         // sixteen loads in flight per turn: the merge is a chain of memory latencies otherwise
         float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
@@ -351,13 +373,14 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
 
-    const uint32_t row = blockIdx.y / a.kv_heads;
-    const uint32_t g = blockIdx.y % a.kv_heads;
+    const work_item wi = work_of(a);
+    const uint32_t row = wi.pair / a.kv_heads;
+    const uint32_t g = wi.pair % a.kv_heads;
     const lng_k_row it = row_of(a, row);
     const uint64_t last = it.start;
     const uint64_t first = first_visible(last, it.window);
     const uint64_t base = first & ~(uint64_t)31;
-    const uint64_t c0 = base + (uint64_t)blockIdx.x * a.chunk;
+    const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
     if (c0 > last) return; // this row has fewer chunks than the longest one
     const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
@@ -509,7 +532,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
             uint16_t *op = (uint16_t *)(a.out + it.out_offset) + (uint64_t)head * 64u + d;
             *op = f32_to_bf16_bits(o * keep / z);
         } else {
-            const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
+            const uint64_t slot = ((uint64_t)wi.pair * a.n_chunks + wi.chunk) * group + h;
             if (a.fused) {
                 // device-coherent stores: visible to every XCD once acknowledged, no cache write-back
                 __hip_atomic_store(&a.partial_o[slot * 64u + d], o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -529,19 +552,22 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
     if (row_chunks == 1 || !a.fused) return;
 
     // ---- split-K: the workgroup that finishes last for this (row, kv head) merges the partials ----
-    // Every thread waits for its own coherent stores to be acknowledged, the workgroup meets, and
-    // one thread takes a ticket; whoever draws the last ticket reads the partials back with
-    // coherent loads. No cache-wide write-back or invalidate is involved. The ticket counter
-    // returns to zero for the next dispatch (dispatches run in stream order).
+    // Release: every thread makes its partial stores visible to the whole device (agent-scope release
+    // fence: it waits for the thread's outstanding stores and writes back what this XCD's L2 still
+    // holds), the workgroup meets, and one thread takes a ticket. Acquire: whoever draws the last
+    // ticket passes an agent-scope acquire fence before it reads the partials back with coherent
+    // loads. Only small grids come here, so the fences touch little. The ticket counter returns to
+    // zero for the next dispatch (dispatches run in stream order).
     __shared__ uint32_t s_ticket;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
     __syncthreads();
-    if (threadIdx.x == 0) s_ticket = atomicAdd(&a.tickets[blockIdx.y], 1u);
+    if (threadIdx.x == 0) s_ticket = __hip_atomic_fetch_add(&a.tickets[wi.pair], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != row_chunks - 1u) return;
-    if (threadIdx.x == 0) __hip_atomic_store(&a.tickets[blockIdx.y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (threadIdx.x == 0) __hip_atomic_store(&a.tickets[wi.pair], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
-    merge_chunks<true>(a, it, g, group, row_chunks);
+    merge_chunks<true>(a, it, wi.pair, g, group, row_chunks);
 }
 
 // =============================================================================================
@@ -571,14 +597,15 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
 
-    const uint32_t row = blockIdx.y / a.kv_heads;
-    const uint32_t g = blockIdx.y % a.kv_heads;
+    const work_item wi = work_of(a);
+    const uint32_t row = wi.pair / a.kv_heads;
+    const uint32_t g = wi.pair % a.kv_heads;
     const lng_k_row it = row_of(a, row);
     // positions and slots fit 32 bits (the host refuses shapes whose counts do not)
     const uint32_t last = (uint32_t)it.start;
     const uint32_t first = (uint32_t)first_visible(it.start, it.window);
     const uint32_t base = first & ~31u;
-    const uint64_t c0w = (uint64_t)base + (uint64_t)blockIdx.x * a.chunk;
+    const uint64_t c0w = (uint64_t)base + (uint64_t)wi.chunk * a.chunk;
     if (c0w > last) return; // this row has fewer chunks than the longest one
     const uint32_t c0 = (uint32_t)c0w;
     const uint32_t c1 = (c0w + a.chunk < (uint64_t)last + 1u) ? (uint32_t)(c0w + a.chunk) : last + 1u; // last + 1 fits: last < 2^32 - 1 here or the chunk ends earlier
@@ -739,7 +766,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
             const float z = sum * keep + (sink == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink - all));
             ((float *)(a.out + it.out_offset))[(uint64_t)head * 64u + d] = o * keep / z;
         } else { // lng_decode_merge follows
-            const uint64_t slot = ((uint64_t)blockIdx.y * a.n_chunks + blockIdx.x) * group + h;
+            const uint64_t slot = ((uint64_t)wi.pair * a.n_chunks + wi.chunk) * group + h;
             a.partial_o[slot * 64u + d] = o;
             if (d == 0) {
                 a.partial_ml[slot * 2u] = top;
@@ -751,23 +778,24 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
 
 // The merge as its own dispatch, for large grids (there a workgroup that waits for its coherent stores and
 // its ticket holds a compute unit's slot that another chunk could use) and for the f32 kernel. One workgroup
-// per (row, kv head, query head): thread c turns chunk c's (max, sum) into a weight, then thread (dim, quarter)
+// per (row, kv head, query head), the query head the fast index of the grid: thread c turns chunk c's (max, sum) into a weight, then thread (dim, quarter)
 // adds every fourth chunk's partial output and the quarters meet in LDS: eight times the workgroups of a
 // merge per (row, kv head) and a quarter of the chain of loads per thread.
 extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a) {
     __shared__ float s_w[LNG_MAX_CHUNKS];
     __shared__ float s_red[2][4];
     __shared__ float s_acc[4][64];
-    const uint32_t row = blockIdx.y / a.kv_heads;
-    const uint32_t g = blockIdx.y % a.kv_heads;
+    const uint32_t group = a.heads / a.kv_heads, h = blockIdx.x % group, pair = blockIdx.x / group;
+    const uint32_t row = pair / a.kv_heads;
+    const uint32_t g = pair % a.kv_heads;
     const lng_k_row it = row_of(a, row);
     const uint64_t last = it.start;
     const uint64_t base = first_visible(last, it.window) & ~(uint64_t)31;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
     if (row_chunks == 1) return; // the decode kernel already wrote this row
-    const uint32_t group = a.heads / a.kv_heads, h = blockIdx.x, head = g * group + h;
+    const uint32_t head = g * group + h;
     const uint32_t tid = threadIdx.x, wave = tid >> 6;
-    const uint64_t slot0 = ((uint64_t)blockIdx.y * a.n_chunks) * group + h;
+    const uint64_t slot0 = ((uint64_t)pair * a.n_chunks) * group + h;
     const float sink2 = it.sinks_offset != LNG_NO_SINKS ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
                                                          : LNG_NEG_INF;
     float mc = LNG_NEG_INF, lc = 0.0f;
@@ -2261,5 +2289,5 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     lng_k_row it{};
     it.out_offset = (uint64_t)row * p.heads * 64u * (p.dtype == LNG_F32 ? 4u : 2u);
     it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;
-    merge_chunks<false>(a, it, g, group, p.splits);
+    merge_chunks<false>(a, it, blockIdx.y, g, group, p.splits);
 }
