@@ -171,6 +171,26 @@ int lng_hip_attention_grouped_tiled(lng_batch *batch, lng_slice q, lng_slice k, 
                                     lng_slice out, const lng_slice *sinks,
                                     const lng_grouped_shape *shape, int dtype);
 
+/* No counterpart in the reference: lng_hip_attention_grouped for callers that cannot allocate - code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It takes raw device
+ * addresses instead of slices of a batch, launches at once on the caller's stream `stream` (a hipStream_t;
+ * NULL is the default stream) and returns without waiting; it calls no hipMalloc, hipFree or pinned
+ * allocation and keeps nothing on the host heap. q, out: [t][heads][dim]; k, v: [min(slots, start + t)]
+ * [kv_heads][dim]; sinks: [heads] f32 or NULL; every row is computed as the plain operator computes it
+ * (same shape rules and refusals; operands aligned to their element size; the output may not overlap an
+ * input). The caller vouches for the sizes behind the addresses.
+ *
+ * Split-K partials go to a fixed array of LNG_STATIC_SCRATCH_SLOTS x 264 bytes (16.5 MiB) that every GPU the
+ * library is opened on holds until the process ends. The limit: t x heads <= LNG_STATIC_MAX_ROW_HEADS (32
+ * rows of 64 heads); more is refused with LNG_ERR_DISPATCH (the partials of such a call always fit: a row
+ * is cut into at most 32 chunks once a call has 128 (row, kv head) pairs or more). Every call on one GPU
+ * shares that array: calls that may overlap in time on one GPU (different streams with no ordering between
+ * them) race on it. Nothing in it has to start at zero: a call overwrites every slot it later reads. */
+#define LNG_STATIC_SCRATCH_SLOTS 65536u
+#define LNG_STATIC_MAX_ROW_HEADS 2048u
+int lng_hip_attention_grouped_static(lng_gpu *gpu, void *stream, const void *q, const void *k, const void *v,
+                                     void *out, const float *sinks, const lng_grouped_shape *shape, int dtype);
+
 /* apple.rs:1762 Batch::copy_rows((src, src_stride), (dst, dst_stride), rows, width): how
  * gpt-oss/src/gpu.rs:744-759 writes new K and V rows into a cache. Strides and width count
  * elements. src_dtype != dst_dtype converts (f32 -> bf16 rounds to nearest even): the new

@@ -1,5 +1,6 @@
 """Builds liblng_hip.so in-tree: the gfx950 code object from csrc/lng_kernels.hip
-(``hipcc --genco``), embedded into the host library compiled from csrc/lng_hip.cpp.
+(``hipcc --genco``), embedded into the host library compiled from csrc/lng_hip.cpp, plus
+csrc/lng_static.hip (the fixed device scratch array and the host code that finds it).
 
     python -m loadngo_amd.build
 """
@@ -34,11 +35,18 @@ def build(verbose=False):
     out = _run([hipcc] + DEVICE_FLAGS + [os.path.join(CSRC, "lng_kernels.hip"), "-o", HSACO])
     if verbose and out:
         print(out)
+    # the fixed scratch array and its set-up: a HIP source of its own (device array + the host code that finds it)
+    static_obj = os.path.join(HERE, "lng_static.o")
+    out = _run([hipcc, "-c", "-fPIC", "--offload-arch=gfx950", "-O2", "-std=c++17",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                os.path.join(CSRC, "lng_static.hip"), "-o", static_obj])
+    if verbose and out:
+        print(out)
     out = _run([
         "g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wextra", "-Wno-unused-result", "-pthread",
         "-D__HIP_PLATFORM_AMD__", "-DLNG_HSACO_PATH=\"%s\"" % HSACO,
         "-I" + os.path.join(ROCM, "include"),
-        os.path.join(CSRC, "lng_hip.cpp"), "-o", LIB,
+        os.path.join(CSRC, "lng_hip.cpp"), static_obj, "-o", LIB,
         "-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(ROCM, "lib"),
     ])
     if verbose and out:

@@ -120,6 +120,7 @@ SYMBOLS = {
                                                  ctypes.POINTER(_Shape), ctypes.c_int]),
     "lng_hip_attention_grouped_tiled": (ctypes.c_int, [_P, _Slice, _Slice, _Slice, _Slice, ctypes.POINTER(_Slice),
                                                        ctypes.POINTER(_Shape), ctypes.c_int]),
+    "lng_hip_attention_grouped_static": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, ctypes.POINTER(_Shape), ctypes.c_int]),
     "lng_hip_copy_rows": (ctypes.c_int, [_P, _Slice, _U64, ctypes.c_int, _Slice, _U64, ctypes.c_int, _U64, _U64]),
     "lng_hip_attention_decode_batched": (ctypes.c_int, [_P, _U64, _U64, _U64, _U64, _U64, ctypes.POINTER(_Item),
                                                         ctypes.c_size_t, _U64, _U64, _U64, ctypes.c_float,
@@ -366,6 +367,13 @@ class Gpu:
 
     def batch(self, buffers, dispatch="serial"):
         return Batch(self, list(buffers))
+
+    def attention_grouped_static(self, q, k, v, out, sinks, shape, dtype=F32, stream=None):
+        """The plain operator on raw device addresses (``Buffer.device_ptr()`` plus a byte offset), launched at
+        once on ``stream`` (a hipStream_t as an integer; None: the default stream) without allocating anything;
+        no counterpart in the reference. Returns without waiting."""
+        _check(library().lng_hip_attention_grouped_static(self._h, stream, q, k, v, out, sinks or None,
+                                                          ctypes.byref(shape._c()), dtype))
 
     def close(self):
         if self._h:

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "lng_kernel_args.h"
+#include "lng_static.h"
 
 // The code object, placed in .rodata by the assembler (path given by the build).
 #ifndef LNG_HSACO_PATH
@@ -108,6 +109,7 @@ struct lng_gpu {
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
     std::atomic<long> live_buffers{0};
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
+    char *static_scratch = nullptr; // this device's copy of the fixed scratch array (LNG_STATIC_SCRATCH_BYTES)
 
     // completion thread (only for batches committed with a callback)
     std::thread worker;
@@ -464,7 +466,8 @@ RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, 
     return p;
 }
 
-// The (at most two) launches of a planned set of rows.
+// The (at most two) launches of a planned set of rows; no heap, so that the entry point that allocates
+// nothing can share it.
 struct RowsLaunches {
     int n = 0;
     struct One {
@@ -776,6 +779,15 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         delete g;
         return fail(LNG_ERR_NO_DEVICE, "cannot create a stream");
     }
+    // this device's copy of the fixed scratch array (for lng_hip_attention_grouped_static)
+    if (const int rc = lng_static_scratch_setup(device)) {
+        const int code = fail(LNG_ERR_COMPILE, "the fixed scratch array is not there on device %d: %s", device, hip_text((hipError_t)rc));
+        hipStreamDestroy(g->stream);
+        hipModuleUnload(g->module);
+        delete g;
+        return code;
+    }
+    g->static_scratch = (char *)lng_static_scratch(device);
     if (const char *env = getenv("LNG_DECODE_WGS")) {
         const long n = atol(env);
         if (n >= 1 && n <= (1 << 20)) g->decode_wgs = (unsigned)n;
@@ -1069,6 +1081,79 @@ extern "C" int lng_hip_attention_grouped(lng_batch *b, lng_slice q, lng_slice k,
 extern "C" int lng_hip_attention_grouped_tiled(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out,
                                                const lng_slice *sinks, const lng_grouped_shape *shape, int dtype) {
     return attention(b, q, k, v, out, sinks, shape, dtype, true);
+}
+
+// The plain operator on raw device pointers, launched at once on the caller's stream, with its split-K
+// partials in the fixed scratch array: no hipMalloc, no hipFree, no pinned tables, no host heap.
+extern "C" int lng_hip_attention_grouped_static(lng_gpu *g, void *stream, const void *q, const void *k, const void *v,
+                                                void *out, const float *sinks, const lng_grouped_shape *shape,
+                                                int dtype) {
+    if (!g) return fail(LNG_ERR_DISPATCH, "no gpu");
+    if (!shape) return fail(LNG_ERR_DISPATCH, "no shape");
+    if (dtype != LNG_F32 && dtype != LNG_BF16) return fail(LNG_ERR_DISPATCH, "unknown element type %d", dtype);
+    if (!q || !k || !v || !out) return fail(LNG_ERR_DISPATCH, "q, k, v and out must be device addresses");
+    const lng_grouped_shape &s = *shape;
+    if (int rc = check_shape(s, false)) return rc;
+    if (s.t * s.heads > LNG_STATIC_MAX_ROW_HEADS) {
+        return fail(LNG_ERR_DISPATCH, "%llu rows of %llu heads: the fixed scratch array is sized for rows x heads <= %u",
+                    (unsigned long long)s.t, (unsigned long long)s.heads, (unsigned)LNG_STATIC_MAX_ROW_HEADS);
+    }
+    const uint64_t es = elem_size(dtype);
+    if (!fits_u32(s.heads * s.dim * es)) return fail(LNG_ERR_DISPATCH, "rows of %llu bytes do not fit in u32", (unsigned long long)(s.heads * s.dim * es));
+    const uint64_t end = s.start + s.t;
+    const uint64_t q_bytes = s.t * s.heads * s.dim * es, kv_bytes = std::min(s.slots, end) * s.kv_heads * s.dim * es;
+    const uintptr_t pq = (uintptr_t)q, pk = (uintptr_t)k, pv = (uintptr_t)v, po = (uintptr_t)out;
+    if ((pq | pk | pv | po) % es != 0 || (uintptr_t)sinks % 4 != 0) return fail(LNG_ERR_DISPATCH, "an operand is not aligned to its element size");
+    // apple.rs:896-906: the output may not overlap an input
+    auto apart = [&](uintptr_t x, uint64_t n) { return po + q_bytes <= x || x + n <= po; };
+    if (!apart(pq, q_bytes) || !apart(pk, kv_bytes) || !apart(pv, kv_bytes) || (sinks && !apart((uintptr_t)sinks, s.heads * 4))) {
+        return fail(LNG_ERR_DISPATCH, "output overlaps an input");
+    }
+    lng_k_attn a{};
+    a.q = (const char *)q;
+    a.k = (const char *)k;
+    a.v = (const char *)v;
+    a.out = (char *)out;
+    a.sinks = (const char *)sinks;
+    a.rows = nullptr;
+    a.first.sinks_offset = sinks ? 0 : LNG_NO_SINKS;
+    a.first.start = s.start;
+    a.first.window = s.window;
+    a.first.slots = s.slots;
+    a.n_rows = (uint32_t)s.t;
+    a.heads = (uint32_t)s.heads;
+    a.kv_heads = (uint32_t)s.kv_heads;
+    a.dim = (uint32_t)s.dim;
+    a.chunk = 128;
+    a.n_chunks = 1;
+    a.dtype = (uint32_t)dtype;
+    a.scale = s.scale;
+    const bool aligned16 = ((pq | pk | pv | po) & 15u) == 0;
+    RowsPlan p = plan_rows(g, a, &a.first, s.t, s.t, aligned16);
+    p.fused = false; // lng_decode_merge as the second launch: no arrival counters, nothing that must start at zero
+    if (p.partial_slots > LNG_STATIC_MAX_SLOTS) { // only a planner told to make more workgroups than usual gets here
+        return fail(LNG_ERR_DISPATCH,
+                    "%llu rows of %llu heads in %u chunks need %zu slots of split-K scratch; the fixed array holds %u (%zu bytes)",
+                    (unsigned long long)s.t, (unsigned long long)s.heads, p.chunks.n_chunks, p.partial_slots,
+                    (unsigned)LNG_STATIC_MAX_SLOTS, (size_t)LNG_STATIC_SCRATCH_BYTES);
+    }
+    if (p.partial_slots) {
+        if (!g->static_scratch) return fail(LNG_ERR_COMPILE, "the fixed scratch array was not set up");
+        a.partial_o = (float *)g->static_scratch;
+        a.partial_ml = (float *)(g->static_scratch + LNG_STATIC_O_BYTES);
+        a.tickets = nullptr;
+    }
+    RowsLaunches launches;
+    if (int rc = rows_launches(g, a, p, &a.first, s.t, nullptr, nullptr, &launches)) return rc;
+    if (hipSetDevice(g->device) != hipSuccess) return fail(LNG_ERR_NO_DEVICE, "cannot select HIP device %d", g->device);
+    for (int i = 0; i < launches.n; ++i) {
+        size_t size = sizeof(lng_k_attn);
+        void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launches.l[i].args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                          HIP_LAUNCH_PARAM_END};
+        const hipError_t e = hipModuleLaunchKernel(launches.l[i].fn, launches.l[i].grid, 1, 1, 256, 1, 1, 0, (hipStream_t)stream, nullptr, config);
+        if (e != hipSuccess) return fail(LNG_ERR_GPU, "%s did not launch: %s", launches.l[i].name, hip_text(e));
+    }
+    return LNG_OK;
 }
 
 extern "C" int lng_hip_copy_rows(lng_batch *b, lng_slice src, uint64_t src_stride, int src_dtype, lng_slice dst,
