@@ -29,7 +29,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 from loadngo_amd import compute as C  # noqa: E402
-from loadngo_amd.synthetic import bf16_bits, bf16_widen  # noqa: E402
+from loadngo_amd.synthetic import bf16_bits, bf16_widen, synthetic_values  # noqa: E402
 
 H, G, D = 64, 8, 64
 SCALE = 0.125
@@ -62,49 +62,125 @@ def fill(gpu, buf, seed, scale=0.5, period=0):
 
 
 # ------------------------------------------------------------------------------------------------
-def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24, kv_gap_gib=None):
-    """Configuration 5: the 24-layer decode stack. Caches are allocated layer by layer, K then V, as
-    gpt-oss/src/gpu.rs:567-578 does; kv_gap_gib = N allocates all K caches, N GiB left unused, then all
-    V caches (an experiment on how placement in HBM changes the rate)."""
-    log("allocating %.1f GiB of KV cache" % (layers * 2 * batch_size * ctx * ROW / 2**30))
-    q = gpu.buffer(layers * batch_size * QO)
-    out = gpu.buffer(layers * batch_size * QO)
-    sinks = gpu.upload(np.random.default_rng(5).standard_normal((layers, H)).astype(np.float32))
-    fill(gpu, q, 1000)
-    caches, unused = [], []
-    if kv_gap_gib is None:
-        for l in range(layers):
-            caches += [gpu.buffer(batch_size * ctx * ROW), gpu.buffer(batch_size * ctx * ROW)]
-    else:
-        ks = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
-        if kv_gap_gib:
-            unused.append(gpu.buffer(kv_gap_gib << 30))
-        vs = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
-        for l in range(layers):
-            caches += [ks[l], vs[l]]
-    for i, b in enumerate(caches):
-        fill(gpu, b, i + 1)
-    bufs = [q, out, sinks] + caches
-    tables = []
-    step_bytes = 0
-    for l in range(layers):
-        window = 128 if l % 2 == 0 else C.FULL  # even layers slide (gpt-oss/src/config.rs:99-103)
-        items = [C.DecodeItem((l * batch_size + b) * QO, (l * batch_size + b) * QO, b * ctx * ROW, b * ctx * ROW,
-                              l * H * 4, ctx - 1, window, ctx) for b in range(batch_size)]
-        tables.append(C.decode_items(items))
-        step_bytes += batch_size * decode_bytes(ctx, window)
+STACK_PERIOD = 1024  # positions after which the checking fill repeats
 
-    def step(timing):
-        batch = gpu.batch(bufs)
+
+class Stack:
+    """Configuration 5: the 24-layer decode stack, its caches resident. Caches are allocated layer by layer,
+    K then V, as gpt-oss/src/gpu.rs:567-578 does; kv_gap_gib = N allocates all K caches, N GiB left unused,
+    then all V caches (an experiment on how placement in HBM changes the rate). Cache 2l is layer l's K
+    (fill seed 2l + 1), cache 2l + 1 its V (seed 2l + 2); queries are seed 1000; sinks are N(0,1), seed 5."""
+
+    def __init__(self, gpu, batch_size=16, ctx=131072, layers=24, kv_gap_gib=None):
+        self.gpu, self.batch_size, self.ctx, self.layers = gpu, batch_size, ctx, layers
+        log("allocating %.1f GiB of KV cache" % (layers * 2 * batch_size * ctx * ROW / 2**30))
+        self.q = gpu.buffer(layers * batch_size * QO)
+        self.out = gpu.buffer(layers * batch_size * QO)
+        self.sink_values = np.random.default_rng(5).standard_normal((layers, H)).astype(np.float32)
+        self.sinks = gpu.upload(self.sink_values)
+        fill(gpu, self.q, 1000)
+        self.caches, self.unused = [], []
+        if kv_gap_gib is None:
+            for l in range(layers):
+                self.caches += [gpu.buffer(batch_size * ctx * ROW), gpu.buffer(batch_size * ctx * ROW)]
+        else:
+            ks = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
+            if kv_gap_gib:
+                self.unused.append(gpu.buffer(kv_gap_gib << 30))
+            vs = [gpu.buffer(batch_size * ctx * ROW) for _ in range(layers)]
+            for l in range(layers):
+                self.caches += [ks[l], vs[l]]
+        self.bufs = [self.q, self.out, self.sinks] + self.caches
+        self.tables = []
+        self.step_bytes = 0
+        for l in range(layers):
+            window = self.window(l)
+            items = [C.DecodeItem((l * batch_size + b) * QO, (l * batch_size + b) * QO, b * ctx * ROW, b * ctx * ROW,
+                                  l * H * 4, ctx - 1, window, ctx) for b in range(batch_size)]
+            self.tables.append(C.decode_items(items))
+            self.step_bytes += batch_size * decode_bytes(ctx, window)
+
+    @staticmethod
+    def window(layer):
+        return 128 if layer % 2 == 0 else C.FULL  # even layers slide (gpt-oss/src/config.rs:99-103)
+
+    def fill_caches(self, period=0):
+        """Fills every cache on the device; period (positions) > 0 makes each cache repeat after that many
+        positions (the sequences of a cache then hold the same rows)."""
+        for i, b in enumerate(self.caches):
+            fill(self.gpu, b, i + 1, period=period * G * D)
+
+    def step(self, timing=False):
+        """One decoding step: 24 batched-decode dispatches in one batch. Returns (gpu seconds, (decode kernel
+        seconds, launches) when timing)."""
+        batch = self.gpu.batch(self.bufs)
         if timing:
             batch.set_timing(True)
-        for l in range(layers):
-            batch.attention_decode_batched(0, 3 + 2 * l, 4 + 2 * l, 1, 2, tables[l], H, G, D, SCALE, C.BF16)
+        for l in range(self.layers):
+            batch.attention_decode_batched(0, 3 + 2 * l, 4 + 2 * l, 1, 2, self.tables[l], H, G, D, SCALE, C.BF16)
         batch.commit()
         done = batch.wait()
+        if isinstance(done.gpu_time, Exception):
+            raise done.gpu_time
         ks = batch.kernel_seconds("lng_decode_bf16_d64") if timing else (0.0, 0)
         batch.drop()
         return done.gpu_time, ks
+
+    def outputs(self):
+        """[layers][batch][H][D] f32 of what the last step wrote."""
+        return bf16_widen(self.out.read(np.uint16)).reshape(self.layers, self.batch_size, H, D)
+
+    def queries(self):
+        return bf16_bits(synthetic_values(self.layers * self.batch_size * H * D, 1000, 0.5)).reshape(
+            self.layers, self.batch_size, H, D)
+
+    def check_window_layers(self, got, oracle, period=0):
+        """Every row of every 128-window layer against the oracle on the host's restatement of the fill (the
+        last 128 positions of each sequence: cheap whatever the fill). Returns the largest error."""
+        q = self.queries()
+        worst = 0.0
+        for l in range(0, self.layers, 2):
+            for b in range(self.batch_size):
+                first = (b * self.ctx + self.ctx - 128) * G * D
+                k = bf16_bits(synthetic_values(128 * G * D, 2 * l + 1, 0.5, period * G * D, first)).reshape(128, G, D)
+                v = bf16_bits(synthetic_values(128 * G * D, 2 * l + 2, 0.5, period * G * D, first)).reshape(128, G, D)
+                want = oracle.attention_bf16(q[l, b:b + 1], k, v, self.sink_values[l], 127, window=128, scale=SCALE)
+                err = np.abs(got[l, b] - bf16_widen(want[0]))
+                worst = max(worst, float(np.inf if np.isnan(err).any() else err.max()))
+        return worst
+
+    def check_full_layers_periodic(self, got, oracle):
+        """With the caches filled with period STACK_PERIOD, every weight of a full-causal layer appears
+        ctx / STACK_PERIOD times, so the exact result is attention over one period with the sink lowered by
+        ln(ctx / STACK_PERIOD) (a property of the softmax, pinned on the oracle by its own tests). Every row of
+        every full-causal layer. Returns the largest error."""
+        assert self.ctx % STACK_PERIOD == 0
+        q = self.queries()
+        lowered = self.sink_values - np.float32(np.log(self.ctx // STACK_PERIOD))
+        worst = 0.0
+        for l in range(1, self.layers, 2):
+            k = bf16_bits(synthetic_values(STACK_PERIOD * G * D, 2 * l + 1, 0.5)).reshape(STACK_PERIOD, G, D)
+            v = bf16_bits(synthetic_values(STACK_PERIOD * G * D, 2 * l + 2, 0.5)).reshape(STACK_PERIOD, G, D)
+            for b in range(self.batch_size):
+                want = oracle.attention_bf16(q[l, b:b + 1], k, v, lowered[l], STACK_PERIOD - 1, scale=SCALE, threads=8)
+                err = np.abs(got[l, b] - bf16_widen(want[0]))
+                worst = max(worst, float(np.inf if np.isnan(err).any() else err.max()))
+        return worst
+
+    def free(self):
+        for b in self.bufs + self.unused:
+            b.free()
+
+
+def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24, kv_gap_gib=None, check=True):
+    """Configuration 5, timed; then (outside the timed region) its outputs are checked: the timed step's
+    window layers against the oracle on the same fill, and, after refilling the caches with a fill that
+    repeats every STACK_PERIOD positions, one more step whose every row - 24 layers x 16 sequences x 64 heads -
+    is held to the bf16 bar (2e-2) through the periodic identity."""
+    stack = Stack(gpu, batch_size, ctx, layers, kv_gap_gib)
+    stack.fill_caches()
+    step = stack.step
+    step_bytes = stack.step_bytes
 
     for _ in range(warmup):
         step(False)
@@ -123,8 +199,26 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24, kv_gap_g
         _, (ks, kn) = step(True)
         kern_s += ks
         launches += kn
-    for b in bufs + unused:
-        b.free()
+    checked = None
+    if check:
+        from oracle import oracle  # the checker only: nothing timed above touches it
+        got = stack.outputs()
+        assert np.isfinite(got).all(), "the timed step left outputs that are not finite"
+        e_window = stack.check_window_layers(got, oracle)
+        assert e_window < 2e-2, "window layers of the timed step are %.3g from the oracle" % e_window
+        checked = {"window_layers_of_the_timed_step_max_abs_err": e_window}
+        if ctx % STACK_PERIOD == 0:
+            stack.fill_caches(STACK_PERIOD)
+            stack.out.fill(0xFF)
+            step(False)
+            got = stack.outputs()
+            e_full = stack.check_full_layers_periodic(got, oracle)
+            e_win2 = stack.check_window_layers(got, oracle, STACK_PERIOD)
+            assert e_full < 2e-2 and e_win2 < 2e-2, "the stack is %.3g / %.3g from the oracle" % (e_full, e_win2)
+            checked["all_rows_periodic_fill_max_abs_err"] = max(e_full, e_win2)
+            checked["rows_checked"] = layers * batch_size * H
+        log("stack outputs checked:", checked)
+    stack.free()
     per_launch_bytes = step_bytes * steps / launches
     per_launch_s = kern_s / launches
     return {
@@ -141,6 +235,7 @@ def run_stack(gpu, steps, warmup, batch_size=16, ctx=131072, layers=24, kv_gap_g
         "kernel_bytes_per_launch": per_launch_bytes,
         "kernel_s_per_launch": per_launch_s,
         "kernel_gbs": per_launch_bytes / per_launch_s / 1e9,
+        "outputs_checked": checked,
     }
 
 
@@ -260,9 +355,10 @@ def run_single_decode(gpu, steps, warmup, ctx=4096, burst=64):
             "note": "8 MB working set stays in the 256 MB Infinity Cache across launches: cache-fed, not HBM-fed"}
 
 
-def run_ragged(gpu, steps, warmup, n_seq=32):
-    """Configuration 3: 32 sequences with lengths U{128..8192}; per sequence one full-causal
-    layer and one 128-window layer; both layers of all sequences in one dispatch each."""
+def ragged_case(gpu, steps, warmup, n_seq):
+    """n_seq sequences with lengths U{128..8192} (seed 3); per sequence one full-causal layer and one
+    128-window layer. Timed as a model runs it (a dispatch per layer: all sequences of the full-causal
+    layer, then all of the window layer) and with every (sequence, layer) in one dispatch."""
     rng = np.random.default_rng(3)
     lens = rng.integers(128, 8193, size=n_seq)
     offs = np.concatenate([[0], np.cumsum(lens)[:-1]])
@@ -273,7 +369,7 @@ def run_ragged(gpu, steps, warmup, n_seq=32):
     for i, b in enumerate((q, k, v)):
         fill(gpu, b, 20 + i)
     bufs = [q, k, v, out, sinks]
-    tables, nbytes = [], 0
+    per_layer, nbytes = [], 0
     for layer, window in enumerate((C.FULL, 128)):
         items = []
         for s in range(n_seq):
@@ -281,11 +377,13 @@ def run_ragged(gpu, steps, warmup, n_seq=32):
             items.append(C.DecodeItem(i * QO, i * QO, int(offs[s]) * ROW, int(offs[s]) * ROW, layer * H * 4,
                                       int(lens[s]) - 1, window, int(lens[s])))
             nbytes += decode_bytes(int(lens[s]), window)
-        tables.append(C.decode_items(items))
+        per_layer.append(items)
+    tables = [C.decode_items(items) for items in per_layer]
+    together = [C.decode_items(per_layer[0] + per_layer[1])]
 
-    def go():
+    def go(tbs):
         batch = gpu.batch(bufs)
-        for tb in tables:
+        for tb in tbs:
             batch.attention_decode_batched(0, 1, 2, 3, 4, tb, H, G, D, SCALE, C.BF16)
         t0 = time.perf_counter()
         done = batch.run()
@@ -293,16 +391,35 @@ def run_ragged(gpu, steps, warmup, n_seq=32):
         batch.drop()
         return done.gpu_time, wall
 
-    for _ in range(max(warmup, 5)):
-        go()
-    runs = sorted(go() for _ in range(max(steps, 20)))
+    res = {}
+    for name, tbs in (("dispatch_per_layer", tables), ("one_dispatch", together)):
+        for _ in range(max(warmup, 5)):
+            go(tbs)
+        runs = sorted(go(tbs) for _ in range(max(steps, 20)))
+        res[name] = runs[len(runs) // 2]
     for b in bufs:
         b.free()
-    g, w = runs[len(runs) // 2]
-    return {"workload": "C3 batched decode: 32 sequences, lengths U{128..8192} (seed 3), full + 128-window layer each",
-            "bytes": nbytes, "gpu_us": g * 1e6, "wall_us": w * 1e6, "gbs": nbytes / g / 1e9,
+    return nbytes, res
+
+
+def run_ragged(gpu, steps, warmup, n_seq=32):
+    """Configuration 3 (32 sequences: 261 MB, which the 256 MB last-level cache partly holds across
+    launches) and the same draw with 128 sequences (1.1 GB: fed from HBM)."""
+    nbytes, res = ragged_case(gpu, steps, warmup, n_seq)
+    g, w = res["dispatch_per_layer"]
+    g1, w1 = res["one_dispatch"]
+    big_bytes, big = ragged_case(gpu, steps, warmup, 4 * n_seq)
+    bg, bw = big["dispatch_per_layer"]
+    return {"workload": "C3 batched decode: %d sequences, lengths U{128..8192} (seed 3), full + 128-window layer each, "
+                        "one dispatch per layer" % n_seq,
+            "bytes": nbytes, "gpu_us": g * 1e6, "wall_us": w * 1e6, "gbs": nbytes / g / 1e9, "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS,
             "tokens_per_s": n_seq / w,
-            "note": "about 280 MB per step: close to the 256 MB Infinity Cache, partly cache-fed"}
+            "both_layers_in_one_dispatch": {"gpu_us": g1 * 1e6, "wall_us": w1 * 1e6, "gbs": nbytes / g1 / 1e9},
+            "hbm_fed_%d_sequences" % (4 * n_seq): {"bytes": big_bytes, "gpu_us": bg * 1e6, "wall_us": bw * 1e6,
+                                                    "gbs": big_bytes / bg / 1e9, "hbm_frac": big_bytes / bg / 1e9 / HBM_PEAK_GBS,
+                                                    "tokens_per_s": 4 * n_seq / bw},
+            "note": "the %d-sequence step is about 280 MB: close to the 256 MB Infinity Cache, partly cache-fed; "
+                    "the %d-sequence one is not" % (n_seq, 4 * n_seq)}
 
 
 def run_prefill(gpu, steps, warmup, t=8192):
@@ -849,7 +966,7 @@ def main():
         extra["c3_ragged_batch"]["cpu_baseline"] = host["c3"]
         for name in ("full", "window128"):
             extra["c4_prefill"][name]["cpu_baseline"] = host["c4"][name]
-    extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "step_bytes", "kernel_launches_per_step")}
+    extra["c5_stack"] = {k: r[k] for k in ("tokens_per_s", "gpu_s_per_step", "step_bytes", "kernel_launches_per_step", "outputs_checked")}
     line = {
         "metric": METRIC, "value": r["value_gbs"], "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": r["wall_s_per_step"] * 1e3, "higher_is_better": True,

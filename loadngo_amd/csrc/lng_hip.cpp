@@ -109,6 +109,7 @@ struct lng_gpu {
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
     std::atomic<long> live_buffers{0};
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
+    uint64_t fuse_wgs = 1024;   // decode dispatches of up to this many workgroups merge their chunks in the kernel
     char *static_scratch = nullptr; // this device's copy of the fixed scratch array (LNG_STATIC_SCRATCH_BYTES)
 
     // completion thread (only for batches committed with a callback)
@@ -429,6 +430,9 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     const uint64_t most = std::min<uint64_t>(LNG_MAX_CHUNKS, std::max<uint64_t>(longest <= 8192 && pairs <= 16 ? 16 : 32, fill));
     chunk = std::max<uint64_t>(chunk, ((longest + most - 1) / most + 127) / 128 * 128);
     chunk = std::max<uint64_t>(chunk, ((longest + LNG_MAX_CHUNKS - 1) / LNG_MAX_CHUNKS + 127) / 128 * 128);
+    // Short runs (a 128-token window seen from its 32-aligned start is up to 159 positions) stay whole: two
+    // chunks would mean partials, arrival counters and a merge for five tiles of work.
+    if (longest <= 512) chunk = std::max<uint64_t>(chunk, (longest + 127) / 128 * 128);
     p.chunk = (uint32_t)chunk;
     p.n_chunks = (uint32_t)((longest + chunk - 1) / chunk);
     return p;
@@ -461,7 +465,7 @@ RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, 
     if (p.chunks.n_chunks > 1) {
         p.partial_slots = p.pairs * (size_t)p.chunks.n_chunks * group;
         // Small grids merge inside the kernel; large ones with a second dispatch (the f32 kernel always).
-        p.fused = fast && (uint64_t)p.chunks.n_chunks * p.pairs <= 4ull * g->cus;
+        p.fused = fast && (uint64_t)p.chunks.n_chunks * p.pairs <= g->fuse_wgs;
     }
     return p;
 }
@@ -478,9 +482,10 @@ struct RowsLaunches {
     } l[2];
 };
 
-// `a` already names its scratch. With a table of rows of unequal length the decode kernel takes a list of
-// its live (pair, chunk) workgroups (`work_host` / `work_dev`, room for every live entry of 8 bytes, or NULL:
-// a rectangle of n_chunks workgroups per pair, those past a row's end returning at once).
+// `a` already names its scratch. With a table of rows of unequal length the decode kernel launches its live
+// workgroups only and finds each one's row in a table of running counts (`work_host` / `work_dev`, room for
+// n_rows + 1 counts of 4 bytes; NULL: a rectangle of n_chunks workgroups per pair, those past a row's end
+// returning at once).
 int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *host_rows, size_t n_rows,
                   uint32_t *work_host, const uint32_t *work_dev, RowsLaunches *out) {
     const uint32_t group = a.heads / a.kv_heads;
@@ -503,15 +508,10 @@ int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *
     if (work_host && a.n_chunks > 1) {
         uint64_t n = 0;
         for (size_t r = 0; r < n_rows; ++r) {
-            const uint64_t live = (visible_from_tile(host_rows[r]) + a.chunk - 1) / a.chunk;
-            for (uint32_t kv = 0; kv < a.kv_heads; ++kv) {
-                for (uint64_t c = 0; c < live; ++c) {
-                    work_host[2 * n] = (uint32_t)(r * a.kv_heads + kv);
-                    work_host[2 * n + 1] = (uint32_t)c;
-                    ++n;
-                }
-            }
+            work_host[r] = (uint32_t)n;
+            n += (visible_from_tile(host_rows[r]) + a.chunk - 1) / a.chunk * a.kv_heads;
         }
+        work_host[n_rows] = (uint32_t)n;
         a.work = work_dev;
         wgs = n;
     }
@@ -534,13 +534,13 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         a.partial_ml = g->scratch_ml;
         a.tickets = g->tickets;
     }
-    // Rows of unequal length (a table of sequences): room for the list of live workgroups.
+    // Rows of unequal length (a table of sequences): room for the running counts of live workgroups.
     char *work_host = nullptr, *work_dev = nullptr;
     if (!t_uniform && p.chunks.n_chunks > 1 && p.kind != RowsPlan::Generic) {
         uint64_t live = 0;
         for (size_t r = 0; r < n_rows; ++r) live += (visible_from_tile(host_rows[r]) + p.chunks.chunk - 1) / p.chunks.chunk;
         if (live < (uint64_t)n_rows * p.chunks.n_chunks && live * a.kv_heads <= 0x7fffffffull) {
-            if (int rc = reserve_table(b, live * a.kv_heads * 8, &work_host, &work_dev)) return rc;
+            if (int rc = reserve_table(b, (n_rows + 1) * 4, &work_host, &work_dev)) return rc;
         }
     }
     RowsLaunches launches;
@@ -788,6 +788,11 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         return code;
     }
     g->static_scratch = (char *)lng_static_scratch(device);
+    g->fuse_wgs = 4ull * g->cus;
+    if (const char *env = getenv("LNG_FUSE_WGS")) {
+        const long n = atol(env);
+        if (n >= 0) g->fuse_wgs = (uint64_t)n;
+    }
     if (const char *env = getenv("LNG_DECODE_WGS")) {
         const long n = atol(env);
         if (n >= 1 && n <= (1 << 20)) g->decode_wgs = (unsigned)n;

@@ -24,8 +24,9 @@ typedef struct lng_k_attn {
     float *partial_o;         /* split-K scratch: [row][kv_head][chunk][group][dim] f32 */
     float *partial_ml;        /* split-K scratch: [row][kv_head][chunk][group][2] f32 (max, sum) */
     uint32_t *tickets;        /* split-K scratch: [row][kv_head] arrival counters, zero between dispatches */
-    const uint32_t *work;     /* device list of (row * kv_heads + kv head, chunk) pairs, one per workgroup of a decode
-                                 kernel, or NULL: workgroup w takes pair w / n_chunks, chunk w % n_chunks */
+    const uint32_t *work;     /* device table cum[n_rows + 1]: cum[r] = decode workgroups of rows before r (each row has
+                                 kv_heads x its own number of chunks), or NULL: workgroup w takes pair w / n_chunks,
+                                 chunk w % n_chunks */
     lng_k_row first;          /* row 0 when rows == NULL; row i: q/out advance by one row, start by i */
     uint32_t n_rows;
     uint32_t heads;
