@@ -57,6 +57,8 @@ const char *hip_text(hipError_t e) { return hipGetErrorString(e); }
 
 size_t elem_size(int dtype) { return dtype == LNG_BF16 ? 2 : 4; }
 
+bool env_is(const char *value, const char *what) { return value && strcmp(value, what) == 0; }
+
 struct Table { // one pinned-host / device pair holding row tables of batched dispatches
     char *host = nullptr;
     char *dev = nullptr;
@@ -89,7 +91,7 @@ struct lng_gpu {
     // kernels of the embedded code object
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr;
-    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
+    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
     hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_one_w8 = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
@@ -636,7 +638,12 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const uint64_t visible = p.window == LNG_WINDOW_FULL ? end : std::min<uint64_t>(end, p.window + rows_per_wg);
         const uint64_t key_tiles = (visible + 63) / 64;
         const uint64_t plain_wgs = (uint64_t)p.q_tiles * s.kv_heads;
-        if ((!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
+        // LNG_PREFILL_STREAM: 0 never takes the kernel of workgroups that walk several query tiles, 1 takes it for
+        // every full-causal pass it can run (tests: small shapes), otherwise only when every compute unit has a tile.
+        const char *stream_env = getenv("LNG_PREFILL_STREAM");
+        const bool stream_can = !f32 && !narrow && p.window == LNG_WINDOW_FULL && s.slots >= end && !env_is(stream_env, "0");
+        const bool stream = stream_can && (plain_wgs >= g->cus || env_is(stream_env, "1"));
+        if (!stream && (!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
             uint64_t want = g->cus / plain_wgs;
             want = std::min<uint64_t>(want, key_tiles / 4);
             want = std::min<uint64_t>(want, 64);
@@ -649,13 +656,19 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             p.partial_o = g->scratch_o;
             p.partial_ml = g->scratch_ml;
         }
+        // The long full-causal pass with every compute unit busy anyway: one workgroup per compute unit that stays
+        // there and walks several query tiles (balanced by construction, no per-workgroup start-up between them).
         Cmd c;
         c.grid[0] = p.q_tiles * (unsigned)s.kv_heads * p.splits; // kv head fastest: one XCD's L2 per kv head
+        c.block = 512;
+        if (stream) {
+            const uint64_t per_head = std::min<uint64_t>(p.q_tiles, std::max<uint64_t>(1, g->cus / s.kv_heads));
+            c.grid[0] = (unsigned)(per_head * s.kv_heads);
+        }
         // f32: two workgroups per compute unit only when there are four rounds of them or more (see the kernels)
         const bool f32_two = f32 && c.grid[0] >= 4u * g->cus;
-        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : narrow ? g->prefill_bf16_d64_h1 : g->prefill_bf16_d64;
-        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : narrow ? "lng_prefill_bf16_d64_h1" : "lng_prefill_bf16_d64";
-        c.block = 512;
+        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : g->prefill_bf16_d64;
+        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : "lng_prefill_bf16_d64";
         set_args(c, p);
         b->cmds.push_back(std::move(c));
         if (p.splits > 1) {
@@ -746,6 +759,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_f32_d64", &g->decode_f32_d64, true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
+        {"lng_prefill_bf16_d64_stream", &g->prefill_bf16_d64_stream, true},
         {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
         {"lng_prefill_f32_d64_w4", &g->prefill_f32_d64_w4, true},
         {"lng_prefill_merge", &g->prefill_merge, true},

@@ -1744,6 +1744,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     bf16x8 qreg[NH][4];
     float m[NH], l[NH];
     floatx16 ot[NH][2];
+    const float sl2 = a.scale * LNG_LOG2E;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
 #pragma unroll
@@ -1752,10 +1753,15 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             if (row_ok) {
                 raw = *(const uint4 *)(a.q + (((uint64_t)my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
             }
-            qreg[h][ks] = as_bf16x8(raw);
+            // scale * log2(e) goes into the query operand, once: the products then come out of the matrix unit
+            // in the exponent's own units (one more bf16 rounding of q: 2^-9 relative per element, a few 1e-4 on
+            // a score, an order below the rounding of the weights to bf16)
+            bf16x8 qv = as_bf16x8(raw);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qv[e] = (__bf16)((float)qv[e] * sl2);
+            qreg[h][ks] = qv;
         }
     }
-    const float sl2 = a.scale * LNG_LOG2E;
     bf16x2 ones2;
     ones2[0] = (__bf16)1.0f;
     ones2[1] = (__bf16)1.0f;
@@ -1815,9 +1821,12 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
 
     // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
     // carries no position arithmetic at all.
-    auto step = [&](auto mask_tag, auto fixed_tag, uint32_t tile) {
+    // MODE 0: the running maximum is tracked. MODE 1: it is fixed (weights = 2^(score - m)). MODE 2: it is
+    // fixed at zero (weights = 2^score: nothing but the exponential, the narrowing and the sum per score).
+    auto step = [&](auto mask_tag, auto mode_tag, uint32_t tile) {
         constexpr bool MASK = decltype(mask_tag)::value;
-        constexpr bool FIXED = decltype(fixed_tag)::value;
+        constexpr int MODE = decltype(mode_tag)::value;
+        constexpr bool FIXED = MODE != 0;
         const uint32_t buf = tile & 1u;
         if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
         if (wave_active) {
@@ -1879,7 +1888,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                         float tmax = LNG_NEG_INF;
 #pragma unroll
                         for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
-                        tmax = other_half_max(tmax) * sl2; // scale > 0: max commutes with it
+                        tmax = other_half_max(tmax);
                         const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
                         m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
                         if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
@@ -1893,23 +1902,23 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                             m[h] = m_new;
                         }
                     }
-                    float psum = 0.0f;
+                    float psum[2] = {0.0f, 0.0f}; // two chains of four dependent sums instead of one of eight
 #pragma unroll
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                         for (int e = 0; e < 8; e += 2) {
-                            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[h][8 * jj + e], sl2, -m_safe));
-                            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(st[h][8 * jj + e + 1], sl2, -m_safe));
+                            const float p0 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e] : st[h][8 * jj + e] - m_safe);
+                            const float p1 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e + 1] : st[h][8 * jj + e + 1] - m_safe);
                             bf16x2 pr;
                             pr[0] = (__bf16)p0;
                             pr[1] = (__bf16)p1;
                             pb[h][jj][e] = pr[0];
                             pb[h][jj][e + 1] = pr[1];
                             // the normaliser sums the same rounded weights the product uses
-                            psum = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum, false);
+                            psum[jj] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum[jj], false);
                         }
                     }
-                    l[h] += psum;
+                    l[h] += psum[0] + psum[1];
                 }
                 // ---- O^T += V^T . P^T ---------------------------------------------------------------------
 #pragma unroll
@@ -1930,21 +1939,49 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         const uint32_t kt0 = tile0 + tile * PF_BN;
         return kt0 + (PF_BN - 1) > pos_first || (windowed && kt0 + window < pos_first + PF_BM);
     };
+    using tracked = std::integral_constant<int, 0>;
+    using fixed_at_m = std::integral_constant<int, 1>;
+    using fixed_at_zero = std::integral_constant<int, 2>;
     uint32_t tile = first_tile;
     bool frozen = false;
-    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, std::false_type{}, tile); // window edge
-    if (optimistic) {                                                                             // interior
+    for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tracked{}, tile); // window edge
+    if (optimistic) {                                                                      // interior
+        bool at_zero = false;
         if (tile < n_tiles && !edge(tile)) {
-            step(std::false_type{}, std::false_type{}, tile); // sets the maximum from real scores
+            step(std::false_type{}, tracked{}, tile); // sets the maximum from real scores
             ++tile;
             frozen = true;
+            // Maxima of moderate size (|m| <= 40 in the exponent's units, for every query of the wavefront): move
+            // the reference point to zero once, and the loop below has no subtraction left either.
+            bool moderate = true;
 #pragma unroll
-            for (int h = 0; h < NH; ++h) m[h] = m[h] == LNG_NEG_INF ? 0.0f : m[h];
+            for (int h = 0; h < NH; ++h) {
+                m[h] = m[h] == LNG_NEG_INF ? 0.0f : m[h];
+                moderate = moderate && __builtin_fabsf(m[h]) <= 40.0f;
+            }
+            at_zero = __builtin_amdgcn_ballot_w64(!moderate) == 0;
+            if (at_zero) {
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    const float up = __builtin_amdgcn_exp2f(m[h]);
+                    l[h] *= up;
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) ot[h][db][i] *= up;
+                    }
+                    m[h] = 0.0f;
+                }
+            }
         }
-        // a loop of its own: one path through it, so its registers need no reconciling copies
-        for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, std::true_type{}, tile);
+        // loops of their own: one path through each, so their registers need no reconciling copies
+        if (at_zero) {
+            for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, fixed_at_zero{}, tile);
+        } else {
+            for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, fixed_at_m{}, tile);
+        }
     } else {
-        for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, std::false_type{}, tile);
+        for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tracked{}, tile);
     }
     bool again = false;
     if (NH == 2 && frozen) { // frozen is uniform over the workgroup
@@ -1959,16 +1996,16 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
 #pragma unroll
                     for (int i = 0; i < 16; ++i) top = max(top, __float_as_uint(ot[h][db][i]) & 0x7fffffffu);
                 }
-                // 2^-80 .. 2^60: terms lost below 2^-126 are then under 2^-29 of the total even for 2^17
+                // 2^-90 .. 2^100: terms lost below 2^-126 are then under 2^-19 of the total even for 2^17
                 // keys, and nothing overflowed (a NaN fails the comparison)
-                bad |= !(total >= 8.271806e-25f && total <= 1.1529215e18f) || top >= 0x7f800000u;
+                bad |= !(total >= 8.0779357e-28f && total <= 1.2676506e30f) || top >= 0x7f800000u;
             }
             bad = row_ok ? bad : 0;
         }
         again = __syncthreads_or(bad) != 0;
     }
     if (!again) {
-        for (; tile < n_tiles; ++tile) step(std::true_type{}, std::false_type{}, tile);           // diagonal
+        for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile);                    // diagonal
         break;
     }
     }
@@ -2027,6 +2064,503 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
 
 extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1(lng_k_prefill a) {
     prefill_body<1>(a);
+}
+
+// =============================================================================================
+// The long full-causal prompt pass (no window, no ring, keys not split): lng_prefill_bf16_d64's
+// arithmetic, tile for tile, in a workgroup that STAYS on its compute unit and walks several
+// query tiles.
+//
+// Why: with one workgroup per (query tile, kv head) a compute unit runs about four workgroups one
+// after the other on an 8192-position pass, and each pays about 20 us that no other work hides (it is
+// alone on its unit): the dispatch gap, a round trip for its queries and another for its first K/V
+// tile, the one-off tiles, the scattered stores - a tenth of the pass - and the units finish up to
+// 60 us apart. Here the grid is one workgroup per compute unit (kv head = id % kv_heads, so the ids
+// of one kv head share an XCD and its L2), and workgroup c of the C that share a kv head takes query
+// tiles c, 2C-1-c, 2C+c, 4C-1-c, ... counted from the longest: every unit gets the same number of key
+// tiles to within one per round. Queries and the first two K/V tiles of a query tile arrive in one
+// round trip.
+//
+// K/V tiles go through THREE LDS buffers: tile i + 2 is fetched into registers during tile i and
+// stored at its end, so when a tile starts, the next one is already visible, and the K operands of
+// the next tile's first block are read before the barrier, under the last products of this one
+// (with two buffers every tile began by waiting for its first LDS reads with the matrix unit idle).
+// =============================================================================================
+// (Measured and not kept: two four-wavefront workgroups of 32 rows per compute unit, which share no barrier:
+// 565 us against 521 us; tiles of 128 keys per barrier: 546 us.)
+extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_stream(lng_k_prefill a) {
+    constexpr int NH = 2;
+    constexpr int QB = 2;                    // blocks of 32 query rows per workgroup
+    constexpr uint32_t PF_BM = 32u * QB;
+    constexpr int KB = 2;                    // blocks of 32 keys per tile, i.e. per barrier
+    constexpr uint32_t SBN = 32u * KB;       // keys per tile
+    constexpr int LD = (int)SBN / (32 * QB); // keys of a tile each thread loads
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[3][SBN * PF_KSTRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[3][SBN * PF_VSTRIDE];
+
+    const uint32_t g = blockIdx.x % a.kv_heads;
+    const uint32_t c = blockIdx.x / a.kv_heads;   // this workgroup among the C of its kv head
+    const uint32_t C = gridDim.x / a.kv_heads;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n = lane & 31u;
+    const uint32_t hh = lane >> 5;
+    const uint32_t qb = QB == 2 ? (wave & 1u) : 0u;
+    const uint32_t hp = QB == 2 ? (wave >> 1) : wave;
+    const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
+
+    const bool wave_active = hp * NH < group;
+    const bool second_ok = hp * 2u + 1u < group;
+    uint32_t head[NH];
+    head[0] = g * group + (wave_active ? hp * NH : 0u);
+    head[1] = second_ok ? head[0] + 1u : head[0];
+    const float sl2 = a.scale * LNG_LOG2E;
+    bf16x2 ones2;
+    ones2[0] = (__bf16)1.0f;
+    ones2[1] = (__bf16)1.0f;
+
+    const uint32_t ld_key = tid >> 3; // a thread's further keys are 32 * QB apart
+    const uint32_t ld_chunk = tid & 7u;
+    const char *kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
+    const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
+    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;
+    const uint32_t L = lane & 15u;
+    const uint32_t blk16 = lane >> 4;
+    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+
+    using tracked = std::integral_constant<int, 0>;
+    using fixed_at_m = std::integral_constant<int, 1>;
+    using fixed_at_zero = std::integral_constant<int, 2>;
+
+    for (uint32_t round = 0;; ++round) {
+        const uint32_t idx = round * C + ((round & 1u) ? C - 1u - c : c);
+        if (idx >= a.q_tiles) break; // idx grows with the round for every c: nothing later either
+        const uint32_t qtile = a.q_tiles - 1u - idx;
+        const uint32_t q0 = qtile * PF_BM;
+        const uint32_t rows_here = t - q0 < PF_BM ? t - q0 : PF_BM;
+        const uint32_t pos_first = start + q0;
+        const uint32_t pos_last = pos_first + rows_here - 1;
+        const uint32_t n_tiles = pos_last / SBN + 1;
+        const uint32_t n_interior = (pos_first + 1u) / SBN; // tiles whose every key every query of the tile sees
+        const uint32_t my_row = q0 + 32u * qb + n;
+        const uint32_t my_pos = start + my_row;
+        const bool row_ok = my_row < t;
+
+        auto fetch = [&](uint32_t tile, uint4 (&kr)[LD], uint4 (&vr)[LD]) {
+#pragma unroll
+            for (int u = 0; u < LD; ++u) {
+                uint32_t p = tile * SBN + ld_key + (32u * QB) * u;
+                p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway
+                kr[u] = *(const uint4 *)(kbase + (uint64_t)p * row_bytes);
+                vr[u] = *(const uint4 *)(vbase + (uint64_t)p * row_bytes);
+            }
+        };
+        auto stash = [&](uint32_t buf, const uint4 (&kr)[LD], const uint4 (&vr)[LD]) {
+#pragma unroll
+            for (int u = 0; u < LD; ++u) {
+                *(uint4 *)(&s_k[buf][(ld_key + (32u * QB) * u) * PF_KSTRIDE + ld_chunk * 8u]) = kr[u];
+                *(uint4 *)(&s_v[buf][(ld_key + (32u * QB) * u) * PF_VSTRIDE + ld_chunk * 8u]) = vr[u];
+            }
+        };
+        auto read_k = [&](uint32_t buf, int kb, bf16x8 (&ka)[4]) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
+            }
+        };
+
+        // ---- queries (scaled once, see lng_prefill_bf16_d64) and the first two tiles: one round trip ----
+        bf16x8 qreg[NH][4];
+        {
+            uint4 raw[NH][4];
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    raw[h][ks] = make_uint4(0, 0, 0, 0);
+                    if (row_ok) {
+                        raw[h][ks] = *(const uint4 *)(a.q + (((uint64_t)my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
+                    }
+                }
+            }
+            uint4 k0[LD], v0[LD], k1[LD], v1[LD];
+            fetch(0, k0, v0);
+            fetch(n_tiles > 1u ? 1u : 0u, k1, v1);
+            stash(0, k0, v0);
+            stash(1, k1, v1);
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    bf16x8 qv = as_bf16x8(raw[h][ks]);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) qv[e] = (__bf16)((float)qv[e] * sl2);
+                    qreg[h][ks] = qv;
+                }
+            }
+        }
+        __syncthreads();
+
+        float m[NH], l[NH];
+        floatx16 ot[NH][2];
+        uint4 kr[LD], vr[LD];
+        bf16x8 ka0[4];       // K operands of the coming tile's first block of 32 keys
+        uint32_t buf = 0;    // LDS buffer of the coming tile; tile + 1 is in buf + 1, tile + 2 goes to buf + 2 (mod 3)
+
+        auto step = [&](auto mask_tag, auto mode_tag, uint32_t tile) {
+            constexpr bool MASK = decltype(mask_tag)::value;
+            constexpr int MODE = decltype(mode_tag)::value;
+            constexpr bool FIXED = MODE != 0;
+            const uint32_t nxt = buf == 2u ? 0u : buf + 1u;
+            const uint32_t after = nxt == 2u ? 0u : nxt + 1u;
+            fetch(tile + 2, kr, vr); // (past the last tile: its rows again, stored where nobody reads them)
+            if (wave_active) {
+                const uint32_t kt0 = tile * SBN;
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    if constexpr (MASK) { // a block of keys past the last row of the tile: nobody sees it
+                        if (kt0 + 32u * kb > pos_last) continue;
+                    }
+                    bf16x8 ka[4];
+                    if (kb == 0) {
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) ka[ks] = ka0[ks];
+                    } else {
+                        read_k(buf, kb, ka);
+                    }
+                    floatx16 st[NH];
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) st[h][i] = 0.0f;
+                    }
+#pragma unroll
+                    for (int ks = 0; ks < 4; ++ks) {
+                        st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[0][ks], st[0], 0, 0, 0);
+                        st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[1][ks], st[1], 0, 0, 0);
+                    }
+                    bf16x8 va[2][2];
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                        for (int db = 0; db < 2; ++db) {
+                            const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                            va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                        }
+                    }
+                    // the next tile's first operands, under this block's arithmetic and products (after the last
+                    // tile this reads a buffer that nobody uses: no branch in the middle of the tile)
+                    if (kb == KB - 1) read_k(nxt, 0, ka0);
+                    bf16x8 pb[NH][2];
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+                        if constexpr (MASK) {
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                const uint32_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
+                                st[h][i] = kp <= my_pos ? st[h][i] : LNG_NEG_INF;
+                            }
+                        }
+                        float m_safe;
+                        if constexpr (FIXED) {
+                            m_safe = m[h];
+                        } else {
+                            float tmax = LNG_NEG_INF;
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
+                            tmax = other_half_max(tmax);
+                            const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
+                            m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                            if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
+                                const float alpha = __builtin_amdgcn_exp2f(m[h] - m_safe);
+                                l[h] *= alpha;
+#pragma unroll
+                                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                                    for (int i = 0; i < 16; ++i) ot[h][db][i] *= alpha;
+                                }
+                                m[h] = m_new;
+                            }
+                        }
+                        float psum[2] = {0.0f, 0.0f};
+#pragma unroll
+                        for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                            for (int e = 0; e < 8; e += 2) {
+                                const float p0 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e] : st[h][8 * jj + e] - m_safe);
+                                const float p1 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e + 1] : st[h][8 * jj + e + 1] - m_safe);
+                                bf16x2 pr;
+                                pr[0] = (__bf16)p0;
+                                pr[1] = (__bf16)p1;
+                                pb[h][jj][e] = pr[0];
+                                pb[h][jj][e + 1] = pr[1];
+                                psum[jj] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum[jj], false);
+                            }
+                        }
+                        l[h] += psum[0] + psum[1];
+                    }
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                        for (int db = 0; db < 2; ++db) {
+                            ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[0][jj], ot[0][db], 0, 0, 0);
+                            ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            stash(after, kr, vr);
+            __syncthreads();
+            buf = nxt;
+        };
+
+        // ---- the interior tiles with the maximum fixed at zero, as a software pipeline ----------------------
+        // Unit = (block of 32 keys, one head): four matrix instructions of scores, 32 arithmetic instructions
+        // (16 exponentials, 8 narrowings, 8 sums), four matrix instructions of values. While a unit's arithmetic
+        // issues, the matrix unit runs the NEXT unit's scores and the PREVIOUS unit's values, one matrix
+        // instruction in front of every four arithmetic ones, so neither pipe waits for the other inside a
+        // wavefront (the plain tile issues eight score products back to back, waits for them, and only then
+        // starts on the exponentials). The next tile is visible one tile early (three buffers), so the pipeline
+        // runs across the tile barrier: the scores of the next tile's first unit are under way before it.
+        auto pipe = [&](uint32_t &tile) {
+            floatx16 st_cur;          // scores of the coming unit (first block of keys, first head)
+            bf16x8 pb_prev[2];        // weights of the last finished unit, their value product pending
+            bf16x8 va_prev[2][2];     // and its V^T operands
+            auto zero16 = [&]() {
+                floatx16 z;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) z[i] = 0.0f;
+                return z;
+            };
+            // one unit: `sc` -> weights `pw` (and the running sum), with score products (kq . qq -> so) and value
+            // products (vz . pz -> oz) of its neighbours in between
+            auto unit = [&](floatx16 &sc, float &lsum, const bf16x8 (&kq)[4], const bf16x8 (&qq)[4], floatx16 &so,
+                            const bf16x8 (&vz)[2][2], const bf16x8 (&pz)[2], floatx16 (&oz)[2], bf16x8 (&pw)[2]) {
+                float ps0 = 0.0f, ps1 = 0.0f;
+                bf16x2 pr[8];
+                __builtin_amdgcn_sched_barrier(0);
+                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[0], qq[0], zero16(), 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
+                __builtin_amdgcn_sched_barrier(0);
+                oz[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[0][0], pz[0], oz[0], 0, 0, 0);
+#pragma unroll
+                for (int i = 4; i < 8; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
+                __builtin_amdgcn_sched_barrier(0);
+                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[1], qq[1], so, 0, 0, 0);
+#pragma unroll
+                for (int i = 8; i < 12; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
+                __builtin_amdgcn_sched_barrier(0);
+                oz[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[0][1], pz[0], oz[1], 0, 0, 0);
+#pragma unroll
+                for (int i = 12; i < 16; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
+                __builtin_amdgcn_sched_barrier(0);
+                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[2], qq[2], so, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pr[e][0] = (__bf16)sc[2 * e];
+                    pr[e][1] = (__bf16)sc[2 * e + 1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                oz[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[1][0], pz[1], oz[0], 0, 0, 0);
+#pragma unroll
+                for (int e = 4; e < 8; ++e) {
+                    pr[e][0] = (__bf16)sc[2 * e];
+                    pr[e][1] = (__bf16)sc[2 * e + 1];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[3], qq[3], so, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) ps0 = __builtin_amdgcn_fdot2_f32_bf16(pr[e], ones2, ps0, false);
+                __builtin_amdgcn_sched_barrier(0);
+                oz[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[1][1], pz[1], oz[1], 0, 0, 0);
+#pragma unroll
+                for (int e = 4; e < 8; ++e) ps1 = __builtin_amdgcn_fdot2_f32_bf16(pr[e], ones2, ps1, false);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    pw[0][2 * e] = pr[e][0];
+                    pw[0][2 * e + 1] = pr[e][1];
+                    pw[1][2 * e] = pr[4 + e][0];
+                    pw[1][2 * e + 1] = pr[4 + e][1];
+                }
+                lsum += ps0 + ps1;
+            };
+            auto read_v = [&](uint32_t b, int kb, bf16x8 (&va)[2][2]) {
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+                        const uint16_t *vp = &s_v[b][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                        va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                    }
+                }
+            };
+            if (wave_active) {
+                // nothing pending yet: weights of zero against any finite operands
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pb_prev[jj][e] = (__bf16)0.0f;
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) va_prev[jj][db] = pb_prev[jj];
+                }
+                st_cur = zero16();
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) st_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[ks], qreg[0][ks], st_cur, 0, 0, 0);
+            }
+            for (; tile < n_interior; ++tile) {
+                const uint32_t nxt = buf == 2u ? 0u : buf + 1u;
+                const uint32_t after = nxt == 2u ? 0u : nxt + 1u;
+                fetch(tile + 2, kr, vr);
+                if (wave_active) {
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb) {
+                        bf16x8 kan[4], va[2][2], pbA[2];
+                        floatx16 stB;
+                        if (kb + 1 < KB) {
+                            read_k(buf, kb + 1, kan);
+                        } else {
+                            read_k(nxt, 0, kan);
+                        }
+                        read_v(buf, kb, va);
+                        unit(st_cur, l[0], ka0, qreg[1], stB, va_prev, pb_prev, ot[1], pbA);  // (block kb, head 0)
+                        unit(stB, l[1], kan, qreg[0], st_cur, va, pbA, ot[0], pb_prev);        // (block kb, head 1)
+#pragma unroll
+                        for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                            for (int db = 0; db < 2; ++db) va_prev[jj][db] = va[jj][db];
+                        }
+#pragma unroll
+                        for (int ks = 0; ks < 4; ++ks) ka0[ks] = kan[ks];
+                    }
+                }
+                stash(after, kr, vr);
+                __syncthreads();
+                buf = nxt;
+            }
+            if (wave_active) { // the last unit's values; the scores under way belong to the tile that follows
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va_prev[jj][db], pb_prev[jj], ot[1][db], 0, 0, 0);
+                    }
+                }
+            }
+        };
+
+        for (int attempt = 0; attempt < 2; ++attempt) {
+            const bool optimistic = attempt == 0;
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+                l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
+                }
+            }
+            if (attempt != 0) { // the tiles again from the first: the buffers hold later ones by now
+                uint4 k0[LD], v0[LD], k1[LD], v1[LD];
+                fetch(0, k0, v0);
+                fetch(n_tiles > 1u ? 1u : 0u, k1, v1);
+                stash(0, k0, v0);
+                stash(1, k1, v1);
+                __syncthreads();
+            }
+            buf = 0;
+            if (wave_active) read_k(0, 0, ka0);
+            uint32_t tile = 0;
+            bool frozen = false;
+            if (optimistic) {
+                bool at_zero = false;
+                if (n_interior > 0u) {
+                    step(std::false_type{}, tracked{}, tile); // sets the maximum from real scores
+                    ++tile;
+                    frozen = true;
+                    bool moderate = true;
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+                        m[h] = m[h] == LNG_NEG_INF ? 0.0f : m[h];
+                        moderate = moderate && __builtin_fabsf(m[h]) <= 40.0f;
+                    }
+                    at_zero = __builtin_amdgcn_ballot_w64(!moderate) == 0;
+                    if (at_zero) {
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) {
+                            const float up = __builtin_amdgcn_exp2f(m[h]);
+                            l[h] *= up;
+#pragma unroll
+                            for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                                for (int i = 0; i < 16; ++i) ot[h][db][i] *= up;
+                            }
+                            m[h] = 0.0f;
+                        }
+                    }
+                }
+                if (at_zero) {
+                    pipe(tile);
+                } else {
+                    for (; tile < n_interior; ++tile) step(std::false_type{}, fixed_at_m{}, tile);
+                }
+            } else {
+                for (; tile < n_interior; ++tile) step(std::false_type{}, tracked{}, tile);
+            }
+            bool again = false;
+            if (frozen) { // uniform over the workgroup
+                int bad = 0;
+                if (wave_active) {
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) {
+                        const float total = l[h] + __shfl_xor(l[h], 32, 64);
+                        uint32_t top = 0;
+#pragma unroll
+                        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) top = max(top, __float_as_uint(ot[h][db][i]) & 0x7fffffffu);
+                        }
+                        bad |= !(total >= 8.0779357e-28f && total <= 1.2676506e30f) || top >= 0x7f800000u;
+                    }
+                    bad = row_ok ? bad : 0;
+                }
+                again = __syncthreads_or(bad) != 0;
+            }
+            if (!again) {
+                for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile); // the diagonal
+                break;
+            }
+        }
+
+        // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query ------------------
+        if (wave_active && row_ok) {
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                if (h == 1 && !second_ok) continue;
+                const float total = l[h] + __shfl_xor(l[h], 32, 64);
+                const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+                uint16_t *op = (uint16_t *)a.out + ((uint64_t)my_row * a.heads + head[h]) * 64u;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int blk = 0; blk < 4; ++blk) {
+                        ushort4 w;
+                        w.x = f32_to_bf16_bits(ot[h][db][4 * blk + 0] * inv);
+                        w.y = f32_to_bf16_bits(ot[h][db][4 * blk + 1] * inv);
+                        w.z = f32_to_bf16_bits(ot[h][db][4 * blk + 2] * inv);
+                        w.w = f32_to_bf16_bits(ot[h][db][4 * blk + 3] * inv);
+                        *(ushort4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
+                    }
+                }
+            }
+        }
+        // (the last step of this query tile ended with a barrier: every wavefront is done with the buffers)
+    }
 }
 
 // =============================================================================================
