@@ -2118,6 +2118,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
     head[0] = g * group + (wave_active ? hp * NH : 0u);
     head[1] = second_ok ? head[0] + 1u : head[0];
     const float sl2 = a.scale * LNG_LOG2E;
+    float sink2[NH]; // read once, not per query tile
+#pragma unroll
+    for (int h = 0; h < NH; ++h) sink2[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
     bf16x2 ones2;
     ones2[0] = (__bf16)1.0f;
     ones2[1] = (__bf16)1.0f;
@@ -2457,7 +2460,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
             const bool optimistic = attempt == 0;
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
-                m[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+                m[h] = sink2[h];
                 l[h] = (a.sinks && hh == 0) ? 1.0f : 0.0f;
 #pragma unroll
                 for (int db = 0; db < 2; ++db) {
