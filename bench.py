@@ -38,9 +38,35 @@ QO = H * D * 2           # bytes of one query (or output) row
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X f32 matrix
-# HBM bytes per launch of the decode kernel on the default stack workload, from rocprofv3 FETCH_SIZE
-# and WRITE_SIZE scaled by a 1 GiB copy (profiles/decode_stack_c5_hbm_traffic.md).
-STACK_TRAFFIC_PER_LAUNCH = 2155619789
+# HBM bytes per launch of the decode kernel on the default stack workload come from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE runs scaled by a 1 GiB copy; the figure and the sources it was measured on are kept in
+# profiles/decode_stack_c5_hbm_traffic.json and only reported while those sources are unchanged.
+TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "decode_stack_c5_hbm_traffic.json")
+TRAFFIC_SOURCES = ("loadngo_amd/csrc/lng_kernels.hip", "loadngo_amd/csrc/lng_hip.cpp", "loadngo_amd/csrc/lng_kernel_args.h")
+
+
+def sources_digest():
+    """sha256 over the kernel and planner sources the traffic measurement depends on."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in TRAFFIC_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def stack_traffic_per_launch(ctx, batch):
+    """The measured HBM bytes per launch, or None when the record is missing, for another workload, or stale."""
+    try:
+        with open(TRAFFIC_RECORD) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if (rec.get("ctx"), rec.get("batch")) != (ctx, batch) or rec.get("sources_sha256") != sources_digest():
+        return None
+    return rec.get("hbm_bytes_per_launch")
+
+
 METRIC = "decode attn GB/s (% HBM peak) + prefill attn TFLOP/s (% MFMA), gpt-oss shapes"
 
 
@@ -684,7 +710,7 @@ def cpu_extras():
     all cores (OpenMP over query rows and heads) and on one thread. Configuration 4 is timed on 64
     query rows spread over the pass and scaled by the ratio of query-key pairs (stated as extrapolated)."""
     from oracle import oracle
-    cores = min(16, os.cpu_count() or 1)
+    cores = oracle_threads()
     rng = np.random.default_rng(21)
 
     def timed(fn):
@@ -887,6 +913,20 @@ def run_prepare(gpu, steps, warmup):
     return out
 
 
+def oracle_threads():
+    """Threads the oracle is timed on: the cores this process may use (its affinity mask, and OMP_NUM_THREADS when
+    the environment sets it: the GPU boxes grant a one-GPU job 16 of the host's cores), never more than the host has."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, len(os.sched_getaffinity(0)))
+    except (AttributeError, OSError):
+        pass
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    if env.isdigit() and int(env) > 0:
+        n = min(n, int(env))
+    return n
+
+
 def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
     """The oracle (port of the reference's CPU attention, f32 on widened bf16 inputs) on a
     bounded sample of the headline workload: one sequence, one full-causal and one 128-window
@@ -897,7 +937,7 @@ def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
     k = bf16_widen(bf16_bits(rng.standard_normal((ctx, G, D), dtype=np.float32) * 0.5))
     v = bf16_widen(bf16_bits(rng.standard_normal((ctx, G, D), dtype=np.float32) * 0.5))
     sinks = rng.standard_normal(H).astype(np.float32)
-    cores = min(16, os.cpu_count() or 1)
+    cores = oracle_threads()
     nbytes = decode_bytes(ctx, C.FULL) + decode_bytes(ctx, 128)
     out = {}
     for label, threads in (("all", cores), ("one", 1)):
@@ -908,7 +948,7 @@ def cpu_baseline(step_bytes_per_seq_pair, ctx=131072):
             oracle.attention_f32(q, k, v, sinks, ctx - 1, window=128, scale=SCALE, threads=threads)
             times.append(time.perf_counter() - t0)
         out[label] = sorted(times)[1]
-    return {"value": nbytes / out["all"] / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+    return {"value": nbytes / out["all"] / 1e9, "unit": "GB/s", "cores": cores, "host_cpu_count": os.cpu_count(), "kind": "port",
             "sample": "1 sequence x (1 full-causal + 1 window-128 layer) at context %d, %.0f MB of bf16 KV; "
                       "the 16 x 12 such pairs of a step scale linearly; median of 3 runs" % (ctx, nbytes / 1e6),
             "seconds": out["all"], "value_1thread": nbytes / out["one"] / 1e9, "seconds_1thread": out["one"],
@@ -977,7 +1017,7 @@ def main():
                    "hbm_frac_of_value": r["value_gbs"] / HBM_PEAK_GBS},
         "roofline": {"bound": "hbm", "kernel": r["kernel"], "achieved": r["kernel_gbs"], "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": r["kernel_gbs"] / HBM_PEAK_GBS,
-                     "traffic": STACK_TRAFFIC_PER_LAUNCH if (args.ctx, args.batch) == (131072, 16) else None,
+                     "traffic": stack_traffic_per_launch(args.ctx, args.batch),
                      "bytes_per_launch": r["kernel_bytes_per_launch"], "s_per_launch": r["kernel_s_per_launch"]},
         "cpu_baseline": cpu,
         "extra": extra,

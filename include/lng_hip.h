@@ -88,7 +88,10 @@ const char *lng_hip_last_error(void);
 /* apple.rs:105 Gpu::new — opens HIP device `device`, loads the gfx950 code object embedded
  * in the library and resolves every kernel. LNG_ERR_NO_DEVICE / LNG_ERR_COMPILE. */
 int lng_hip_open(int device, lng_gpu **gpu);
-/* Drop of Gpu. Waits for submitted batches; buffers must have been freed before. */
+/* Drop of Gpu. Waits for submitted batches. Buffers, residents and batches that are still alive keep working
+ * for lng_hip_buffer_free / lng_hip_batch_drop (the reference's buffers share their device the same way); the
+ * device's resources go when the last of them has gone. Recording or committing after close is an error of
+ * the caller. */
 void lng_hip_close(lng_gpu *gpu);
 /* Device name (e.g. "gfx950..."), copied into `name` (NUL-terminated, truncated to `cap`). */
 int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
@@ -116,8 +119,11 @@ int lng_hip_fill(lng_buffer *buffer, size_t offset, int byte, size_t len);
 
 /* ---- batches -------------------------------------------------------------------------- */
 
-/* apple.rs:365 Gpu::batch(buffers, Dispatch::Serial) — starts recording a batch that owns
- * `buffers` until it completes or is dropped; dispatches name them by position. */
+/* apple.rs:365 Gpu::batch(buffers, dispatch) — starts recording a batch that owns `buffers` until it completes
+ * or is dropped; dispatches name them by position. Both of the reference's modes (apple.rs:67-70
+ * Dispatch::Serial / Dispatch::Concurrent, the latter ordered by explicit barrier() calls) record the same
+ * thing here: dispatches run in the order recorded, which is a valid execution of either mode, so there is
+ * no mode argument and lng_hip_batch_barrier has nothing to add. */
 int lng_hip_batch(lng_gpu *gpu, lng_buffer *const *buffers, size_t n_buffers, lng_batch **batch);
 /* apple.rs:835 Batch::attach(&resident) -> Slice covering the whole resident. */
 int lng_hip_batch_attach(lng_batch *batch, lng_buffer *resident, lng_slice *whole);

@@ -109,7 +109,8 @@ struct lng_gpu {
     char *scratch_x = nullptr;   // bf16 planes of the positions of a Q8_0 product
     size_t scratch_x_len = 0;
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
-    std::atomic<long> live_buffers{0};
+    std::atomic<long> live_buffers{0}; // buffers, residents and batches that still name this gpu
+    std::atomic<bool> closed{false};   // lng_hip_close was called while some were alive: the last one to go frees the gpu
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
     uint64_t fuse_wgs = 1024;   // decode dispatches of up to this many workgroups merge their chunks in the kernel
     char *static_scratch = nullptr; // this device's copy of the fixed scratch array (LNG_STATIC_SCRATCH_BYTES)
@@ -351,11 +352,15 @@ void finish(lng_batch *b) {
     release(b);
 }
 
+void object_gone(lng_gpu *g);
+
 void destroy(lng_batch *b) {
     if (b->ev0) hipEventDestroy(b->ev0);
     if (b->ev1) hipEventDestroy(b->ev1);
     for (hipEvent_t mark : b->marks) hipEventDestroy(mark);
+    lng_gpu *g = b->gpu;
     delete b;
+    object_gone(g);
 }
 
 void worker_loop(lng_gpu *g) {
@@ -815,18 +820,9 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
     return LNG_OK;
 }
 
-extern "C" void lng_hip_close(lng_gpu *g) {
-    if (!g) return;
+namespace {
+void destroy_gpu(lng_gpu *g) {
     hipSetDevice(g->device);
-    if (g->worker.joinable()) {
-        {
-            std::lock_guard<std::mutex> lock(g->qmu);
-            g->stopping = true;
-        }
-        g->qcv.notify_all();
-        g->worker.join();
-    }
-    hipStreamSynchronize(g->stream);
     for (Table &t : g->free_tables) {
         hipHostFree(t.host);
         hipFree(t.dev);
@@ -839,6 +835,31 @@ extern "C" void lng_hip_close(lng_gpu *g) {
     hipStreamDestroy(g->stream);
     hipModuleUnload(g->module);
     delete g;
+}
+
+// A buffer or batch of `g` went away: the last one after lng_hip_close takes the gpu with it.
+void object_gone(lng_gpu *g) {
+    if (g->live_buffers.fetch_sub(1) == 1 && g->closed.load()) destroy_gpu(g);
+}
+} // namespace
+
+extern "C" void lng_hip_close(lng_gpu *g) {
+    if (!g) return;
+    hipSetDevice(g->device);
+    if (g->worker.joinable()) {
+        {
+            std::lock_guard<std::mutex> lock(g->qmu);
+            g->stopping = true;
+        }
+        g->qcv.notify_all();
+        g->worker.join();
+    }
+    hipStreamSynchronize(g->stream);
+    // Buffers, residents and batches keep the gpu alive, as the reference's own do (they borrow or share it): with
+    // some still around, the handle stays valid for freeing and dropping them and goes with the last of them.
+    g->live_buffers.fetch_add(1);
+    g->closed.store(true);
+    object_gone(g);
 }
 
 extern "C" int lng_hip_device_name(lng_gpu *g, char *name, size_t cap) {
@@ -883,8 +904,9 @@ extern "C" int lng_hip_buffer_free(lng_buffer *b) {
     if (b->holds.load() != 0) return fail(LNG_ERR_DISPATCH, "the buffer belongs to a batch that has not finished");
     hipSetDevice(b->gpu->device);
     hipFree(b->ptr);
-    b->gpu->live_buffers.fetch_sub(1);
+    lng_gpu *g = b->gpu;
     delete b;
+    object_gone(g);
     return LNG_OK;
 }
 
@@ -946,6 +968,7 @@ extern "C" int lng_hip_batch(lng_gpu *g, lng_buffer *const *buffers, size_t n, l
     lng_batch *b = new lng_batch;
     b->gpu = g;
     b->buffers.assign(buffers, buffers + n);
+    g->live_buffers.fetch_add(1);
     *out = b;
     return LNG_OK;
 }

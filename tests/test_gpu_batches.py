@@ -91,3 +91,82 @@ def test_batches_recorded_and_committed_on_several_threads_at_once(gpu):
     for t in threads:
         t.join(120)
     assert not errors, errors
+
+
+def test_a_dispatch_of_more_rows_than_one_grid_dimension_holds(gpu):
+    """9,000 sequences of 8 kv heads are 72,000 (row, kv head) pairs, past the 65,535 workgroups one grid dimension
+    holds: the dispatch is one-dimensional, so it is accepted and every row comes out right (the reference accepts
+    any rows x heads that fit u32, apple.rs:1257-1272). Rows of unequal length: the list of live workgroups
+    is found through the table of running counts over 9,001 entries (three levels of the 64-way search)."""
+    n, ctx = 9000, 20000
+    rng = np.random.default_rng(77)
+    k = to_bf16_bits((rng.standard_normal((ctx, G, D)) * 0.5).astype(np.float32))
+    v = to_bf16_bits((rng.standard_normal((ctx, G, D)) * 0.5).astype(np.float32))
+    q = to_bf16_bits((rng.standard_normal((n, H, D)) * 0.5).astype(np.float32))
+    sinks = rng.standard_normal(H).astype(np.float32)
+    lens = rng.integers(1, 701, size=n)
+    lens[[17, 4000, 4001, 8999]] = [ctx, ctx - 1, 13000, 6500]  # a few long rows: these are cut into chunks, the rest are not
+    bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.buffer(q.nbytes), gpu.upload(sinks)]
+    bufs[3].fill(0xFF)
+    items = [C.DecodeItem(i * H * D * 2, i * H * D * 2, 0, 0, 0, int(lens[i]) - 1, C.FULL, int(lens[i])) for i in range(n)]
+    batch = gpu.batch(bufs)
+    batch.attention_decode_batched(0, 1, 2, 3, 4, items, H, G, D, 0.125, C.BF16)
+    done = batch.run()
+    assert not isinstance(done.gpu_time, Exception)
+    got = from_bf16_bits(bufs[3].read(np.uint16).reshape(q.shape))
+    batch.drop()
+    for b in bufs:
+        b.free()
+    assert not np.isnan(got).any()
+    for i in list(rng.integers(0, n, 60)) + [0, n - 1, 17, 4000, 4001, 4002, 8999, 8998, int(np.argmin(lens))]:
+        want = orc.attention_bf16(q[i:i + 1], k[:lens[i]], v[:lens[i]], sinks, int(lens[i]) - 1, scale=0.125)
+        assert np.abs(got[i] - from_bf16_bits(want[0])).max() < 2e-2, (i, lens[i])
+
+
+def test_many_small_decodes_merged_inside_the_kernel(gpu):
+    """The split-K merge inside the decode kernel (small grids: the workgroup that finishes last for a (row, kv
+    head) reads the other workgroups' partials) rests on an ordering between workgroups on different XCDs, so it
+    is exercised many times, not once: 3,000 decodes of one or two rows over fresh queries and fresh stretches of
+    a cache, each compared with the CPU reference; stops at the first mismatch."""
+    rng = np.random.default_rng(5)
+    total = 1 << 16
+    k = to_bf16_bits((rng.standard_normal((total, G, D)) * 0.5).astype(np.float32))
+    v = to_bf16_bits((rng.standard_normal((total, G, D)) * 0.5).astype(np.float32))
+    kf, vf = from_bf16_bits(k), from_bf16_bits(v)
+    sinks = rng.standard_normal(H).astype(np.float32)
+    bufs = [gpu.buffer(2 * H * D * 2), gpu.upload(k), gpu.upload(v), gpu.buffer(2 * H * D * 2), gpu.upload(sinks)]
+    row = G * D * 2
+    for it in range(3000):
+        t = 1 + (it & 1)
+        ctx = int(rng.integers(300, 6000))
+        base = int(rng.integers(0, total - ctx))
+        q = to_bf16_bits((rng.standard_normal((t, H, D)) * 0.5).astype(np.float32))
+        bufs[0].write(q)
+        batch = gpu.batch(bufs)
+        shape = C.GroupedShape(t, ctx - t, H, G, D, C.FULL, ctx, 0.125)
+        batch.attention_grouped_with_sinks((C.Slice(0, 0, q.nbytes), C.Slice(1, base * row, ctx * row),
+                                            C.Slice(2, base * row, ctx * row)), C.Slice(4, 0, H * 4),
+                                           C.Slice(3, 0, q.nbytes), shape, C.BF16)
+        done = batch.run()
+        batch.drop()
+        assert not isinstance(done.gpu_time, Exception)
+        got = from_bf16_bits(bufs[3].read(np.uint16, count=t * H * D).reshape(t, H, D))
+        want = orc.attention_f32(from_bf16_bits(q), kf[base:base + ctx], vf[base:base + ctx], sinks, ctx - t,
+                                 scale=0.125, threads=THREADS)
+        err = np.abs(got - want).max()
+        assert err < 2e-2 and not np.isnan(err), (it, t, ctx, base, err)
+    for b in bufs:
+        b.free()
+
+
+def test_buffers_outlive_a_closed_gpu():
+    """Closing a gpu whose buffers are still alive leaves them valid to free (they share the device the way the
+    reference's buffers share theirs); the device goes with the last of them."""
+    g = C.Gpu()
+    a, b = g.upload(np.arange(16, dtype=np.float32)), g.buffer(64)
+    batch = g.batch([b])
+    g.close()
+    batch.drop()
+    assert np.array_equal(a.read(np.float32), np.arange(16, dtype=np.float32))
+    a.free()
+    b.free()
