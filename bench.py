@@ -913,6 +913,51 @@ def run_prepare(gpu, steps, warmup):
     return out
 
 
+def run_wide_heads(gpu, steps, warmup):
+    """The operator's other caller in the reference (decider/src/gpu.rs:878-893): 32 heads over 16 kv heads of
+    width 256, decoding. bf16 caches, one dispatch per layer: one sequence and sixteen at 32,768 cached positions
+    (0.5 and 8.6 GB of cache rows per launch: HBM-fed), the kernels that walk the head in slices of 64 beside the
+    kernel of one wavefront per (row, head) (LNG_WIDE_GENERIC=1)."""
+    heads, kv_heads, dim, ctx = 32, 16, 256, 32768
+    row, qo = kv_heads * dim * 2, heads * dim * 2
+    scale = 1.0 / float(np.sqrt(np.float32(dim)))
+    out = {"workload": "32 heads over 16 kv heads of width 256, bf16, 32768 cached positions, decode"}
+    sinks = gpu.upload(np.random.default_rng(3).standard_normal(heads).astype(np.float32))
+    for n_seq in (1, 16):
+        q, o = gpu.buffer(n_seq * qo), gpu.buffer(n_seq * qo)
+        k, v = gpu.buffer(n_seq * ctx * row), gpu.buffer(n_seq * ctx * row)
+        for i, b in enumerate((q, k, v)):
+            fill(gpu, b, 60 + i)
+        items = C.decode_items([C.DecodeItem(i * qo, i * qo, i * ctx * row, i * ctx * row, 0, ctx - 1, C.FULL, ctx)
+                                for i in range(n_seq)])
+
+        def go():
+            batch = gpu.batch([q, k, v, o, sinks])
+            batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, scale, C.BF16)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time
+
+        nbytes = n_seq * (2 * ctx * row + 2 * qo + heads * 4)
+        res = {"bytes": nbytes}
+        for name, env in (("sliced", None), ("one_wavefront_per_head", "1")):
+            if env:
+                os.environ["LNG_WIDE_GENERIC"] = env
+            try:
+                for _ in range(max(2, warmup)):
+                    go()
+                n = max(steps, 9)
+                t = sorted(go() for _ in range(n))[n // 2]
+            finally:
+                os.environ.pop("LNG_WIDE_GENERIC", None)
+            res[name] = {"gpu_us": t * 1e6, "gbs": nbytes / t / 1e9, "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
+        out["%d_sequences" % n_seq] = res
+        for b in (q, o, k, v):
+            b.free()
+    sinks.free()
+    return out
+
+
 def oracle_threads():
     """Threads the oracle is timed on: the cores this process may use (its affinity mask, and OMP_NUM_THREADS when
     the environment sets it: the GPU boxes grant a one-GPU job 16 of the host's cores), never more than the host has."""
@@ -966,7 +1011,7 @@ def main():
     ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
                     "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block,wide: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     args = ap.parse_args()
@@ -978,7 +1023,7 @@ def main():
     extra = {}
     if args.only:
         runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare, "block": run_block,
-                "c4act": run_prefill_activity, "q8": run_q8}
+                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -997,6 +1042,8 @@ def main():
         extra["decode_block_one_token"] = run_block(gpu, args.steps, args.warmup)
         log("block", extra["decode_block_one_token"])
         extra["c1_fp32"] = run_config1(gpu, args.steps, args.warmup)
+        extra["head_width_256"] = run_wide_heads(gpu, args.steps, args.warmup)
+        log("wide", extra["head_width_256"])
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)
     log("c5", r)
     gpu.close()

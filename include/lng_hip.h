@@ -187,9 +187,10 @@ int lng_hip_attention_grouped_tiled(lng_batch *batch, lng_slice q, lng_slice k, 
  * input). The caller vouches for the sizes behind the addresses.
  *
  * Split-K partials go to a fixed array of LNG_STATIC_SCRATCH_SLOTS x 264 bytes (16.5 MiB) that every GPU the
- * library is opened on holds until the process ends. The limit: t x heads <= LNG_STATIC_MAX_ROW_HEADS (32
- * rows of 64 heads); more is refused with LNG_ERR_DISPATCH (the partials of such a call always fit: a row
- * is cut into at most 32 chunks once a call has 128 (row, kv head) pairs or more). Every call on one GPU
+ * library is opened on holds until the process ends. The limit: t x heads x ceil(dim / 64) <=
+ * LNG_STATIC_MAX_ROW_HEADS (32 rows of 64 heads of width 64; 16 rows of 32 heads of width 256); more is
+ * refused with LNG_ERR_DISPATCH (the partials of such a call fit: a row is cut into at most 32 chunks once
+ * a call has 128 (row, kv head) pairs or more; a plan that would not fit is refused the same way). Every call on one GPU
  * shares that array: calls that may overlap in time on one GPU (different streams with no ordering between
  * them) race on it. Nothing in it has to start at zero: a call overwrites every slot it later reads. */
 #define LNG_STATIC_SCRATCH_SLOTS 65536u

@@ -91,6 +91,7 @@ struct lng_gpu {
     // kernels of the embedded code object
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr;
+    hipFunction_t decode_bf16_wide[3] = {}, decode_f32_wide[3] = {}; // head widths 128, 256, 512
     hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
@@ -403,7 +404,8 @@ uint64_t visible_from_tile(const lng_k_row &r) { // positions from the tile-alig
     return last + 1 - (first & ~(uint64_t)31);
 }
 
-DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_uniform, uint32_t kv_heads, unsigned wgs_per_cu) {
+DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_uniform, uint32_t kv_heads, unsigned wgs_per_cu,
+                       unsigned width = 1 /* head width in units of 64: bytes per position grow with it */) {
     // rows == the table, or one row standing for t_uniform consecutive queries of one cache
     uint64_t total = 0, longest = 0;
     if (t_uniform) {
@@ -433,7 +435,7 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
     // sequence: 4,096 keys 13.9 -> 12.3 us, 131,072 keys 76 -> 50 us); never more than LNG_MAX_CHUNKS (the merge
     // keeps one weight per chunk in LDS).
     const uint64_t pairs = (t_uniform ? t_uniform : (uint64_t)n) * kv_heads;
-    const uint64_t fill = std::min<uint64_t>((wgs_per_cu * g->cus + pairs - 1) / pairs, longest / 512);
+    const uint64_t fill = std::min<uint64_t>((wgs_per_cu * g->cus + pairs - 1) / pairs, longest / std::max(128u, 512u / width));
     const uint64_t most = std::min<uint64_t>(LNG_MAX_CHUNKS, std::max<uint64_t>(longest <= 8192 && pairs <= 16 ? 16 : 32, fill));
     chunk = std::max<uint64_t>(chunk, ((longest + most - 1) / most + 127) / 128 * 128);
     chunk = std::max<uint64_t>(chunk, ((longest + LNG_MAX_CHUNKS - 1) / LNG_MAX_CHUNKS + 127) / 128 * 128);
@@ -448,6 +450,7 @@ DecodePlan plan_decode(lng_gpu *g, const lng_k_row *rows, size_t n, uint64_t t_u
 // What a set of single-query rows (decode, and short passes row by row) runs as.
 struct RowsPlan {
     enum Kind { Generic, Bf16, F32 } kind = Generic;
+    int wide = -1;               // -1: head width 64; 0, 1, 2: the kernels for widths 128, 256, 512
     DecodePlan chunks;
     bool fused = false;          // split-K merged inside the decode kernel (tickets) instead of by lng_decode_merge
     size_t partial_slots = 0;    // (row, kv head, chunk, query head of the group) slots of split-K partials; 0: none
@@ -458,21 +461,26 @@ RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, 
                    bool aligned16) {
     RowsPlan p;
     const uint32_t group = a.heads / a.kv_heads;
-    const bool fast = a.dtype == LNG_BF16 && a.dim == 64 && group <= 16 && aligned16;
+    // Head widths the matrix kernels serve: 64 (gpt-oss), and 128, 256, 512 in slices of 64. Anything else, groups of
+    // more than 16 query heads and operands off 16-byte boundaries go to the kernel of one wavefront per (row, head).
+    const int wide = a.dim == 128 ? 0 : a.dim == 256 ? 1 : a.dim == 512 ? 2 : -1;
+    const bool dim_ok = a.dim == 64 || (wide >= 0 && !getenv("LNG_WIDE_GENERIC"));
+    const bool fast = a.dtype == LNG_BF16 && dim_ok && group <= 16 && aligned16;
     // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the f32 matrix instruction
     // (that kernel counts positions in 32 bits and looks up to 63 past the last one)
     uint64_t latest = t_uniform ? host_rows[0].start + t_uniform - 1 : 0;
     for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
-    const bool fast_f32 = a.dtype == LNG_F32 && a.dim == 64 && group <= 16 && aligned16 && latest < 0xffffff00ull &&
+    const bool fast_f32 = a.dtype == LNG_F32 && dim_ok && group <= 16 && aligned16 && latest < 0xffffff00ull &&
                           a.scale > 0.0f && a.scale <= 3.0e38f && !getenv("LNG_F32_GENERIC");
     p.pairs = n_rows * (size_t)a.kv_heads;
     if (!fast && !fast_f32) return p;
     p.kind = fast ? RowsPlan::Bf16 : RowsPlan::F32;
-    p.chunks = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads, fast ? 1u : 2u);
+    p.wide = wide;
+    p.chunks = plan_decode(g, host_rows, n_rows, t_uniform, a.kv_heads, fast ? 1u : 2u, a.dim / 64);
     if (p.chunks.n_chunks > 1) {
         p.partial_slots = p.pairs * (size_t)p.chunks.n_chunks * group;
-        // Small grids merge inside the kernel; large ones with a second dispatch (the f32 kernel always).
-        p.fused = fast && (uint64_t)p.chunks.n_chunks * p.pairs <= g->fuse_wgs;
+        // Small grids merge inside the kernel; large ones with a second dispatch (the f32 and wide-head kernels always).
+        p.fused = fast && wide < 0 && (uint64_t)p.chunks.n_chunks * p.pairs <= g->fuse_wgs;
     }
     return p;
 }
@@ -522,8 +530,15 @@ int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *
         a.work = work_dev;
         wgs = n;
     }
-    out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_d64 : g->decode_f32_d64,
-                        p.kind == RowsPlan::Bf16 ? "lng_decode_bf16_d64" : "lng_decode_f32_d64", (unsigned)wgs, a};
+    static const char *const wide_bf16[3] = {"lng_decode_bf16_w128", "lng_decode_bf16_w256", "lng_decode_bf16_w512"};
+    static const char *const wide_f32[3] = {"lng_decode_f32_w128", "lng_decode_f32_w256", "lng_decode_f32_w512"};
+    if (p.wide >= 0) {
+        out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_wide[p.wide] : g->decode_f32_wide[p.wide],
+                            p.kind == RowsPlan::Bf16 ? wide_bf16[p.wide] : wide_f32[p.wide], (unsigned)wgs, a};
+    } else {
+        out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_d64 : g->decode_f32_d64,
+                            p.kind == RowsPlan::Bf16 ? "lng_decode_bf16_d64" : "lng_decode_f32_d64", (unsigned)wgs, a};
+    }
     if (a.n_chunks > 1 && !a.fused) { // a workgroup per (row, kv head, query head)
         out->l[out->n++] = {g->decode_merge, "lng_decode_merge", (unsigned)(p.pairs * group), a};
     }
@@ -536,7 +551,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     lng_gpu *g = b->gpu;
     const RowsPlan p = plan_rows(g, a, host_rows, n_rows, t_uniform, aligned16);
     if (p.partial_slots) {
-        if (int rc = reserve_scratch(g, p.partial_slots * 64, p.partial_slots * 2, p.pairs)) return rc;
+        if (int rc = reserve_scratch(g, p.partial_slots * a.dim, p.partial_slots * 2, p.pairs)) return rc;
         a.partial_o = g->scratch_o;
         a.partial_ml = g->scratch_ml;
         a.tickets = g->tickets;
@@ -762,6 +777,12 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
         {"lng_decode_merge", &g->decode_merge, true},
         {"lng_decode_f32_d64", &g->decode_f32_d64, true},
+        {"lng_decode_bf16_w128", &g->decode_bf16_wide[0], true},
+        {"lng_decode_bf16_w256", &g->decode_bf16_wide[1], true},
+        {"lng_decode_bf16_w512", &g->decode_bf16_wide[2], true},
+        {"lng_decode_f32_w128", &g->decode_f32_wide[0], true},
+        {"lng_decode_f32_w256", &g->decode_f32_wide[1], true},
+        {"lng_decode_f32_w512", &g->decode_f32_wide[2], true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_prefill_bf16_d64_stream", &g->prefill_bf16_d64_stream, true},
@@ -1136,9 +1157,10 @@ extern "C" int lng_hip_attention_grouped_static(lng_gpu *g, void *stream, const 
     if (!q || !k || !v || !out) return fail(LNG_ERR_DISPATCH, "q, k, v and out must be device addresses");
     const lng_grouped_shape &s = *shape;
     if (int rc = check_shape(s, false)) return rc;
-    if (s.t * s.heads > LNG_STATIC_MAX_ROW_HEADS) {
-        return fail(LNG_ERR_DISPATCH, "%llu rows of %llu heads: the fixed scratch array is sized for rows x heads <= %u",
-                    (unsigned long long)s.t, (unsigned long long)s.heads, (unsigned)LNG_STATIC_MAX_ROW_HEADS);
+    const uint64_t width = std::max<uint64_t>(1, (s.dim + 63) / 64); // partial outputs take `dim` floats per slot
+    if (s.t * s.heads * width > LNG_STATIC_MAX_ROW_HEADS) {
+        return fail(LNG_ERR_DISPATCH, "%llu rows of %llu heads of width %llu: the fixed scratch array is sized for rows x heads x ceil(dim / 64) <= %u",
+                    (unsigned long long)s.t, (unsigned long long)s.heads, (unsigned long long)s.dim, (unsigned)LNG_STATIC_MAX_ROW_HEADS);
     }
     const uint64_t es = elem_size(dtype);
     if (!fits_u32(s.heads * s.dim * es)) return fail(LNG_ERR_DISPATCH, "rows of %llu bytes do not fit in u32", (unsigned long long)(s.heads * s.dim * es));
@@ -1173,10 +1195,10 @@ extern "C" int lng_hip_attention_grouped_static(lng_gpu *g, void *stream, const 
     const bool aligned16 = ((pq | pk | pv | po) & 15u) == 0;
     RowsPlan p = plan_rows(g, a, &a.first, s.t, s.t, aligned16);
     p.fused = false; // lng_decode_merge as the second launch: no arrival counters, nothing that must start at zero
-    if (p.partial_slots > LNG_STATIC_MAX_SLOTS) { // only a planner told to make more workgroups than usual gets here
+    if (p.partial_slots * (s.dim / 64) > LNG_STATIC_MAX_SLOTS) { // only a planner told to make more workgroups than usual gets here
         return fail(LNG_ERR_DISPATCH,
                     "%llu rows of %llu heads in %u chunks need %zu slots of split-K scratch; the fixed array holds %u (%zu bytes)",
-                    (unsigned long long)s.t, (unsigned long long)s.heads, p.chunks.n_chunks, p.partial_slots,
+                    (unsigned long long)s.t, (unsigned long long)s.heads, p.chunks.n_chunks, p.partial_slots * (size_t)(s.dim / 64),
                     (unsigned)LNG_STATIC_MAX_SLOTS, (size_t)LNG_STATIC_SCRATCH_BYTES);
     }
     if (p.partial_slots) {

@@ -7,8 +7,11 @@
 //     first = max(0, last + 1 - window);  s_p = (q . k_p) * scale for p in first..=last
 //     m = max(sink, max_p s_p);  Z = exp(sink - m) + sum_p exp(s_p - m)
 //     out = sum_p exp(s_p - m) / Z * v_p                      (position p is in row p % slots)
-// Nothing below is translated from the Metal kernels; the work split, layouts and reductions
-// are chosen for 64-wide wavefronts, MFMA and HBM streaming.
+// The kernels that carry the load (head widths 64, 128, 256 and 512, groups of up to 16 query heads per kv head)
+// choose their work split, layouts and reductions for 64-wide wavefronts, MFMA and HBM streaming: K and V are read
+// once per kv head, long rows are cut into chunks. One kernel keeps the reference's own split of a workgroup per
+// (row, head) - lng_attn_generic_* - and serves only what is left: other widths, larger groups, scales that are
+// not positive, operands off 16-byte boundaries.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -120,11 +123,11 @@ __device__ __forceinline__ float wave_sum(float x) {
 
 // =============================================================================================
 // Generic kernel: any element type, any head width up to 512, any group size. One workgroup
-// per (row, head); its four wavefronts take every fourth position, lanes split the head
+// per (row, head) (the reference's split, kernels.metal:500-560: each query head reads its kv head's
+// rows again); its four wavefronts take every fourth position, lanes split the head
 // dimension; per-wavefront online softmax, merged in LDS with the sink joining the merge.
-// Used for f32 (the reference's element type), for widths other than 64 and as the fallback
-// when an operand is not 16-byte aligned. Accurate exp/divide: this is the path held to
-// 1e-5 relative against the CPU reference.
+// The remainder kernel: head widths other than 64, 128, 256, 512, groups of more than 16 query heads,
+// f32 with a scale that is not positive, operands off 16-byte boundaries. Accurate exp/divide.
 // =============================================================================================
 template <typename T>
 __device__ __forceinline__ void attn_generic(const lng_k_attn &a) {
@@ -800,6 +803,450 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
     }
 }
 
+// =============================================================================================
+// Decode kernels for head widths 128, 256 and 512 (DS slices of 64 dimensions): the plan of the two
+// kernels above - one workgroup per (row, kv head, chunk) serves every query head of the group, so K
+// and V are read once per kv head; chunks, partials and lng_decode_merge are shared - with the head
+// dimension walked in slices. Scores accumulate over the slices of K on the matrix unit; after the
+// softmax each slice of V gives its 64 output dimensions. Loads run one batch ahead of the
+// arithmetic (a batch = two slices of K or of V for bf16, one for f32), across tiles too.
+// Callers: the reference's other user of this operator has 32 heads over 16 kv heads of width 256
+// (decider/src/gpu.rs:878-893), its own tests go to width 512 (attention_grouped.rs:187-199).
+// =============================================================================================
+template <int DS> __device__ __forceinline__ void decode_wide_bf16(const lng_k_attn &a) {
+    __shared__ float s_m[4][16];
+    __shared__ float s_l[4][16];
+    __shared__ float s_o[4][16][65];
+    constexpr int SB = DS >= 8 ? 4 : 2; // slices per batch of loads
+    constexpr int KBATCH = DS / SB;    // batches of K per tile, and as many of V
+    constexpr int NBATCH = 2 * KBATCH;
+
+    const work_item wi = work_of(a);
+    const uint32_t row = wi.pair / a.kv_heads;
+    const uint32_t g = wi.pair % a.kv_heads;
+    const lng_k_row it = row_of(a, row);
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+    const uint64_t base = first & ~(uint64_t)31;
+    const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
+    if (c0 > last) return;
+    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n = lane & 15u;
+    const uint32_t j = lane >> 4;
+    const uint32_t group = a.heads / a.kv_heads;
+    const bool wraps = it.slots <= last;
+    constexpr uint32_t head_bytes = 128u * DS;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * head_bytes;
+    const char *kb = a.k + it.k_offset + (uint64_t)g * head_bytes + j * 16u;
+    const char *vb = a.v + it.v_offset + (uint64_t)g * head_bytes + j * 16u;
+
+    bf16x8 qb[DS][2]; // head n of this group: the lane's 8 k-slots of each step of each slice
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+        uint4 q0 = make_uint4(0, 0, 0, 0), q1 = q0;
+        if (n < group) {
+            const char *qp = a.q + it.q_offset + ((uint64_t)g * group + n) * head_bytes + s * 128u + j * 16u;
+            q0 = *(const uint4 *)qp;
+            q1 = *(const uint4 *)(qp + 64);
+        }
+        qb[s][0] = as_bf16x8(q0);
+        qb[s][1] = as_bf16x8(q1);
+    }
+    bf16x8 sel[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sel[b][e] = (8u * j + (uint32_t)e == 16u * (uint32_t)b + n) ? (__bf16)1.0f : (__bf16)0.0f;
+        }
+    }
+
+    struct batch {
+        uint4 x[2][SB][2]; // [position half][slice of the batch][k step]
+    };
+    struct rows2 {
+        uint64_t lo, hi; // byte offsets of the cache rows of the lane's two positions of a tile
+    };
+    auto row_at = [&](uint64_t p) -> uint64_t {
+        p = p < first ? first : p;
+        p = p > last ? last : p;
+        return (wraps ? p % it.slots : p) * row_bytes;
+    };
+    auto offsets = [&](uint64_t tp) -> rows2 { return rows2{row_at(tp + n), row_at(tp + 16u + n)}; };
+    auto load_batch = [&](const rows2 &off, int b, batch &t) {
+        const char *from = (b < KBATCH ? kb : vb) + (uint32_t)((b % KBATCH) * SB) * 128u;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const char *at = from + (half ? off.hi : off.lo);
+#pragma unroll
+            for (int u = 0; u < SB; ++u) {
+                t.x[half][u][0] = *(const uint4 *)(at + u * 128);
+                t.x[half][u][1] = *(const uint4 *)(at + u * 128 + 64);
+            }
+        }
+    };
+
+    const float sl2 = a.scale * LNG_LOG2E;
+    float m = LNG_NEG_INF, l = 0.0f;
+    floatx4 ot[DS][4]; // O^T[64s + 16mm + 4j + i][head n]
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) ot[s][mm] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    }
+    const floatx4 zero4 = (floatx4){0.f, 0.f, 0.f, 0.f};
+
+    batch cur, nxt;
+    rows2 off = {0, 0}, off_next = {0, 0};
+    uint64_t tp = c0 + (uint64_t)wave * 32u;
+    if (tp < c1) {
+        off = offsets(tp);
+        load_batch(off, 0, cur);
+    }
+    for (; tp < c1; tp += 128u) {
+        const bool more = tp + 128u < c1;
+        if (more) off_next = offsets(tp + 128u);
+        floatx4 st[2] = {zero4, zero4};
+        float alpha = 1.0f;
+        bf16x8 pb;
+#pragma unroll
+        for (int b = 0; b < NBATCH; ++b) {
+            if (b + 1 < NBATCH) {
+                load_batch(off, b + 1, nxt);
+            } else if (more) {
+                load_batch(off_next, 0, nxt);
+            }
+            if (b < KBATCH) {
+#pragma unroll
+                for (int u = 0; u < SB; ++u) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.x[half][u][0]), qb[b * SB + u][0], st[half], 0, 0, 0);
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.x[half][u][1]), qb[b * SB + u][1], st[half], 0, 0, 0);
+                    }
+                }
+                if (b == KBATCH - 1) { // every slice of K is in: the tile's softmax
+                    float tmax = LNG_NEG_INF;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint64_t p = tp + (uint64_t)(half * 16 + i) + 4u * j;
+                            const float x = (p >= first && p <= last) ? st[half][i] * sl2 : LNG_NEG_INF;
+                            st[half][i] = x;
+                            tmax = fmaxf(tmax, x);
+                        }
+                    }
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                    const float m_new = fmaxf(m, tmax);
+                    const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                    alpha = __builtin_amdgcn_exp2f(m - m_safe);
+                    float psum = 0.0f;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float pw = __builtin_amdgcn_exp2f(st[half][i] - m_safe);
+                            st[half][i] = pw;
+                            psum += pw;
+                        }
+                    }
+                    l = l * alpha + psum;
+                    m = m_new;
+                    pb = narrow8(st[0], st[1]);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < SB; ++u) {
+                    const int s = (b - KBATCH) * SB + u;
+#pragma unroll
+                    for (int mm = 0; mm < 4; ++mm) {
+                        const floatx4 t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.x[0][u][mm >> 1]), sel[mm & 1], zero4, 0, 0, 0);
+                        const floatx4 t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(cur.x[1][u][mm >> 1]), sel[mm & 1], zero4, 0, 0, 0);
+                        const bf16x8 va = narrow8(t0, t1);
+                        ot[s][mm] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pb, ot[s][mm] * alpha, 0, 0, 0);
+                    }
+                }
+            }
+            cur = nxt;
+        }
+        off = off_next;
+    }
+
+    // ---- merge the four wavefronts, 64 output dimensions at a time ---------------------------------
+    {
+        float lt = l + __shfl_xor(l, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (j == 0) {
+            s_m[wave][n] = m;
+            s_l[wave][n] = lt;
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+        if (s) __syncthreads(); // the previous slice has been read
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_o[wave][n][16 * mm + 4 * j + i] = ot[s][mm][i];
+        }
+        __syncthreads();
+        for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
+            const uint32_t h = idx >> 6;
+            const uint32_t d = idx & 63u;
+            float top = LNG_NEG_INF;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) top = fmaxf(top, s_m[w][h]);
+            float sum = 0.0f, o = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(s_m[w][h] - top);
+                sum += s_l[w][h] * wt;
+                o += s_o[w][h][d] * wt;
+            }
+            if (row_chunks == 1) {
+                const uint32_t head = g * group + h;
+                const float sink2 = it.sinks_offset != LNG_NO_SINKS
+                                        ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                        : LNG_NEG_INF;
+                const float all = fmaxf(top, sink2);
+                const float keep = __builtin_amdgcn_exp2f(top - all);
+                const float z = sum * keep + (sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - all));
+                uint16_t *op = (uint16_t *)(a.out + it.out_offset) + (uint64_t)head * (64u * DS) + 64u * s + d;
+                *op = f32_to_bf16_bits(o * keep / z);
+            } else { // lng_decode_merge runs as the next dispatch
+                const uint64_t slot = ((uint64_t)wi.pair * a.n_chunks + wi.chunk) * group + h;
+                a.partial_o[slot * (64u * DS) + 64u * s + d] = o;
+                if (s == 0 && d == 0) {
+                    a.partial_ml[slot * 2u] = top;
+                    a.partial_ml[slot * 2u + 1u] = sum;
+                }
+            }
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void lng_decode_bf16_w128(lng_k_attn a) { decode_wide_bf16<2>(a); }
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void lng_decode_bf16_w256(lng_k_attn a) { decode_wide_bf16<4>(a); }
+extern "C" __global__ __launch_bounds__(256) void lng_decode_bf16_w512(lng_k_attn a) { decode_wide_bf16<8>(a); }
+
+// f32 (the reference's element type): lng_decode_f32_d64's products (v_mfma_f32_16x16x4_f32, V arriving transposed
+// straight from memory), a slice of 64 dimensions per batch of loads. The queries wait in LDS (16 heads x 512 floats
+// would not fit the registers beside 128 accumulators).
+template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_attn &a) {
+    __shared__ float s_m[4][16];
+    __shared__ float s_l[4][16];
+    __shared__ float s_o[4][16][65];
+    __shared__ __attribute__((aligned(16))) float s_q[16][64 * DS + 4];
+    constexpr int NBATCH = 2 * DS;
+
+    const work_item wi = work_of(a);
+    const uint32_t row = wi.pair / a.kv_heads;
+    const uint32_t g = wi.pair % a.kv_heads;
+    const lng_k_row it = row_of(a, row);
+    const uint64_t last = it.start;
+    const uint64_t first = first_visible(last, it.window);
+    const uint64_t base = first & ~(uint64_t)31;
+    const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
+    if (c0 > last) return;
+    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t n = lane & 15u;
+    const uint32_t j = lane >> 4;
+    const uint32_t group = a.heads / a.kv_heads;
+    const bool wraps = it.slots <= last;
+    constexpr uint32_t D = 64u * DS;
+    const uint64_t row_floats = (uint64_t)a.kv_heads * D;
+    const float *kb = (const float *)(a.k + it.k_offset) + (uint64_t)g * D + 4u * j;
+    const float *vb = (const float *)(a.v + it.v_offset) + (uint64_t)g * D + n;
+
+    for (uint32_t idx = threadIdx.x; idx < 16u * D; idx += 256u) { // heads past the group: zero queries
+        const uint32_t h = idx / D, d = idx % D;
+        s_q[h][d] = h < group ? ((const float *)(a.q + it.q_offset))[((uint64_t)g * group + h) * D + d] : 0.0f;
+    }
+    __syncthreads();
+
+    struct batch {
+        float4 k[2][4]; // K: [position half][dim step of the slice]
+    };                  // V reuses the 32 registers: [half][4 * i + mm] = position 4j + i, dim 16mm + n of the slice
+    auto row_of_pos = [&](uint64_t p) -> uint64_t {
+        p = p < first ? first : p;
+        p = p > last ? last : p;
+        return (wraps ? p % it.slots : p) * row_floats;
+    };
+    auto load_batch = [&](uint64_t tp, int b, batch &t) {
+        if (b < DS) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const float *kp = kb + row_of_pos(tp + 16u * half + n) + 64 * b;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) t.k[half][s] = *(const float4 *)(kp + 16 * s);
+            }
+        } else {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float *vp = vb + row_of_pos(tp + 16u * half + 4u * j + i) + 64 * (b - DS);
+                    float4 x;
+                    x.x = vp[0];
+                    x.y = vp[16];
+                    x.z = vp[32];
+                    x.w = vp[48];
+                    t.k[half][i] = x; // .x .y .z .w = dim blocks mm = 0..3
+                }
+            }
+        }
+    };
+
+    const float sl2 = a.scale * LNG_LOG2E;
+    float m = LNG_NEG_INF, l = 0.0f;
+    floatx4 ot[DS][4];
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) ot[s][mm] = (floatx4){0.f, 0.f, 0.f, 0.f};
+    }
+
+    batch cur, nxt;
+    uint64_t tp = c0 + (uint64_t)wave * 32u;
+    if (tp < c1) load_batch(tp, 0, cur);
+    for (; tp < c1; tp += 128u) {
+        const bool more = tp + 128u < c1;
+        floatx4 st[2] = {(floatx4){0.f, 0.f, 0.f, 0.f}, (floatx4){0.f, 0.f, 0.f, 0.f}};
+        float alpha = 1.0f;
+#pragma unroll
+        for (int b = 0; b < NBATCH; ++b) {
+            if (b + 1 < NBATCH) {
+                load_batch(tp, b + 1, nxt);
+            } else if (more) {
+                load_batch(tp + 128u, 0, nxt);
+            }
+            if (b < DS) {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const float4 qv = *(const float4 *)(&s_q[n][64 * b + 16 * s + 4 * j]);
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].x, qv.x, st[half], 0, 0, 0);
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].y, qv.y, st[half], 0, 0, 0);
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].z, qv.z, st[half], 0, 0, 0);
+                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].w, qv.w, st[half], 0, 0, 0);
+                    }
+                }
+                if (b == DS - 1) {
+                    float tmax = LNG_NEG_INF;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint64_t p = tp + (uint64_t)(half * 16 + i) + 4u * j;
+                            const float x = (p >= first && p <= last) ? st[half][i] : LNG_NEG_INF;
+                            st[half][i] = x;
+                            tmax = fmaxf(tmax, x);
+                        }
+                    }
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+                    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                    const float m_new = fmaxf(m, tmax * sl2); // scale > 0: the maximum commutes with it
+                    const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+                    alpha = __builtin_amdgcn_exp2f(m - m_safe);
+                    float psum = 0.0f;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float pw = __builtin_amdgcn_exp2f(__builtin_fmaf(st[half][i], sl2, -m_safe));
+                            st[half][i] = pw;
+                            psum += pw;
+                        }
+                    }
+                    l = l * alpha + psum;
+                    m = m_new;
+                }
+            } else {
+                const int s = b - DS;
+#pragma unroll
+                for (int mm = 0; mm < 4; ++mm) {
+                    ot[s][mm] = ot[s][mm] * alpha;
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const float4 x = cur.k[half][i];
+                            const float vx = mm == 0 ? x.x : mm == 1 ? x.y : mm == 2 ? x.z : x.w;
+                            ot[s][mm] = __builtin_amdgcn_mfma_f32_16x16x4f32(vx, st[half][i], ot[s][mm], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            cur = nxt;
+        }
+    }
+
+    {
+        float lt = l + __shfl_xor(l, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+        if (j == 0) {
+            s_m[wave][n] = m;
+            s_l[wave][n] = lt;
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+        if (s) __syncthreads();
+#pragma unroll
+        for (int mm = 0; mm < 4; ++mm) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s_o[wave][n][16 * mm + 4 * j + i] = ot[s][mm][i];
+        }
+        __syncthreads();
+        for (uint32_t idx = threadIdx.x; idx < group * 64u; idx += 256u) {
+            const uint32_t h = idx >> 6;
+            const uint32_t d = idx & 63u;
+            float top = LNG_NEG_INF;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) top = fmaxf(top, s_m[w][h]);
+            float sum = 0.0f, o = 0.0f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float wt = s_m[w][h] == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(s_m[w][h] - top);
+                sum += s_l[w][h] * wt;
+                o += s_o[w][h][d] * wt;
+            }
+            if (row_chunks == 1) {
+                const uint32_t head = g * group + h;
+                const float sink = it.sinks_offset != LNG_NO_SINKS
+                                       ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
+                                       : LNG_NEG_INF;
+                const float all = fmaxf(top, sink);
+                const float keep = top == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(top - all);
+                const float z = sum * keep + (sink == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink - all));
+                ((float *)(a.out + it.out_offset))[(uint64_t)head * D + 64u * s + d] = o * keep / z;
+            } else {
+                const uint64_t slot = ((uint64_t)wi.pair * a.n_chunks + wi.chunk) * group + h;
+                a.partial_o[slot * D + 64u * s + d] = o;
+                if (s == 0 && d == 0) {
+                    a.partial_ml[slot * 2u] = top;
+                    a.partial_ml[slot * 2u + 1u] = sum;
+                }
+            }
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void lng_decode_f32_w128(lng_k_attn a) { decode_wide_f32<2>(a); }
+extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_w256(lng_k_attn a) { decode_wide_f32<4>(a); }
+extern "C" __global__ __launch_bounds__(256) void lng_decode_f32_w512(lng_k_attn a) { decode_wide_f32<8>(a); }
+
 // The merge as its own dispatch, for large grids (there a workgroup that waits for its coherent stores and
 // its ticket holds a compute unit's slot that another chunk could use) and for the f32 kernel. One workgroup
 // per (row, kv head, query head), the query head the fast index of the grid: thread c turns chunk c's (max, sum) into a weight, then thread (dim, quarter)
@@ -844,27 +1291,31 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a)
     z = (s_red[1][0] + s_red[1][1]) + (s_red[1][2] + s_red[1][3]) +
         (sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top));
     const uint32_t d = tid & 63u;
-    const float *po = a.partial_o + slot0 * 64u + d;
-    const uint64_t step = (uint64_t)group * 64u;
-    float o = 0.0f;
-    uint32_t c = wave;
-    for (; c + 28u < row_chunks; c += 32u) { // eight loads in flight per turn
-        float x[8];
+    const uint64_t step = (uint64_t)group * a.dim;
+    for (uint32_t db = 0; db < a.dim; db += 64u) { // 64 dimensions at a time (one turn at the gpt-oss head width)
+        const float *po = a.partial_o + slot0 * a.dim + db + d;
+        float o = 0.0f;
+        uint32_t c = wave;
+        for (; c + 28u < row_chunks; c += 32u) { // eight loads in flight per turn
+            float x[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) x[u] = po[(c + 4u * u) * step];
+            for (int u = 0; u < 8; ++u) x[u] = po[(c + 4u * u) * step];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) o += x[u] * s_w[c + 4u * u];
-    }
-    for (; c < row_chunks; c += 4u) o += po[c * step] * s_w[c];
-    s_acc[wave][d] = o;
-    __syncthreads();
-    if (wave != 0) return;
-    const float res = ((s_acc[0][d] + s_acc[1][d]) + (s_acc[2][d] + s_acc[3][d])) / z;
-    const uint64_t at = (uint64_t)head * 64u + d;
-    if (a.dtype == LNG_F32) {
-        ((float *)(a.out + it.out_offset))[at] = res;
-    } else {
-        ((uint16_t *)(a.out + it.out_offset))[at] = f32_to_bf16_bits(res);
+            for (int u = 0; u < 8; ++u) o += x[u] * s_w[c + 4u * u];
+        }
+        for (; c < row_chunks; c += 4u) o += po[c * step] * s_w[c];
+        if (db) __syncthreads(); // the previous turn's sums have been read
+        s_acc[wave][d] = o;
+        __syncthreads();
+        if (wave == 0) {
+            const float res = ((s_acc[0][d] + s_acc[1][d]) + (s_acc[2][d] + s_acc[3][d])) / z;
+            const uint64_t at = (uint64_t)head * a.dim + db + d;
+            if (a.dtype == LNG_F32) {
+                ((float *)(a.out + it.out_offset))[at] = res;
+            } else {
+                ((uint16_t *)(a.out + it.out_offset))[at] = f32_to_bf16_bits(res);
+            }
+        }
     }
 }
 

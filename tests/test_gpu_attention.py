@@ -134,8 +134,8 @@ def test_decode_bf16_window_ring_and_edges(gpu, start, window, slots):
 @pytest.mark.parametrize("heads,kv_heads,dim", [(8, 8, 64), (16, 1, 64), (12, 4, 64), (64, 2, 64), (8, 2, 128),
                                                 (4, 4, 32)])
 def test_decode_bf16_other_groupings(gpu, heads, kv_heads, dim):
-    """Group sizes 1..32 and widths other than 64 (the latter, and groups over 16, take the
-    general kernel)."""
+    """Group sizes 1..32 and widths other than 64 (width 32, and groups over 16, take the
+    general kernel; width 128 the kernel that walks the head dimension in slices)."""
     start = 777
     q, k, v, sinks = normal_inputs(5, 3, start + 3, heads, kv_heads, dim, scale=0.5)
     qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
@@ -634,3 +634,88 @@ def test_scales_that_are_not_positive(gpu, scale):
         wantb = oracle.attention_bf16(qb, kb, vb, sinks, start, window=FULL, scale=scale, threads=THREADS)
         gotb = run_attention(gpu, qb, krb, vrb, sinks, shape, tiled, C.BF16)
         assert max_error(from_bf16_bits(gotb), from_bf16_bits(wantb)) < BF16_TOL
+
+
+# ---- head widths 128, 256 and 512: K and V read once per kv head, the head dimension walked in slices of 64 ----
+WIDE_CASES = [
+    # the reference's other user of the operator: 32 heads over 16 kv heads of width 256 (decider/src/gpu.rs:878-893)
+    (1, 0, FULL, 1, 32, 16, 256), (1, 36, FULL, 37, 32, 16, 256), (1, 4095, FULL, 4096, 32, 16, 256),
+    (1, 5000, 128, 200, 32, 16, 256), (1, 9000, FULL, 9001, 32, 16, 256), (4, 700, FULL, 704, 32, 16, 256),
+    (1, 33000, FULL, 33001, 8, 4, 256), (1, 50000, 30000, 32768, 16, 1, 256),
+    (3, 2000, FULL, 2003, 8, 8, 128), (7, 900, 33, 41, 6, 2, 128), (1, 40000, FULL, 40001, 16, 1, 128),
+    (1, 131, FULL, 132, 64, 8, 128), (2, 31, FULL, 33, 5, 1, 128),
+    (2, 9000, 1, 3, 8, 2, 512), (1, 9000, FULL, 9001, 8, 2, 512), (5, 260, 300, 305, 24, 8, 512),
+    (1, 20000, 7000, 8192, 4, 1, 512), (1, 63, FULL, 64, 16, 1, 512),
+]
+
+
+@pytest.mark.parametrize("dtype", [C.BF16, C.F32])
+@pytest.mark.parametrize("t,start,window,slots,heads,kv_heads,dim", WIDE_CASES)
+def test_decode_at_head_widths_128_256_512(gpu, dtype, t, start, window, slots, heads, kv_heads, dim, monkeypatch):
+    """The row-by-row operator at the wider heads: one chunk and many (merged by a second dispatch), rings that
+    have wrapped, windows that start inside a tile, groups of 1..16, with and without sinks; rows the operator must
+    not read hold NaN (attention_grouped.rs:57). To the bars of the width-64 kernels against the CPU reference, and
+    the kernel of one wavefront per (row, head) (LNG_WIDE_GENERIC) agrees."""
+    end = start + t
+    rng = np.random.default_rng(start + t + dim)
+    scale = float(1.0 / np.sqrt(np.float32(dim)))
+    q = rng.standard_normal((t, heads, dim), dtype=np.float32) * np.float32(0.7)
+    first = 0 if window == FULL else max(0, start + 1 - window)
+    kept = max(first, end - slots)
+    k = np.full((end, kv_heads, dim), np.nan, np.float32)
+    v = np.full((end, kv_heads, dim), np.nan, np.float32)
+    k[kept:] = rng.standard_normal((end - kept, kv_heads, dim), dtype=np.float32) * np.float32(0.7)
+    v[kept:] = rng.standard_normal((end - kept, kv_heads, dim), dtype=np.float32)
+    shape = C.GroupedShape(t, start, heads, kv_heads, dim, window, slots, scale)
+    kr, vr = ring_layout(k, t, start, slots, False), ring_layout(v, t, start, slots, False)
+    kz, vz = np.nan_to_num(k), np.nan_to_num(v)     # the oracle multiplies unseen rows by zero weights
+    if dtype == C.BF16:
+        q, kr, vr, kz, vz = (to_bf16_bits(x) for x in (q, kr, vr, kz, vz))
+    for sinks in (rng.standard_normal(heads).astype(np.float32), None):
+        if dtype == C.F32:
+            want = oracle.attention_f32(q, kz, vz, sinks, start, window=window, scale=scale, threads=THREADS)
+            err = lambda got: rel_error(got, want)  # noqa: E731
+            bar = F32_RTOL
+        else:
+            want = from_bf16_bits(oracle.attention_bf16(q, kz, vz, sinks, start, window=window, scale=scale, threads=THREADS))
+            err = lambda got: max_error(from_bf16_bits(got), want)  # noqa: E731
+            bar = BF16_TOL
+        got = run_attention(gpu, q, kr, vr, sinks, shape, False, dtype)
+        assert err(got) <= bar
+        monkeypatch.setenv("LNG_WIDE_GENERIC", "1")
+        generic = run_attention(gpu, q, kr, vr, sinks, shape, False, dtype)
+        monkeypatch.delenv("LNG_WIDE_GENERIC")
+        assert err(generic) <= bar
+
+
+def test_ragged_table_of_sequences_at_head_width_256(gpu):
+    """attention_decode_batched at 32 heads over 16 kv heads of width 256: sequences of very different
+    lengths in one dispatch (live workgroups only), each against the CPU reference on its own cache."""
+    heads, kv_heads, dim = 32, 16, 256
+    lens = [1, 40, 129, 700, 5000, 12000, 33, 2048]
+    rng = np.random.default_rng(256)
+    row = kv_heads * dim
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    k_all = to_bf16_bits(rng.standard_normal((int(offs[-1]), kv_heads, dim), dtype=np.float32) * np.float32(0.7))
+    v_all = to_bf16_bits(rng.standard_normal((int(offs[-1]), kv_heads, dim), dtype=np.float32))
+    q = to_bf16_bits(rng.standard_normal((len(lens), heads, dim), dtype=np.float32) * np.float32(0.7))
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    scale = float(1.0 / np.sqrt(np.float32(dim)))
+    bufs = [gpu.upload(q), gpu.upload(k_all), gpu.upload(v_all), gpu.buffer(q.nbytes), gpu.upload(sinks)]
+    bufs[3].fill(0xFF)
+    items = [C.DecodeItem(i * heads * dim * 2, i * heads * dim * 2, int(offs[i]) * row * 2, int(offs[i]) * row * 2, 0,
+                          n - 1, FULL, n) for i, n in enumerate(lens)]
+    batch = gpu.batch(bufs)
+    try:
+        batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, scale, C.BF16)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        out = bufs[3].read(np.uint16).reshape(len(lens), heads, dim)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    for i, n in enumerate(lens):
+        ks, vs = k_all[offs[i]:offs[i + 1]], v_all[offs[i]:offs[i + 1]]
+        want = oracle.attention_bf16(q[i:i + 1], ks, vs, sinks, n - 1, scale=scale, threads=THREADS)
+        assert max_error(from_bf16_bits(out[i:i + 1]), from_bf16_bits(want)) < BF16_TOL, (i, n)

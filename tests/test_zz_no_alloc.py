@@ -66,14 +66,22 @@ def test_static_entry_point_matches_the_batch_entry_point_on_calls_in_a_row(gpu,
             assert rel_error(got, want.astype(np.float64)) < F32_RTOL, (t, ctx, window)
 
 
-def test_static_entry_point_takes_other_head_widths(gpu):
-    """Widths the split-K kernels do not take run on the kernel without scratch."""
-    t, ctx, heads, kv_heads, dim = 2, 300, 8, 2, 128
-    q, k, v, sinks = normal_inputs(7, t, ctx, heads, kv_heads, dim, scale=0.5)
-    shape = C.GroupedShape(t, ctx - t, heads, kv_heads, dim, FULL, ctx, 0.1)
-    got = static_call(gpu, q, k, v, sinks, shape, C.F32)
-    want = oracle.attention_f32(q, k, v, sinks, ctx - t, window=FULL, scale=0.1, threads=THREADS)
-    assert rel_error(got, want.astype(np.float64)) < F32_RTOL
+@pytest.mark.parametrize("dtype", [C.BF16, C.F32])
+def test_static_entry_point_takes_other_head_widths(gpu, dtype):
+    """Width 256 (32 heads over 16 kv heads) in many chunks and then in one, sharing the fixed array (partials of
+    `dim` floats per slot); width 96 runs on the kernel without scratch."""
+    for t, ctx, heads, kv_heads, dim in [(1, 20000, 32, 16, 256), (2, 300, 32, 16, 256), (2, 300, 8, 2, 96)]:
+        q, k, v, sinks = normal_inputs(7 + ctx, t, ctx, heads, kv_heads, dim, scale=0.5)
+        shape = C.GroupedShape(t, ctx - t, heads, kv_heads, dim, FULL, ctx, 0.1)
+        if dtype == C.BF16:
+            qd, kd, vd = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+            got = static_call(gpu, qd, kd, vd, sinks, shape, dtype)
+            want = oracle.attention_bf16(qd, kd, vd, sinks, ctx - t, window=FULL, scale=0.1, threads=THREADS)
+            assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL, (t, ctx, dim)
+        else:
+            got = static_call(gpu, q, k, v, sinks, shape, dtype)
+            want = oracle.attention_f32(q, k, v, sinks, ctx - t, window=FULL, scale=0.1, threads=THREADS)
+            assert rel_error(got, want.astype(np.float64)) < F32_RTOL, (t, ctx, dim)
 
 
 def test_static_entry_point_refuses_what_does_not_fit_or_is_malformed(gpu):
@@ -85,6 +93,11 @@ def test_static_entry_point_refuses_what_does_not_fit_or_is_malformed(gpu):
         big = C.GroupedShape(33, 1000, heads, kv_heads, dim, FULL, 2048, 0.125)
         with pytest.raises(C.Dispatch) as e:
             gpu.attention_grouped_static(p, p + 4096, p + 8192, p + 12288, None, big, C.BF16)
+        assert "fixed scratch array" in str(e.value)
+        # wider heads take proportionally more of the array: 16 rows of 64 heads of width 128 is the limit
+        with pytest.raises(C.Dispatch) as e:
+            gpu.attention_grouped_static(p, p + 4096, p + 8192, p + 12288, None,
+                                         C.GroupedShape(17, 1000, heads, kv_heads, 128, FULL, 2048, 0.125), C.BF16)
         assert "fixed scratch array" in str(e.value)
         ok = C.GroupedShape(1, 10, heads, kv_heads, dim, FULL, 11, 0.125)
         with pytest.raises(C.Dispatch):  # the reference's shape rules
