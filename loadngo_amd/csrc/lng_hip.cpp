@@ -621,7 +621,8 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     // (the matrix kernels take the maximum of the raw products and scale it afterwards: scale > 0; any other
     // scale goes to the kernels that scale first)
     const bool scale_positive = s.scale > 0.0f && s.scale <= 3.0e38f;
-    if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 && scale_positive &&
+    // (the prompt-pass kernels compare distances between positions as signed 32-bit numbers)
+    if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 && scale_positive && end <= 0x7fffffffull &&
         (dtype == LNG_BF16 || !getenv("LNG_F32_GENERIC"))) {
         const bool f32 = dtype == LNG_F32;
         lng_k_prefill p{};

@@ -2272,24 +2272,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     }
     __syncthreads();
 
-    // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
-    // carries no position arithmetic at all.
     // MODE 0: the running maximum is tracked. MODE 1: it is fixed (weights = 2^(score - m)). MODE 2: it is
     // fixed at zero (weights = 2^score: nothing but the exponential, the narrowing and the sum per score).
-    auto step = [&](auto mask_tag, auto mode_tag, uint32_t tile) {
+    // One block of 32 keys (kb = 0, 1 of a tile) for every head of the wavefront.
+    auto block = [&](auto mask_tag, auto mode_tag, uint32_t tile, int kb) {
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool FIXED = MODE != 0;
         const uint32_t buf = tile & 1u;
-        if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
-        if (wave_active) {
-            const uint32_t kt0 = tile0 + tile * PF_BN; // position of the tile's first key
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) { // the tile's two blocks of 32 keys
-                if constexpr (MASK && NH == 1) { // windows: a block no query of the workgroup sees (before the window, past the last row)
-                    const uint32_t b0 = kt0 + 32u * kb;
-                    if (b0 > pos_last || b0 + 31u < kfirst) continue;
-                }
+        const uint32_t kt0 = tile0 + tile * PF_BN; // position of the tile's first key
+            {
+                {
                 // ---- S^T = K . Q^T, both heads ------------------------------------------------------
                 bf16x8 ka[4];
 #pragma unroll
@@ -2310,14 +2303,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                 // V^T operands of this block: two groups of 16 keys x two halves of the head width;
                 // issued now, their LDS latency hides behind the softmax arithmetic
                 bf16x8 va[2][2];
+                auto read_v = [&]() {
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj) {
+                    for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-                    for (int db = 0; db < 2; ++db) {
-                        const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
-                        va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                        for (int db = 0; db < 2; ++db) {
+                            const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                            va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                        }
                     }
-                }
+                };
+                read_v();
                 // ---- online softmax, one query per lane -----------------------------------------------
                 // The running maximum only moves when the block's maximum exceeds it by PF_TAU (log2
                 // domain): weights then stay below 2^PF_TAU, and the accumulators are rescaled only
@@ -2327,14 +2323,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
 #pragma unroll
                 for (int h = 0; h < NH; ++h) {
                     if constexpr (MASK) {
+                        // key kp = kt0 + 32 kb + 4 hh + o_i is visible when 0 <= my_pos - kp < window, i.e. when the
+                        // constant o_i lies in (dist - window, dist]: two compares against per-block bounds
+                        const int dist = (int)(my_pos - (kt0 + 32u * kb + 4u * hh));
+                        const int below = windowed ? dist - (int)window : -0x40000000;
 #pragma unroll
                         for (int i = 0; i < 16; ++i) {
-                            const uint32_t kp = kt0 + 32u * kb + 8u * (i >> 2) + 4u * hh + (i & 3);
-                            const bool vis = kp <= my_pos && (!windowed || kp + window > my_pos);
-                            st[h][i] = vis ? st[h][i] : LNG_NEG_INF;
+                            const int o = 8 * (i >> 2) + (i & 3);
+                            st[h][i] = (o <= dist && o > below) ? st[h][i] : LNG_NEG_INF;
                         }
                     }
-                    float m_safe;
+                    float m_safe = 0.0f;
                     if constexpr (FIXED) {
                         m_safe = m[h]; // not -inf once frozen
                     } else {
@@ -2384,6 +2383,22 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                 }
             }
         }
+    };
+    // One tile step. Edge tiles (MASK) are a separate instantiation so that the interior loop
+    // carries no position arithmetic at all.
+    auto step = [&](auto mask_tag, auto mode_tag, uint32_t tile) {
+        const uint32_t buf = tile & 1u;
+        if (tile + 1 < n_tiles) fetch(tile + 1, kr, vr);
+        if (wave_active) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                if constexpr (decltype(mask_tag)::value && NH == 1) { // windows: a block no query of the workgroup sees
+                    const uint32_t b0 = tile0 + tile * PF_BN + 32u * kb;
+                    if (b0 > pos_last || b0 + 31u < kfirst) continue;
+                }
+                block(mask_tag, mode_tag, tile, kb);
+            }
+        }
         if (tile + 1 < n_tiles) stash(buf ^ 1u, kr, vr);
         __syncthreads();
     };
@@ -2397,6 +2412,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     using fixed_at_zero = std::integral_constant<int, 2>;
     uint32_t tile = first_tile;
     bool frozen = false;
+    {
     for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tracked{}, tile); // window edge
     if (optimistic) {                                                                      // interior
         bool at_zero = false;
@@ -2435,6 +2451,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         }
     } else {
         for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tracked{}, tile);
+    }
     }
     bool again = false;
     if (NH == 2 && frozen) { // frozen is uniform over the workgroup
@@ -2499,12 +2516,10 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             for (int db = 0; db < 2; ++db) {
 #pragma unroll
                 for (int blk = 0; blk < 4; ++blk) {
-                    ushort4 w;
-                    w.x = f32_to_bf16_bits(ot[h][db][4 * blk + 0] * inv);
-                    w.y = f32_to_bf16_bits(ot[h][db][4 * blk + 1] * inv);
-                    w.z = f32_to_bf16_bits(ot[h][db][4 * blk + 2] * inv);
-                    w.w = f32_to_bf16_bits(ot[h][db][4 * blk + 3] * inv);
-                    *(ushort4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
+                    bf16x4 w; // narrowed by the conversion instruction (round to nearest even)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) w[i] = (__bf16)(ot[h][db][4 * blk + i] * inv);
+                    *(bf16x4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
                 }
             }
         }

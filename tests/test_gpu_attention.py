@@ -387,6 +387,37 @@ def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sin
     assert np.abs(late - from_bf16_bits(vb)[spike_at][None, :, None, :].repeat(heads // kv_heads, 2).reshape(1, heads, 64)).max() < BF16_TOL
 
 
+@pytest.mark.parametrize("case", ["spike", "all_far_below", "all_far_above", "huge_sink", "usual"])
+@pytest.mark.parametrize("window,start", [(128, 0), (100, 777), (33, 64)])
+def test_windowed_prefill_with_scores_far_outside_the_usual_range(gpu, case, window, start):
+    """Passes under a window (one head per wavefront, the maximum tracked throughout) with a score near 10,000, with
+    every score of a row below -600 or above 600, with sinks of +-300: against the CPU reference, with and without
+    sinks."""
+    t, heads, kv_heads = 500, 16, 2
+    end = start + t
+    q, k, v, sinks = normal_inputs(5 + window, t, end, heads, kv_heads, 64, scale=0.5)
+    if case == "spike":
+        q[:] = np.abs(q) + 1.0
+        k[start + 300] = 30.0
+    elif case == "all_far_below":   # q . k about -64 * 1.4 * 9 * 8 * 0.125 = -800
+        q[:] = np.abs(q) + 1.0
+        k[:] = -np.abs(k) * 8.0 - 5.0
+    elif case == "all_far_above":
+        q[:] = np.abs(q) + 1.0
+        k[:] = np.abs(k) * 8.0 + 5.0
+    elif case == "huge_sink":
+        sinks[:] = 300.0
+        sinks[::3] = -300.0
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    slots = end
+    kr, vr = ring_layout(kb, t, start, slots, True), ring_layout(vb, t, start, slots, True)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    for sk in (sinks, None):
+        want = oracle.attention_bf16(qb, kb, vb, sk, start, window=window, scale=0.125, threads=THREADS)
+        got = run_attention(gpu, qb, kr, vr, sk, shape, True, C.BF16)
+        assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
 @pytest.mark.parametrize("t,start,heads,kv_heads,sinks_on", [
     (300, 0, 64, 8, True), (1000, 0, 32, 8, True), (777, 1300, 64, 8, False), (64, 0, 16, 2, True), (65, 63, 8, 1, True),
     (130, 4000, 24, 8, True), (2048, 0, 64, 8, True)])
