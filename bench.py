@@ -67,6 +67,49 @@ def stack_traffic_per_launch(ctx, batch):
     return rec.get("hbm_bytes_per_launch")
 
 
+def record_traffic(root, ctx, batch):
+    """Writes profiles/decode_stack_c5_hbm_traffic.json from four rocprofv3 counter runs under `root`:
+    pmc_c5_FETCH_SIZE, pmc_c5_WRITE_SIZE (this file with --no-extras --no-cpu) and pmc_copy_FETCH_SIZE,
+    pmc_copy_WRITE_SIZE (--only copy: a plain copy of 1 GiB, the yardstick each counter is scaled by).
+    The record carries a digest of the sources it was measured on; stack_traffic_per_launch ignores it
+    once they change."""
+    import csv
+    import glob
+
+    def per_dispatch(sub, kernel):
+        files = glob.glob(os.path.join(root, sub, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit("no counter_collection.csv under %s" % os.path.join(root, sub))
+        by_grid = {}
+        for row in csv.DictReader(open(files[0])):
+            if row["Kernel_Name"] == kernel:
+                by_grid.setdefault(int(row["Grid_Size"]), []).append(float(row["Counter_Value"]))
+        return {g: sum(v) / len(v) for g, v in by_grid.items()}
+
+    gib = float(1 << 30)
+    scale = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        seen = per_dispatch("pmc_copy_" + counter, "lng_copy_rows")
+        scale[counter] = gib / (max(seen.values()) * 1024.0)
+    total = 0.0
+    detail = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        for kernel in ("lng_decode_bf16_d64", "lng_decode_merge"):
+            for grid, kib in per_dispatch("pmc_c5_" + counter, kernel).items():
+                nbytes = kib * 1024.0 * scale[counter]
+                detail["%s grid %d %s" % (kernel, grid, counter)] = {"kib_per_dispatch": kib, "bytes": nbytes}
+                if kernel == "lng_decode_bf16_d64":
+                    total += nbytes / 2.0  # a step has 12 launches of each of the kernel's two grids: the mean over the 24
+    rec = {"ctx": ctx, "batch": batch, "sources_sha256": sources_digest(), "hbm_bytes_per_launch": round(total),
+           "scale_factor": scale, "per_dispatch": detail,
+           "how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per run) on `python3 bench.py --no-extras --no-cpu "
+                  "--steps 2 --warmup 1`, each scaled by what the counter reads for `python3 bench.py --only copy` (1 GiB in, 1 GiB out)"}
+    with open(TRAFFIC_RECORD, "w") as f:
+        json.dump(rec, f, indent=1)
+        f.write("\n")
+    print(json.dumps(rec, indent=1))
+
+
 METRIC = "decode attn GB/s (% HBM peak) + prefill attn TFLOP/s (% MFMA), gpt-oss shapes"
 
 
@@ -1014,10 +1057,15 @@ def main():
     ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block,wide: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--record-traffic", metavar="DIR", default="", help="no GPU work: turn the rocprofv3 counter runs under DIR "
+                    "(see record_traffic) into profiles/decode_stack_c5_hbm_traffic.json")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
         sys.exit(2)
+    if args.record_traffic:
+        record_traffic(args.record_traffic, args.ctx, args.batch)
+        return
     gpu = C.Gpu(0)
     log("device:", gpu.name())
     extra = {}
