@@ -100,7 +100,13 @@ def record_traffic(root, ctx, batch):
                 detail["%s grid %d %s" % (kernel, grid, counter)] = {"kib_per_dispatch": kib, "bytes": nbytes}
                 if kernel == "lng_decode_bf16_d64":
                     total += nbytes / 2.0  # a step has 12 launches of each of the kernel's two grids: the mean over the 24
-    rec = {"ctx": ctx, "batch": batch, "sources_sha256": sources_digest(), "hbm_bytes_per_launch": round(total),
+    try:  # the last commit that touched the measured sources (empty outside a git checkout)
+        import subprocess
+        commit = subprocess.run(["git", "-C", ROOT, "log", "-1", "--format=%H", "--"] + list(TRAFFIC_SOURCES),
+                                capture_output=True, text=True, timeout=20).stdout.strip()
+    except (OSError, subprocess.SubprocessError):
+        commit = ""
+    rec = {"ctx": ctx, "batch": batch, "sources_commit": commit, "sources_sha256": sources_digest(), "hbm_bytes_per_launch": round(total),
            "scale_factor": scale, "per_dispatch": detail,
            "how": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (one counter per run) on `python3 bench.py --no-extras --no-cpu "
                   "--steps 2 --warmup 1`, each scaled by what the counter reads for `python3 bench.py --only copy` (1 GiB in, 1 GiB out)"}
