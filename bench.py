@@ -1003,6 +1003,34 @@ def run_wide_heads(gpu, steps, warmup):
         out["%d_sequences" % n_seq] = res
         for b in (q, o, k, v):
             b.free()
+    # the reference's own element type at the same shape: 16 sequences of 16,384 positions (8.6 GB of f32 cache rows)
+    n_seq, ctx32 = 16, 16384
+    row32, qo32 = kv_heads * dim * 4, heads * dim * 4
+    q, o = gpu.buffer(n_seq * qo32), gpu.buffer(n_seq * qo32)
+    k, v = gpu.buffer(n_seq * ctx32 * row32), gpu.buffer(n_seq * ctx32 * row32)
+    for i, b in enumerate((q, k, v)):
+        bb = gpu.batch([b])
+        bb.fill_synthetic(C.Slice(0, 0, b.len), C.F32, 70 + i, 0.5, 0)
+        bb.run()
+        bb.drop()
+    items = C.decode_items([C.DecodeItem(i * qo32, i * qo32, i * ctx32 * row32, i * ctx32 * row32, 0, ctx32 - 1, C.FULL, ctx32)
+                            for i in range(n_seq)])
+
+    def go32():
+        batch = gpu.batch([q, k, v, o, sinks])
+        batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, scale, C.F32)
+        done = batch.run()
+        batch.drop()
+        return done.gpu_time
+
+    for _ in range(max(2, warmup)):
+        go32()
+    n = max(steps, 9)
+    t = sorted(go32() for _ in range(n))[n // 2]
+    nbytes = n_seq * (2 * ctx32 * row32 + 2 * qo32 + heads * 4)
+    out["f32_16_sequences_16384"] = {"bytes": nbytes, "gpu_us": t * 1e6, "gbs": nbytes / t / 1e9, "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
+    for b in (q, o, k, v):
+        b.free()
     sinks.free()
     return out
 

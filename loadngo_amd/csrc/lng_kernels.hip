@@ -1038,14 +1038,17 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_bf16_w256(lng_k_att
 extern "C" __global__ __launch_bounds__(256) void lng_decode_bf16_w512(lng_k_attn a) { decode_wide_bf16<8>(a); }
 
 // f32 (the reference's element type): lng_decode_f32_d64's products (v_mfma_f32_16x16x4_f32, V arriving transposed
-// straight from memory), a slice of 64 dimensions per batch of loads. The queries wait in LDS (16 heads x 512 floats
+// straight from memory), one or two slices of 64 dimensions per batch of loads. The queries wait in LDS (16 heads x 512 floats
 // would not fit the registers beside 128 accumulators).
 template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_attn &a) {
     __shared__ float s_m[4][16];
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
     __shared__ __attribute__((aligned(16))) float s_q[16][64 * DS + 4];
-    constexpr int NBATCH = 2 * DS;
+    constexpr int SB = DS == 4 ? 2 : 1; // slices per batch of loads (width 256: 512 contiguous bytes per row, 1.54 against 1.60 ms
+                                        // on 16 sequences of 16,384 positions; at width 512 two slices no longer fit the registers)
+    constexpr int KBATCH = DS / SB;                    // batches of K per tile, and as many of V
+    constexpr int NBATCH = 2 * KBATCH;
 
     const work_item wi = work_of(a);
     const uint32_t row = wi.pair / a.kv_heads;
@@ -1077,33 +1080,39 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
     __syncthreads();
 
     struct batch {
-        float4 k[2][4]; // K: [position half][dim step of the slice]
-    };                  // V reuses the 32 registers: [half][4 * i + mm] = position 4j + i, dim 16mm + n of the slice
+        float4 k[SB][2][4]; // K: [slice of the batch][position half][dim step of the slice]
+    };                      // V reuses the registers: [slice][half][i] = position 4j + i, .x .y .z .w = dims 16mm + n of the slice
     auto row_of_pos = [&](uint64_t p) -> uint64_t {
         p = p < first ? first : p;
         p = p > last ? last : p;
         return (wraps ? p % it.slots : p) * row_floats;
     };
     auto load_batch = [&](uint64_t tp, int b, batch &t) {
-        if (b < DS) {
+        if (b < KBATCH) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
-                const float *kp = kb + row_of_pos(tp + 16u * half + n) + 64 * b;
+                const float *kp = kb + row_of_pos(tp + 16u * half + n) + 64 * SB * b;
 #pragma unroll
-                for (int s = 0; s < 4; ++s) t.k[half][s] = *(const float4 *)(kp + 16 * s);
+                for (int u = 0; u < SB; ++u) {
+#pragma unroll
+                    for (int s = 0; s < 4; ++s) t.k[u][half][s] = *(const float4 *)(kp + 64 * u + 16 * s);
+                }
             }
         } else {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float *vp = vb + row_of_pos(tp + 16u * half + 4u * j + i) + 64 * (b - DS);
-                    float4 x;
-                    x.x = vp[0];
-                    x.y = vp[16];
-                    x.z = vp[32];
-                    x.w = vp[48];
-                    t.k[half][i] = x; // .x .y .z .w = dim blocks mm = 0..3
+                    const float *vp = vb + row_of_pos(tp + 16u * half + 4u * j + i) + 64 * SB * (b - KBATCH);
+#pragma unroll
+                    for (int u = 0; u < SB; ++u) {
+                        float4 x;
+                        x.x = vp[64 * u];
+                        x.y = vp[64 * u + 16];
+                        x.z = vp[64 * u + 32];
+                        x.w = vp[64 * u + 48];
+                        t.k[u][half][i] = x; // .x .y .z .w = dim blocks mm = 0..3
+                    }
                 }
             }
         }
@@ -1132,19 +1141,22 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
             } else if (more) {
                 load_batch(tp + 128u, 0, nxt);
             }
-            if (b < DS) {
+            if (b < KBATCH) {
 #pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const float4 qv = *(const float4 *)(&s_q[n][64 * b + 16 * s + 4 * j]);
+                for (int u = 0; u < SB; ++u) {
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].x, qv.x, st[half], 0, 0, 0);
-                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].y, qv.y, st[half], 0, 0, 0);
-                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].z, qv.z, st[half], 0, 0, 0);
-                        st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[half][s].w, qv.w, st[half], 0, 0, 0);
+                    for (int s = 0; s < 4; ++s) {
+                        const float4 qv = *(const float4 *)(&s_q[n][64 * (SB * b + u) + 16 * s + 4 * j]);
+#pragma unroll
+                        for (int half = 0; half < 2; ++half) {
+                            st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[u][half][s].x, qv.x, st[half], 0, 0, 0);
+                            st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[u][half][s].y, qv.y, st[half], 0, 0, 0);
+                            st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[u][half][s].z, qv.z, st[half], 0, 0, 0);
+                            st[half] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.k[u][half][s].w, qv.w, st[half], 0, 0, 0);
+                        }
                     }
                 }
-                if (b == DS - 1) {
+                if (b == KBATCH - 1) {
                     float tmax = LNG_NEG_INF;
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
@@ -1175,17 +1187,20 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
                     m = m_new;
                 }
             } else {
-                const int s = b - DS;
 #pragma unroll
-                for (int mm = 0; mm < 4; ++mm) {
-                    ot[s][mm] = ot[s][mm] * alpha;
+                for (int u = 0; u < SB; ++u) {
+                    const int s = SB * (b - KBATCH) + u;
 #pragma unroll
-                    for (int half = 0; half < 2; ++half) {
+                    for (int mm = 0; mm < 4; ++mm) {
+                        ot[s][mm] = ot[s][mm] * alpha;
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const float4 x = cur.k[half][i];
-                            const float vx = mm == 0 ? x.x : mm == 1 ? x.y : mm == 2 ? x.z : x.w;
-                            ot[s][mm] = __builtin_amdgcn_mfma_f32_16x16x4f32(vx, st[half][i], ot[s][mm], 0, 0, 0);
+                        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                const float4 x = cur.k[u][half][i];
+                                const float vx = mm == 0 ? x.x : mm == 1 ? x.y : mm == 2 ? x.z : x.w;
+                                ot[s][mm] = __builtin_amdgcn_mfma_f32_16x16x4f32(vx, st[half][i], ot[s][mm], 0, 0, 0);
+                            }
                         }
                     }
                 }
