@@ -42,6 +42,7 @@ MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X f32 matrix
 # WRITE_SIZE runs scaled by a 1 GiB copy; the figure and the sources it was measured on are kept in
 # profiles/decode_stack_c5_hbm_traffic.json and only reported while those sources are unchanged.
 TRAFFIC_RECORD = os.path.join(ROOT, "profiles", "decode_stack_c5_hbm_traffic.json")
+DECODE_KERNELS = ("lng_decode_bf16_d64", "lng_decode_bf16_d64_o4")
 TRAFFIC_SOURCES = ("loadngo_amd/csrc/lng_kernels.hip", "loadngo_amd/csrc/lng_hip.cpp", "loadngo_amd/csrc/lng_kernel_args.h")
 
 
@@ -94,11 +95,11 @@ def record_traffic(root, ctx, batch):
     total = 0.0
     detail = {}
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        for kernel in ("lng_decode_bf16_d64", "lng_decode_merge"):
+        for kernel in DECODE_KERNELS + ("lng_decode_merge",):
             for grid, kib in per_dispatch("pmc_c5_" + counter, kernel).items():
                 nbytes = kib * 1024.0 * scale[counter]
                 detail["%s grid %d %s" % (kernel, grid, counter)] = {"kib_per_dispatch": kib, "bytes": nbytes}
-                if kernel == "lng_decode_bf16_d64":
+                if kernel in DECODE_KERNELS:
                     total += nbytes / 2.0  # a step has 12 launches of each of the kernel's two grids: the mean over the 24
     try:  # the last commit that touched the measured sources (empty outside a git checkout)
         import subprocess
@@ -197,7 +198,10 @@ class Stack:
         done = batch.wait()
         if isinstance(done.gpu_time, Exception):
             raise done.gpu_time
-        ks = batch.kernel_seconds("lng_decode_bf16_d64") if timing else (0.0, 0)
+        ks = (0.0, 0)
+        if timing:  # both builds of the decode kernel (the second one serves dispatches of many short chunks: none in this stack)
+            per = [batch.kernel_seconds(name) for name in DECODE_KERNELS]
+            ks = (sum(p[0] for p in per), sum(p[1] for p in per))
         batch.drop()
         return done.gpu_time, ks
 

@@ -90,7 +90,7 @@ struct lng_gpu {
     hipModule_t module = nullptr;
     // kernels of the embedded code object
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
-    hipFunction_t decode_bf16_d64 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr, decode_merge_few = nullptr;
+    hipFunction_t decode_bf16_d64 = nullptr, decode_bf16_d64_o4 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr, decode_merge_few = nullptr;
     hipFunction_t decode_bf16_wide[3] = {}, decode_f32_wide[3] = {}; // head widths 128, 256, 512
     hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
@@ -536,8 +536,10 @@ int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *
         out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_wide[p.wide] : g->decode_f32_wide[p.wide],
                             p.kind == RowsPlan::Bf16 ? wide_bf16[p.wide] : wide_f32[p.wide], (unsigned)wgs, a};
     } else {
-        out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? g->decode_bf16_d64 : g->decode_f32_d64,
-                            p.kind == RowsPlan::Bf16 ? "lng_decode_bf16_d64" : "lng_decode_f32_d64", (unsigned)wgs, a};
+        // (many workgroups of short chunks - a table of sequences: the build of the bf16 kernel with four wavefronts per SIMD)
+        const bool o4 = p.kind == RowsPlan::Bf16 && a.chunk < 2048u && wgs > 3ull * g->cus && !getenv("LNG_DECODE_O3");
+        out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? (o4 ? g->decode_bf16_d64_o4 : g->decode_bf16_d64) : g->decode_f32_d64,
+                            p.kind == RowsPlan::Bf16 ? (o4 ? "lng_decode_bf16_d64_o4" : "lng_decode_bf16_d64") : "lng_decode_f32_d64", (unsigned)wgs, a};
     }
     if (a.n_chunks > 1 && !a.fused) {
         if (a.n_chunks <= 8 && !getenv("LNG_MERGE_WIDE")) { // a wavefront per (row, kv head, query head), four to a workgroup
@@ -780,6 +782,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_attn_generic_f32", &g->generic_f32, true},
         {"lng_attn_generic_bf16", &g->generic_bf16, true},
         {"lng_decode_bf16_d64", &g->decode_bf16_d64, true},
+        {"lng_decode_bf16_d64_o4", &g->decode_bf16_d64_o4, true},
         {"lng_decode_merge", &g->decode_merge, true},
         {"lng_decode_merge_few", &g->decode_merge_few, true},
         {"lng_decode_f32_d64", &g->decode_f32_d64, true},

@@ -389,7 +389,7 @@ struct kv_tile {
     uint4 v[2][2];
 };
 
-extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_attn a) {
+__device__ __forceinline__ void decode_bf16_d64_body(const lng_k_attn a) {
     __shared__ float s_m[4][16];
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
@@ -596,6 +596,13 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_a
 
     merge_chunks<true>(a, it, wi.pair, g, group, row_chunks);
 }
+
+// Two builds of the same body: 130 registers and three wavefronts per SIMD for long chunks (what a long context
+// streams best with), 125 registers and four for dispatches of many workgroups with chunks under 2,048 positions
+// (a table of sequences), where workgroups are short-lived and a fourth one per compute unit hides more of their
+// start-up (32 sequences 65 -> 62 us, 128 sequences 243 -> 236 us; on 4,096-position chunks it is 1.7 % slower).
+extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_bf16_d64(lng_k_attn a) { decode_bf16_d64_body(a); }
+extern "C" __global__ __launch_bounds__(256, 4) void lng_decode_bf16_d64_o4(lng_k_attn a) { decode_bf16_d64_body(a); }
 
 // =============================================================================================
 // Decode kernel, f32 (the reference's own element type), head width 64, up to 16 query heads per
@@ -813,7 +820,7 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
 // Callers: the reference's other user of this operator has 32 heads over 16 kv heads of width 256
 // (decider/src/gpu.rs:878-893), its own tests go to width 512 (attention_grouped.rs:187-199).
 // =============================================================================================
-template <int DS> __device__ __forceinline__ void decode_wide_bf16(const lng_k_attn &a) {
+template <int DS> __device__ __forceinline__ void decode_wide_bf16(const lng_k_attn a) {
     __shared__ float s_m[4][16];
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
@@ -1040,7 +1047,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_bf16_w512(lng_k_att
 // f32 (the reference's element type): lng_decode_f32_d64's products (v_mfma_f32_16x16x4_f32, V arriving transposed
 // straight from memory), one or two slices of 64 dimensions per batch of loads. The queries wait in LDS (16 heads x 512 floats
 // would not fit the registers beside 128 accumulators).
-template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_attn &a) {
+template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_attn a) {
     __shared__ float s_m[4][16];
     __shared__ float s_l[4][16];
     __shared__ float s_o[4][16][65];
