@@ -15,6 +15,7 @@
 //!   f32 accumulation; sinks stay f32).
 //!
 //! Additions without a counterpart in metal-compute are grouped at the end of `impl Batch`.
+#![warn(unsafe_op_in_unsafe_fn)]
 
 pub mod ffi;
 
