@@ -159,6 +159,53 @@ def test_many_small_decodes_merged_inside_the_kernel(gpu):
         b.free()
 
 
+@pytest.mark.parametrize("dtype,dim,heads,kv_heads", [(C.BF16, 64, 64, 8), (C.F32, 64, 16, 8), (C.BF16, 128, 16, 8)])
+def test_a_table_of_many_short_sequences_takes_the_small_merge_and_the_four_wavefront_build(gpu, dtype, dim, heads, kv_heads):
+    """160 sequences of 300..2,400 positions in one dispatch: rows of two to seven chunks, several thousand
+    workgroups, merged by the second dispatch (lng_decode_merge_few; the per-kernel times say which kernels ran),
+    each sequence against the CPU reference on its own cache."""
+    n_seq = 160
+    rng = np.random.default_rng(160 + dim)
+    lens = rng.integers(300, 2401, size=n_seq)
+    offs = np.concatenate([[0], np.cumsum(lens)])
+    es = 2 if dtype == C.BF16 else 4
+    row = kv_heads * dim
+    scale = float(1.0 / np.sqrt(np.float32(dim)))
+    k_all = rng.standard_normal((int(offs[-1]), kv_heads, dim), dtype=np.float32) * np.float32(0.7)
+    v_all = rng.standard_normal((int(offs[-1]), kv_heads, dim), dtype=np.float32)
+    q = rng.standard_normal((n_seq, heads, dim), dtype=np.float32) * np.float32(0.7)
+    sinks = rng.standard_normal(heads).astype(np.float32)
+    if dtype == C.BF16:
+        q, k_all, v_all = to_bf16_bits(q), to_bf16_bits(k_all), to_bf16_bits(v_all)
+    bufs = [gpu.upload(q), gpu.upload(k_all), gpu.upload(v_all), gpu.buffer(q.size * es), gpu.upload(sinks)]
+    bufs[3].fill(0xFF)
+    items = [C.DecodeItem(i * heads * dim * es, i * heads * dim * es, int(offs[i]) * row * es, int(offs[i]) * row * es, 0,
+                          int(n) - 1, C.FULL, int(n)) for i, n in enumerate(lens)]
+    batch = gpu.batch(bufs)
+    try:
+        batch.set_timing(True)
+        batch.attention_decode_batched(0, 1, 2, 3, 4, items, heads, kv_heads, dim, scale, dtype)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        assert batch.kernel_seconds("lng_decode_merge_few")[1] == 1
+        if dtype == C.BF16 and dim == 64:
+            assert batch.kernel_seconds("lng_decode_bf16_d64_o4")[1] == 1
+        out = bufs[3].read(np.uint16 if dtype == C.BF16 else np.float32).reshape(n_seq, heads, dim)
+    finally:
+        batch.drop()
+        for b in bufs:
+            b.free()
+    for i in range(0, n_seq, 7):
+        ks, vs = k_all[offs[i]:offs[i + 1]], v_all[offs[i]:offs[i + 1]]
+        if dtype == C.BF16:
+            want = from_bf16_bits(orc.attention_bf16(q[i:i + 1], ks, vs, sinks, int(lens[i]) - 1, scale=scale, threads=THREADS))
+            assert np.abs(from_bf16_bits(out[i:i + 1]) - want).max() < 2e-2, i
+        else:
+            want = orc.attention_f32(q[i:i + 1], ks, vs, sinks, int(lens[i]) - 1, scale=scale, threads=THREADS)
+            err = np.abs(out[i:i + 1].astype(np.float64) - want) / (np.abs(want) + 1.0)
+            assert err.max() <= 1e-5, i
+
+
 def test_buffers_outlive_a_closed_gpu():
     """Closing a gpu whose buffers are still alive leaves them valid to free (they share the device the way the
     reference's buffers share theirs); the device goes with the last of them."""
