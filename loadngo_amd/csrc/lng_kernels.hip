@@ -2877,79 +2877,88 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
             buf = nxt;
         };
 
-        // ---- the interior tiles with the maximum fixed at zero, as a software pipeline ----------------------
-        // Unit = (block of 32 keys, one head): four matrix instructions of scores, 32 arithmetic instructions
-        // (16 exponentials, 8 narrowings, 8 sums), four matrix instructions of values. While a unit's arithmetic
-        // issues, the matrix unit runs the NEXT unit's scores and the PREVIOUS unit's values, one matrix
-        // instruction in front of every four arithmetic ones, so neither pipe waits for the other inside a
-        // wavefront (the plain tile issues eight score products back to back, waits for them, and only then
-        // starts on the exponentials). The next tile is visible one tile early (three buffers), so the pipeline
-        // runs across the tile barrier: the scores of the next tile's first unit are under way before it.
+        // ---- the interior tiles with the maximum fixed at zero: matrix and arithmetic phases, the two wavefronts
+        // of a SIMD one phase apart ----------------------------------------------------------------------------
+        // Per block of 32 keys a wavefront (two heads) has a MATRIX phase - the 8 score products of the block, the 8
+        // value products and 4 normaliser products of the block before, then the LDS reads of the next operands -
+        // and an ARITHMETIC phase - 32 exponentials and 16 narrowings, nothing else. A wavefront that issues both
+        // kinds side by side overlaps them only partly on this part, and two wavefronts that are in the same phase
+        // at the same time share one pipe while the other idles; a wavefront in its matrix phase beside one in its
+        // arithmetic phase keeps both busy. The tile barrier would put all wavefronts in the same phase, so the
+        // second wavefront of every SIMD (w + 4) passes it one phase earlier in its own sequence: after the second
+        // matrix phase of the tile, where the first passes it after the second arithmetic phase. Both make the
+        // same phases in the same order and pass one barrier per tile.
+        // LDS: every read of a tile's buffer is issued before the barrier that ends the tile (the late wavefronts
+        // have read the second block's V operands and the next tile's first K operands by then); the buffer is
+        // written again two tiles later. K/V rows are asked for a whole tile before they are stored to LDS: a
+        // barrier waits for the slowest load of 512 threads.
         auto pipe = [&](uint32_t &tile) {
-            floatx16 st_cur;          // scores of the coming unit (first block of keys, first head)
-            bf16x8 pb_prev[2];        // weights of the last finished unit, their value product pending
-            bf16x8 va_prev[2][2];     // and its V^T operands
+            const bool late = wave >= 4u;
+            floatx16 st[NH];
+            bf16x8 pb[NH][2];   // weights of the last block, their value products pending
+            // The normaliser is summed by the matrix unit as well: the weights of 16 keys x 32 queries, as they lie in
+            // registers for the value product (lane = query n, half hh = keys 8hh..8hh+7), read as the B operand of a
+            // 16x16x32 product are 16 columns x 32 slots, column c holding query c in slots 0-7 and 16-23 and query
+            // c + 16 in slots 8-15 and 24-31. An A operand with ones in row 0 at the first and row 1 at the second set of
+            // slots leaves the sums of queries c and c + 16 in rows 0 and 1 of column c: lanes 0..15, registers 0 and 1.
+            floatx4 lacc[NH];
+#pragma unroll
+            for (int h = 0; h < NH; ++h) lacc[h] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+            // (built where it is used, from a lane mask: four registers that would otherwise be spilled and reloaded
+            // in the loop, and a reload there waits for the K/V loads in flight)
+            auto selector = [&]() {
+                uint32_t z = 0u;
+                asm volatile("" : "+v"(z)); // not a loop invariant: nothing of this is kept in a register between uses
+                const uint32_t l31 = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z)) & 31u;
+                const uint32_t w = (l31 == 0u || l31 == 17u) ? 0x3f803f80u : 0u; // rows 0 / 1 at slot groups 0, 2 / 1, 3
+                return as_bf16x8(make_uint4(w, w, w, w));
+            };
+            bf16x8 va[2][2];    // and its V^T operands
             auto zero16 = [&]() {
                 floatx16 z;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) z[i] = 0.0f;
                 return z;
             };
-            // one unit: `sc` -> weights `pw` (and the running sum), with score products (kq . qq -> so) and value
-            // products (vz . pz -> oz) of its neighbours in between
-            auto unit = [&](floatx16 &sc, float &lsum, const bf16x8 (&kq)[4], const bf16x8 (&qq)[4], floatx16 &so,
-                            const bf16x8 (&vz)[2][2], const bf16x8 (&pz)[2], floatx16 (&oz)[2], bf16x8 (&pw)[2]) {
-                float ps0 = 0.0f, ps1 = 0.0f;
-                bf16x2 pr[8];
-                __builtin_amdgcn_sched_barrier(0);
-                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[0], qq[0], zero16(), 0, 0, 0);
+            // nothing pending yet: weights of zero against any finite operands
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
-                __builtin_amdgcn_sched_barrier(0);
-                oz[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[0][0], pz[0], oz[0], 0, 0, 0);
+            for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-                for (int i = 4; i < 8; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
-                __builtin_amdgcn_sched_barrier(0);
-                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[1], qq[1], so, 0, 0, 0);
+                for (int h = 0; h < NH; ++h) {
 #pragma unroll
-                for (int i = 8; i < 12; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
-                __builtin_amdgcn_sched_barrier(0);
-                oz[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[0][1], pz[0], oz[1], 0, 0, 0);
+                    for (int e = 0; e < 8; ++e) pb[h][jj][e] = (__bf16)0.0f;
+                }
 #pragma unroll
-                for (int i = 12; i < 16; ++i) sc[i] = __builtin_amdgcn_exp2f(sc[i]);
+                for (int db = 0; db < 2; ++db) va[jj][db] = pb[0][jj];
+            }
+            // matrix phase of block kb of the tile in `b`: scores of the block, values and weight sums of the block
+            // before, then the operands of the next matrix phase (K of the next block, V of this one)
+            auto matrix = [&](uint32_t b, uint32_t b_next, int kb) {
+                const bf16x8 sel = selector();
                 __builtin_amdgcn_sched_barrier(0);
-                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[2], qq[2], so, 0, 0, 0);
+                st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[0], qreg[0][0], zero16(), 0, 0, 0);
+                st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[0], qreg[1][0], zero16(), 0, 0, 0);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    pr[e][0] = (__bf16)sc[2 * e];
-                    pr[e][1] = (__bf16)sc[2 * e + 1];
+                for (int ks = 1; ks < 4; ++ks) {
+                    st[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[ks], qreg[0][ks], st[0], 0, 0, 0);
+                    st[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[ks], qreg[1][ks], st[1], 0, 0, 0);
+                }
+#pragma unroll
+                for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) {
+                        ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[0][jj], ot[0][db], 0, 0, 0);
+                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
+                    }
+                    lacc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sel, pb[0][jj], lacc[0], 0, 0, 0);
+                    lacc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sel, pb[1][jj], lacc[1], 0, 0, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                oz[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[1][0], pz[1], oz[0], 0, 0, 0);
-#pragma unroll
-                for (int e = 4; e < 8; ++e) {
-                    pr[e][0] = (__bf16)sc[2 * e];
-                    pr[e][1] = (__bf16)sc[2 * e + 1];
+                if (kb + 1 < KB) {
+                    read_k(b, kb + 1, ka0);
+                } else {
+                    read_k(b_next, 0, ka0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                so = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kq[3], qq[3], so, 0, 0, 0);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) ps0 = __builtin_amdgcn_fdot2_f32_bf16(pr[e], ones2, ps0, false);
-                __builtin_amdgcn_sched_barrier(0);
-                oz[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vz[1][1], pz[1], oz[1], 0, 0, 0);
-#pragma unroll
-                for (int e = 4; e < 8; ++e) ps1 = __builtin_amdgcn_fdot2_f32_bf16(pr[e], ones2, ps1, false);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    pw[0][2 * e] = pr[e][0];
-                    pw[0][2 * e + 1] = pr[e][1];
-                    pw[1][2 * e] = pr[4 + e][0];
-                    pw[1][2 * e + 1] = pr[4 + e][1];
-                }
-                lsum += ps0 + ps1;
-            };
-            auto read_v = [&](uint32_t b, int kb, bf16x8 (&va)[2][2]) {
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
@@ -2958,57 +2967,83 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                         va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             };
-            if (wave_active) {
-                // nothing pending yet: weights of zero against any finite operands
+            // (the empty asm statements keep the phase where it is written: its arithmetic has no side effects, and
+            // the compiler would otherwise move parts of it behind the matrix phase and the barrier that follow)
+            auto arithmetic = [&]() {
 #pragma unroll
-                for (int jj = 0; jj < 2; ++jj) {
+                for (int h = 0; h < NH; ++h) asm volatile("" : "+v"(st[h]));
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) pb_prev[jj][e] = (__bf16)0.0f;
+                for (int h = 0; h < NH; ++h) {
 #pragma unroll
-                    for (int db = 0; db < 2; ++db) va_prev[jj][db] = pb_prev[jj];
-                }
-                st_cur = zero16();
+                    for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) st_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka0[ks], qreg[0][ks], st_cur, 0, 0, 0);
-            }
-            for (; tile < n_interior; ++tile) {
-                const uint32_t nxt = buf == 2u ? 0u : buf + 1u;
-                const uint32_t after = nxt == 2u ? 0u : nxt + 1u;
-                fetch(tile + 2, kr, vr);
-                if (wave_active) {
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb) {
-                        bf16x8 kan[4], va[2][2], pbA[2];
-                        floatx16 stB;
-                        if (kb + 1 < KB) {
-                            read_k(buf, kb + 1, kan);
-                        } else {
-                            read_k(nxt, 0, kan);
+                        for (int e = 0; e < 8; e += 2) {
+                            const float p0 = __builtin_amdgcn_exp2f(st[h][8 * jj + e]);
+                            const float p1 = __builtin_amdgcn_exp2f(st[h][8 * jj + e + 1]);
+                            pb[h][jj][e] = (__bf16)p0;
+                            pb[h][jj][e + 1] = (__bf16)p1;
                         }
-                        read_v(buf, kb, va);
-                        unit(st_cur, l[0], ka0, qreg[1], stB, va_prev, pb_prev, ot[1], pbA);  // (block kb, head 0)
-                        unit(stB, l[1], kan, qreg[0], st_cur, va, pbA, ot[0], pb_prev);        // (block kb, head 1)
-#pragma unroll
-                        for (int jj = 0; jj < 2; ++jj) {
-#pragma unroll
-                            for (int db = 0; db < 2; ++db) va_prev[jj][db] = va[jj][db];
-                        }
-#pragma unroll
-                        for (int ks = 0; ks < 4; ++ks) ka0[ks] = kan[ks];
                     }
                 }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) asm volatile("" : "+v"(pb[h][0]), "+v"(pb[h][1]));
+            };
+            auto publish = [&](uint32_t after) { // the tile after next goes to LDS, the one after that is asked for; the tile ends
                 stash(after, kr, vr);
-                __syncthreads();
-                buf = nxt;
+                fetch(tile + 3, kr, vr); // a whole tile before it is stored (past the last tile: its rows again, never stored)
+                __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+                __builtin_amdgcn_s_barrier();
+            };
+            fetch(tile + 2, kr, vr);
+            auto loop = [&](auto active_tag) {
+                constexpr bool ACTIVE = decltype(active_tag)::value;
+                for (; tile < n_interior; ++tile) {
+                    const uint32_t nxt = buf == 2u ? 0u : buf + 1u;
+                    const uint32_t after = nxt == 2u ? 0u : nxt + 1u;
+                    if constexpr (ACTIVE) {
+#pragma unroll
+                        for (int kb = 0; kb + 1 < KB; ++kb) {
+                            matrix(buf, nxt, kb);
+                            arithmetic();
+                        }
+                        matrix(buf, nxt, KB - 1);
+                        if (late) publish(after);
+                        arithmetic();
+                        if (!late) publish(after);
+                    } else {
+                        publish(after);
+                    }
+                    buf = nxt;
+                }
+            };
+            if (wave_active) {
+                loop(std::true_type{});
+            } else {
+                loop(std::false_type{});
             }
-            if (wave_active) { // the last unit's values; the scores under way belong to the tile that follows
+            if (wave_active) { // the last block's values
+                const bf16x8 sel = selector();
 #pragma unroll
                 for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                     for (int db = 0; db < 2; ++db) {
-                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va_prev[jj][db], pb_prev[jj], ot[1][db], 0, 0, 0);
+                        ot[0][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[0][jj], ot[0][db], 0, 0, 0);
+                        ot[1][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[1][jj], ot[1][db], 0, 0, 0);
                     }
+                    lacc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sel, pb[0][jj], lacc[0], 0, 0, 0);
+                    lacc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sel, pb[1][jj], lacc[1], 0, 0, 0);
+                }
+                // query n's sum is in lane n % 16, register n / 16; l[] is per (query, half) and the halves are added
+                // at the end, so the whole of it goes to the first half
+#pragma unroll
+                for (int h = 0; h < NH; ++h) {
+                    const float lo = __shfl(lacc[h][0], (int)(n & 15u), 64);
+                    const float hi = __shfl(lacc[h][1], (int)(n & 15u), 64);
+                    if (hh == 0u) l[h] += n < 16u ? lo : hi;
                 }
             }
         };
