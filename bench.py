@@ -529,10 +529,18 @@ def run_prefill(gpu, steps, warmup, t=8192):
 
         for _ in range(max(warmup, 5)):
             go()
+        # after idle the clocks take tens of milliseconds of continuous work to settle (the first launches of a
+        # pass run 15-30 % slower than the hundredth): batches of 20 launches until the time per launch stops falling
+        last = go(20)
+        for _ in range(12):
+            cur = go(20)
+            if cur > 0.99 * last:
+                break
+            last = cur
         runs = sorted(go() for _ in range(max(steps, 20)))
         g = runs[len(runs) // 2]
         go(20)
-        sustained = sorted(go(20) for _ in range(5))[2]  # 20 launches back to back: no gap before each kernel, steady clocks
+        sustained = sorted(go(20) for _ in range(5))[2]  # 20 launches back to back: no gap before each kernel
         traffic = 2 * t * QO + 2 * t * ROW
         res[name] = {"pairs": pairs, "flops": flops, "gpu_ms": g * 1e3, "tflops": flops / g / 1e12,
                      "mfma_frac": flops / g / 1e12 / MFMA_BF16_PEAK_TFLOPS,

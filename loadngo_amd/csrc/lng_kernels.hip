@@ -2342,6 +2342,20 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     // with the maximum tracked throughout.
     constexpr int ATTEMPTS = NH == 2 ? 2 : 1;
     uint4 kr, vr;
+    // With the maximum fixed the normaliser needs no rescaling, and the matrix unit sums it: the weights of 16 keys
+    // x 32 queries as they lie in registers for the value product, read as the B operand of a 16x16x32 product, are
+    // 16 columns x 32 slots, column c holding query c in slots 0-7 and 16-23 and query c + 16 in slots 8-15 and
+    // 24-31; an A operand of ones in row 0 at the first and in row 1 at the second set of slots leaves the two sums
+    // in rows 0 and 1 of column c (lanes 0..15, registers 0 and 1). (The sum instruction of the vector unit,
+    // v_dot2c_f32_bf16, runs at two fifths of its rate beside another wavefront's matrix instructions.)
+    floatx4 lacc[NH];
+    auto selector = [&]() { // built where it is used: four registers less to keep (or spill) across the loops
+        uint32_t z = 0u;
+        asm volatile("" : "+v"(z));
+        const uint32_t l31 = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z)) & 31u;
+        const uint32_t w = (l31 == 0u || l31 == 17u) ? 0x3f803f80u : 0u;
+        return as_bf16x8(make_uint4(w, w, w, w));
+    };
     for (int attempt = 0; attempt < ATTEMPTS; ++attempt) {
     const bool optimistic = NH == 2 && attempt == 0;
 #pragma unroll
@@ -2349,6 +2363,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         const bool sink_here = a.sinks && !partial;
         m[h] = sink_here ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
         l[h] = (sink_here && hh == 0) ? 1.0f : 0.0f;
+        lacc[h] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
 #pragma unroll
@@ -2456,10 +2471,18 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                             pb[h][jj][e] = pr[0];
                             pb[h][jj][e + 1] = pr[1];
                             // the normaliser sums the same rounded weights the product uses
-                            psum[jj] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum[jj], false);
+                            if constexpr (!FIXED) psum[jj] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum[jj], false);
                         }
                     }
-                    l[h] += psum[0] + psum[1];
+                    if constexpr (!FIXED) l[h] += psum[0] + psum[1];
+                }
+                if constexpr (FIXED) {
+                    const bf16x8 sel = selector();
+#pragma unroll
+                    for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) lacc[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(sel, pb[h][jj], lacc[h], 0, 0, 0);
+                    }
                 }
                 // ---- O^T += V^T . P^T ---------------------------------------------------------------------
 #pragma unroll
@@ -2544,6 +2567,16 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     }
     bool again = false;
     if (NH == 2 && frozen) { // frozen is uniform over the workgroup
+        if (wave_active) {
+            // query n's sum is in lane n % 16, register n / 16; l[] is per (query, half) and the halves are added at
+            // the end, so the whole of it goes to the first half
+#pragma unroll
+            for (int h = 0; h < NH; ++h) {
+                const float lo = __shfl(lacc[h][0], (int)(n & 15u), 64);
+                const float hi = __shfl(lacc[h][1], (int)(n & 15u), 64);
+                if (hh == 0u) l[h] += n < 16u ? lo : hi;
+            }
+        }
         int bad = 0;
         if (wave_active) {
 #pragma unroll
