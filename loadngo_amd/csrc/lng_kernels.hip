@@ -3134,6 +3134,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                 }
                 if (at_zero) {
                     pipe(tile);
+                    // the diagonal at the same fixed reference point (a masked score is 2^-inf = 0), before the check
+                    for (; tile < n_tiles; ++tile) step(std::true_type{}, fixed_at_zero{}, tile);
                 } else {
                     for (; tile < n_interior; ++tile) step(std::false_type{}, fixed_at_m{}, tile);
                 }
@@ -3160,7 +3162,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                 again = __syncthreads_or(bad) != 0;
             }
             if (!again) {
-                for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile); // the diagonal
+                for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile); // the diagonal, where not done yet
                 break;
             }
         }
@@ -3177,12 +3179,10 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                 for (int db = 0; db < 2; ++db) {
 #pragma unroll
                     for (int blk = 0; blk < 4; ++blk) {
-                        ushort4 w;
-                        w.x = f32_to_bf16_bits(ot[h][db][4 * blk + 0] * inv);
-                        w.y = f32_to_bf16_bits(ot[h][db][4 * blk + 1] * inv);
-                        w.z = f32_to_bf16_bits(ot[h][db][4 * blk + 2] * inv);
-                        w.w = f32_to_bf16_bits(ot[h][db][4 * blk + 3] * inv);
-                        *(ushort4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
+                        bf16x4 w; // narrowed by the conversion instruction (round to nearest even)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) w[i] = (__bf16)(ot[h][db][4 * blk + i] * inv);
+                        *(bf16x4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
                     }
                 }
             }
