@@ -423,7 +423,8 @@ def test_windowed_prefill_with_scores_far_outside_the_usual_range(gpu, case, win
     (130, 4000, 24, 8, True), (2048, 0, 64, 8, True)])
 def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, start, heads, kv_heads, sinks_on, monkeypatch):
     """lng_prefill_bf16_d64_stream (one resident workgroup per compute unit, query tiles dealt out in a snake,
-    K/V tiles through three LDS buffers, the interior as a software pipeline): forced for shapes of every kind it
+    K/V tiles through three LDS buffers, the interior in matrix and arithmetic phases with the second wavefront of
+    every SIMD one phase behind and the normaliser summed by the matrix unit): forced for shapes of every kind it
     takes - a ragged last query tile, positions before the pass, groups that leave wavefronts without a head, fewer
     query tiles than workgroups, no sinks - against the CPU reference, and against the kernel with one workgroup
     per query tile (LNG_PREFILL_STREAM=0), which runs the same arithmetic tile for tile."""
