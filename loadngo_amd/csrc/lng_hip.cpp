@@ -467,10 +467,10 @@ RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, 
     const bool dim_ok = a.dim == 64 || (wide >= 0 && !getenv("LNG_WIDE_GENERIC"));
     const bool fast = a.dtype == LNG_BF16 && dim_ok && group <= 16 && aligned16;
     // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the f32 matrix instruction
-    // (that kernel counts positions in 32 bits and looks up to 63 past the last one)
+    // (that kernel counts positions in 32 bits and steps by up to 256 chunks x 128 positions past the last one)
     uint64_t latest = t_uniform ? host_rows[0].start + t_uniform - 1 : 0;
     for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
-    const bool fast_f32 = a.dtype == LNG_F32 && dim_ok && group <= 16 && aligned16 && latest < 0xffffff00ull &&
+    const bool fast_f32 = a.dtype == LNG_F32 && dim_ok && group <= 16 && aligned16 && latest < 0xffff0000ull &&
                           a.scale > 0.0f && a.scale <= 3.0e38f && !getenv("LNG_F32_GENERIC");
     p.pairs = n_rows * (size_t)a.kv_heads;
     if (!fast && !fast_f32) return p;

@@ -401,10 +401,14 @@ __device__ __forceinline__ void decode_bf16_d64_body(const lng_k_attn a) {
     const uint64_t last = it.start;
     const uint64_t first = first_visible(last, it.window);
     const uint64_t base = first & ~(uint64_t)31;
-    const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
-    if (c0 > last) return; // this row has fewer chunks than the longest one
-    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+    if (wi.chunk >= row_chunks) return; // this row has fewer chunks than the longest one
+    // The row's workgroups take interleaved groups of 128 positions (workgroup c: groups c, c + chunks, ...), not
+    // a run of a.chunk positions each: together they sweep one window of the row, and every workgroup of a row
+    // has the same number of groups to within one, however the row's length divides.
+    const uint64_t c0 = base + (uint64_t)wi.chunk * 128u;
+    const uint64_t c1 = last + 1;
+    const uint64_t tile_stride = 128ull * row_chunks;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = threadIdx.x >> 6;
@@ -465,8 +469,8 @@ __device__ __forceinline__ void decode_bf16_d64_body(const lng_k_attn a) {
     kv_tile cur, nxt;
     uint64_t tp = c0 + (uint64_t)wave * 32u;
     if (tp < c1) load_tile(tp, cur);
-    for (; tp < c1; tp += 128u) {
-        const uint64_t tn = tp + 128u;
+    for (; tp < c1; tp += tile_stride) {
+        const uint64_t tn = tp + tile_stride;
         if (tn < c1) load_tile(tn, nxt);
 
         floatx4 st[2];
@@ -639,11 +643,13 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
     const uint32_t last = (uint32_t)it.start;
     const uint32_t first = (uint32_t)first_visible(it.start, it.window);
     const uint32_t base = first & ~31u;
-    const uint64_t c0w = (uint64_t)base + (uint64_t)wi.chunk * a.chunk;
-    if (c0w > last) return; // this row has fewer chunks than the longest one
-    const uint32_t c0 = (uint32_t)c0w;
-    const uint32_t c1 = (c0w + a.chunk < (uint64_t)last + 1u) ? (uint32_t)(c0w + a.chunk) : last + 1u; // last + 1 fits: last < 2^32 - 1 here or the chunk ends earlier
     const uint32_t row_chunks = (uint32_t)(((uint64_t)last + 1u - base + a.chunk - 1u) / a.chunk);
+    if (wi.chunk >= row_chunks) return; // this row has fewer chunks than the longest one
+    // interleaved groups of 128 positions, as in the bf16 kernel; the host keeps last below 2^32 - 65,536, so
+    // neither last + 1 nor a position plus the stride (at most 256 chunks x 128) leaves 32 bits
+    const uint32_t c0 = base + wi.chunk * 128u;
+    const uint32_t c1 = last + 1u;
+    const uint32_t tile_stride = 128u * row_chunks;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -703,8 +709,8 @@ extern "C" __global__ __launch_bounds__(256, 2) void lng_decode_f32_d64(lng_k_at
     kv_tile_f32 cur, nxt;
     uint32_t tp = c0 + wave * 32u;
     if (tp < c1) load_tile(tp, cur);
-    for (; tp < c1; tp += 128u) {
-        if (c1 - tp > 128u) load_tile(tp + 128u, nxt);
+    for (; tp < c1; tp += tile_stride) {
+        if (c1 - tp > tile_stride) load_tile(tp + tile_stride, nxt);
 
         floatx4 st[2];
 #pragma unroll
@@ -835,6 +841,8 @@ template <int DS> __device__ __forceinline__ void decode_wide_bf16(const lng_k_a
     const uint64_t last = it.start;
     const uint64_t first = first_visible(last, it.window);
     const uint64_t base = first & ~(uint64_t)31;
+    // (a run of a.chunk positions per workgroup: with 256 bytes and more per position and kv head the interleaved
+    // groups of the head-width-64 kernel measured 4-5 % slower here)
     const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
     if (c0 > last) return;
     const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
@@ -1064,10 +1072,14 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
     const uint64_t last = it.start;
     const uint64_t first = first_visible(last, it.window);
     const uint64_t base = first & ~(uint64_t)31;
-    const uint64_t c0 = base + (uint64_t)wi.chunk * a.chunk;
-    if (c0 > last) return;
-    const uint64_t c1 = (c0 + a.chunk < last + 1) ? c0 + a.chunk : last + 1;
     const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk);
+    if (wi.chunk >= row_chunks) return; // this row has fewer chunks than the longest one
+    // The row's workgroups take interleaved groups of 128 positions (workgroup c: groups c, c + chunks, ...), not
+    // a run of a.chunk positions each: together they sweep one window of the row, and every workgroup of a row
+    // has the same number of groups to within one, however the row's length divides.
+    const uint64_t c0 = base + (uint64_t)wi.chunk * 128u;
+    const uint64_t c1 = last + 1;
+    const uint64_t tile_stride = 128ull * row_chunks;
 
     const uint32_t lane = threadIdx.x & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1137,8 +1149,8 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
     batch cur, nxt;
     uint64_t tp = c0 + (uint64_t)wave * 32u;
     if (tp < c1) load_batch(tp, 0, cur);
-    for (; tp < c1; tp += 128u) {
-        const bool more = tp + 128u < c1;
+    for (; tp < c1; tp += tile_stride) {
+        const bool more = tp + tile_stride < c1;
         floatx4 st[2] = {(floatx4){0.f, 0.f, 0.f, 0.f}, (floatx4){0.f, 0.f, 0.f, 0.f}};
         float alpha = 1.0f;
 #pragma unroll
@@ -1146,7 +1158,7 @@ template <int DS> __device__ __forceinline__ void decode_wide_f32(const lng_k_at
             if (b + 1 < NBATCH) {
                 load_batch(tp, b + 1, nxt);
             } else if (more) {
-                load_batch(tp + 128u, 0, nxt);
+                load_batch(tp + tile_stride, 0, nxt);
             }
             if (b < KBATCH) {
 #pragma unroll
