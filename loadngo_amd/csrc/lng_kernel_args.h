@@ -32,7 +32,8 @@ typedef struct lng_k_attn {
     uint32_t heads;
     uint32_t kv_heads;
     uint32_t dim;
-    uint32_t chunk;           /* positions per workgroup along the cache (multiple of 128) */
+    uint32_t chunk;           /* positions per workgroup along the cache (multiple of 128): a row of v visible positions
+                                 has ceil(v / chunk) workgroups per kv head, which share its groups of 128 positions */
     uint32_t n_chunks;        /* chunks of the longest visible run = ceil(it / chunk): the partials keep this many slots per (row, kv head) */
     uint32_t dtype;           /* lng_dtype of q, k, v, out */
     uint32_t fused;           /* split-K: 1 = the last workgroup of a row merges, 0 = lng_decode_merge follows */

@@ -257,10 +257,11 @@ extern "C" __global__ __launch_bounds__(256) void lng_attn_generic_bf16(lng_k_at
 // =============================================================================================
 // Decode kernel, bf16, head width 64, up to 16 query heads per kv head.
 //
-// Grid: one workgroup per (row, kv head, chunk of a.chunk cached positions), see work_of. A workgroup
-// serves ALL query heads of its kv head at once, so each cached K and V row is read from HBM
-// once per group instead of once per query head. Its four wavefronts take interleaved tiles
-// of 32 positions. Everything is lane-local between the three MFMA stages:
+// Grid: one workgroup per (row, kv head, chunk), see work_of; a row of v visible positions has
+// ceil(v / a.chunk) chunks, and chunk c of n is the groups of 128 positions c, c + n, c + 2n, ... of the
+// row. A workgroup serves ALL query heads of its kv head at once, so each cached K and V row is read
+// from HBM once per group instead of once per query head. Its four wavefronts take a tile of 32
+// positions of each group. Everything is lane-local between the three MFMA stages:
 //
 //   S^T[tok][head] = K[tok][:] . Q[head][:]        2x2 v_mfma_f32_16x16x32_bf16 per tile
 //       lane (n = lane%16, j = lane/16) loads, for token half*16 + n, the 16 bytes at
