@@ -447,6 +447,45 @@ def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, st
     assert np.abs(got - other).max() <= 2.0 ** -7  # a bf16 step or two at |o| < 1
 
 
+@pytest.mark.parametrize("t,start,heads,kv_heads", [(2048, 1000, 64, 8), (1000, 0, 32, 8)])
+def test_long_causal_pass_gives_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, monkeypatch):
+    """The resident kernel's wavefronts pass the tile barrier at two different places of their sequence and share
+    three LDS buffers: 256 launches over the same inputs, each into its own output, all bit for bit the first
+    (an LDS row overwritten early or read late would show as a launch that differs)."""
+    monkeypatch.setenv("LNG_PREFILL_STREAM", "1")
+    dim, per_batch, end = 64, 32, start + t
+    rows, krows = (t + 31) // 32 * 32, (end + 31) // 32 * 32
+    one = rows * heads * dim * 2
+    bufs = [gpu.buffer(one), gpu.buffer(krows * kv_heads * dim * 2), gpu.buffer(krows * kv_heads * dim * 2),
+            gpu.buffer(per_batch * one), gpu.upload(np.random.default_rng(1).standard_normal(heads).astype(np.float32))]
+    try:
+        for i in range(3):
+            fill = gpu.batch([bufs[i]])
+            fill.fill_synthetic(C.Slice(0, 0, bufs[i].len), C.BF16, 90 + i, 0.5, 0)
+            fill.run()
+            fill.drop()
+        shape = C.GroupedShape(t, start, heads, kv_heads, dim, FULL, end, 0.125)
+        first = None
+        for _ in range(8):
+            batch = gpu.batch(bufs)
+            for j in range(per_batch):
+                batch.attention_grouped_tiled_with_sinks(
+                    (C.Slice(0, 0, bufs[0].len), C.Slice(1, 0, bufs[1].len), C.Slice(2, 0, bufs[2].len)),
+                    C.Slice(4, 0, heads * 4), C.Slice(3, j * one, one), shape, C.BF16)
+            done = batch.run()
+            batch.drop()
+            assert not isinstance(done.gpu_time, Exception), done.gpu_time
+            got = bufs[3].read(np.uint16).reshape(per_batch, rows, heads, dim)[:, :t]
+            if first is None:
+                first = got[0].copy()
+                assert not np.isnan(from_bf16_bits(first)).any()
+            for j in range(per_batch):
+                assert np.array_equal(got[j], first), "launch %d of a batch differs from the first launch" % j
+    finally:
+        for b in bufs:
+            b.free()
+
+
 @pytest.mark.parametrize("window", [FULL, 128])
 def test_config4_prefill_8192_sampled_rows(gpu, window):
     """The 8192-position prompt pass at its real size; a sample of query rows (first, last,
