@@ -2639,14 +2639,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         return;
     }
 
-    // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query -------------------
-    if (wave_active && row_ok) {
+    // ---- normalise and store. A lane holds 8-byte pieces of its query's row (dims 32db + 8blk + 4hh + i), and 32
+    // such pieces from 32 rows make a poor store: 16 partial writes to every 128-byte line. Through LDS (the K/V
+    // buffers, which nobody reads after the last tile's barrier; 32 rows of 144 bytes per wavefront) eight lanes
+    // write one whole 128-byte head row. No workgroup barrier: a wavefront's LDS operations run in order.
+    if (wave_active) {
+        uint16_t *stage = wave < 4u ? &s_k[0][0] + wave * (32u * 72u) : &s_v[0][0] + (wave - 4u) * (32u * 72u);
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
             if (h == 1 && !second_ok) continue;
             const float total = l[h] + __shfl_xor(l[h], 32, 64);
             const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-            uint16_t *op = (uint16_t *)a.out + ((uint64_t)my_row * a.heads + head[h]) * 64u;
 #pragma unroll
             for (int db = 0; db < 2; ++db) {
 #pragma unroll
@@ -2654,9 +2657,18 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                     bf16x4 w; // narrowed by the conversion instruction (round to nearest even)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) w[i] = (__bf16)(ot[h][db][4 * blk + i] * inv);
-                    *(bf16x4 *)(op + 32 * db + 8 * blk + 4 * hh) = w;
+                    *(bf16x4 *)(stage + n * 72u + 32 * db + 8 * blk + 4 * hh) = w;
                 }
             }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                const uint32_t r = 8u * pass + (lane >> 3), ch = lane & 7u;
+                const uint4 piece = *(const uint4 *)(stage + r * 72u + 8u * ch);
+                const uint32_t row = q0 + 32u * qb + r;
+                if (row < t) *(uint4 *)((uint16_t *)a.out + ((uint64_t)row * a.heads + head[h]) * 64u + 8u * ch) = piece;
+            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
 }
