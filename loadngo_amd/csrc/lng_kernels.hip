@@ -2616,24 +2616,35 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     }
 
 
-    // ---- with splits: leave the partial state, lane holds dims 32db + 8blk + 4hh + i of its query ----
+    // ---- with splits: leave the partial state, lane holds dims 32db + 8blk + 4hh + i of its query. Through LDS
+    // like the outputs below, 32 dimensions (128 bytes of f32) of 32 rows at a time: eight lanes store a whole line.
     if (partial) {
-        if (wave_active && row_ok) {
+        if (wave_active) {
+            float *stage = (float *)(wave < 4u ? &s_k[0][0] + wave * (32u * 72u) : &s_v[0][0] + (wave - 4u) * (32u * 72u));
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
                 if (h == 1 && !second_ok) continue;
                 const float total = l[h] + __shfl_xor(l[h], 32, 64);
                 const uint64_t slot = (((uint64_t)my_row * a.kv_heads + g) * a.splits + split) * group + (head[h] - g * group);
-                float *po = a.partial_o + slot * 64u;
+                if (hh == 0 && row_ok) *(float2 *)(a.partial_ml + slot * 2u) = make_float2(m[h], total);
 #pragma unroll
                 for (int db = 0; db < 2; ++db) {
 #pragma unroll
                     for (int blk = 0; blk < 4; ++blk) {
-                        *(float4 *)(po + 32 * db + 8 * blk + 4 * hh) = make_float4(ot[h][db][4 * blk + 0], ot[h][db][4 * blk + 1],
-                                                                                   ot[h][db][4 * blk + 2], ot[h][db][4 * blk + 3]);
+                        *(float4 *)(stage + n * 36u + 8 * blk + 4 * hh) = make_float4(ot[h][db][4 * blk + 0], ot[h][db][4 * blk + 1],
+                                                                                      ot[h][db][4 * blk + 2], ot[h][db][4 * blk + 3]);
                     }
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int pass = 0; pass < 4; ++pass) {
+                        const uint32_t r = 8u * pass + (lane >> 3), ch = lane & 7u;
+                        const float4 piece = *(const float4 *)(stage + r * 36u + 4u * ch);
+                        const uint32_t row = q0 + 32u * qb + r;
+                        const uint64_t rslot = (((uint64_t)row * a.kv_heads + g) * a.splits + split) * group + (head[h] - g * group);
+                        if (row < t) *(float4 *)(a.partial_o + rslot * 64u + 32 * db + 4u * ch) = piece;
+                    }
+                    __builtin_amdgcn_wave_barrier();
                 }
-                if (hh == 0) *(float2 *)(a.partial_ml + slot * 2u) = make_float2(m[h], total);
             }
         }
         return;
