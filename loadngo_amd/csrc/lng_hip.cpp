@@ -92,7 +92,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_bf16_d64_o4 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr, decode_merge_few = nullptr;
     hipFunction_t decode_bf16_wide[3] = {}, decode_f32_wide[3] = {}; // head widths 128, 256, 512
-    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
+    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_h1w = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
     hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_one_w8 = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
@@ -694,8 +694,11 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         }
         // f32: two workgroups per compute unit only when there are four rounds of them or more (see the kernels)
         const bool f32_two = f32 && c.grid[0] >= 4u * g->cus;
-        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : g->prefill_bf16_d64;
-        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : "lng_prefill_bf16_d64";
+        // Windows of up to 160 positions: the 32 query rows of a workgroup see at most four tiles of 64 keys, and the
+        // one-head kernel asks for all of them at its start, straight into LDS (LNG_PREFILL_UPFRONT=0: never).
+        const bool upfront = narrow && p.window != LNG_WINDOW_FULL && p.window <= 160 && p.splits == 1 && !env_is(getenv("LNG_PREFILL_UPFRONT"), "0");
+        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : upfront ? g->prefill_bf16_d64_h1w : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : g->prefill_bf16_d64;
+        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : upfront ? "lng_prefill_bf16_d64_h1w" : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : "lng_prefill_bf16_d64";
         set_args(c, p);
         b->cmds.push_back(std::move(c));
         if (p.splits > 1) {
@@ -794,6 +797,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_decode_f32_w512", &g->decode_f32_wide[2], true},
         {"lng_prefill_bf16_d64", &g->prefill_bf16_d64, true},
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
+        {"lng_prefill_bf16_d64_h1w", &g->prefill_bf16_d64_h1w, true},
         {"lng_prefill_bf16_d64_stream", &g->prefill_bf16_d64_stream, true},
         {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
         {"lng_prefill_f32_d64_w4", &g->prefill_f32_d64_w4, true},

@@ -2247,14 +2247,32 @@ __device__ __forceinline__ bf16x8 lds_read_tr8(const uint16_t *p0, const uint16_
 // every K/V operand read from LDS feeds two products, which is what a long causal pass needs.
 // NH = 1: 32 query rows per workgroup, wavefront = head; half the registers, so two workgroups share a
 // compute unit (4 wavefronts per SIMD) and short, latency-bound passes (a 128-token window) overlap.
-template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefill &a) {
+//
+// UP (one head per wavefront only; narrow windows, at most PF_UP_TILES key tiles per workgroup, no splits): every
+// K and V row the workgroup needs is requested at the start, together with the queries, by loads that write LDS
+// directly (global_load_lds_dwordx4: no registers in between, so nothing limits how many are in flight), there is
+// one barrier when they have landed, and the blocks of 32 keys then run without any further wait for memory. A
+// pass over a 128-position window otherwise spends a memory round trip per tile: the loads of tile i+1 leave when
+// tile i's arithmetic starts and take longer than it does. Such a load writes the 16 bytes of lane l at
+// base + 16 l, so rows cannot be padded; instead each lane fetches the piece that belongs at its place in a
+// swizzled row: piece c (16 bytes) of K row r sits at c ^ ((r >> 1) & 7) - the 16-byte reads of 16 consecutive
+// rows then fall in 16 different 16-byte bank groups - and piece c of V row r at c ^ (((r >> 1) & 1) << 2): the
+// four rows x 64 bytes that half a wavefront reads transposed fall in four different quarters of the banks.
+#define PF_UP_TILES 4
+template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(const lng_k_prefill &a) {
+    static_assert(!UP || NH == 1, "rows are requested up front in the one-head form only");
     constexpr uint32_t PF_BM = NH == 2 ? 64u : 32u;
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
+    constexpr uint32_t K_BUF = UP ? PF_BN * 64u : PF_BN * PF_KSTRIDE; // elements per tile buffer
+    constexpr uint32_t V_BUF = UP ? PF_BN * 64u : PF_BN * PF_VSTRIDE;
+    constexpr uint32_t N_BUF = UP ? PF_UP_TILES : 2;
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[N_BUF][K_BUF];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[N_BUF][V_BUF];
 
+    const bool partial = a.splits > 1u;
     const uint32_t g = blockIdx.x % a.kv_heads;
-    const uint32_t split = (blockIdx.x / a.kv_heads) % a.splits;
-    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads / a.splits;
+    const uint32_t above = blockIdx.x / a.kv_heads;
+    const uint32_t split = partial ? above % a.splits : 0u;        // an unsplit pass pays for no division by splits
+    const uint32_t qtile = a.q_tiles - 1u - (partial ? above / a.splits : above);
     const uint32_t group = a.heads / a.kv_heads;
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & 63u;
@@ -2278,9 +2296,8 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     const uint32_t all_tiles = (pos_last - tile0) / PF_BN + 1;
     // With splits, this workgroup takes tiles [first_tile, n_tiles) of the query tile's run (possibly
     // none) and leaves (max, sum, unnormalised output) for lng_prefill_merge, which also adds the sink.
-    const bool partial = a.splits > 1u;
-    const uint32_t first_tile = (uint32_t)((uint64_t)all_tiles * split / a.splits);
-    const uint32_t n_tiles = (uint32_t)((uint64_t)all_tiles * (split + 1u) / a.splits);
+    const uint32_t first_tile = partial ? (uint32_t)((uint64_t)all_tiles * split / a.splits) : 0u;
+    const uint32_t n_tiles = partial ? (uint32_t)((uint64_t)all_tiles * (split + 1u) / a.splits) : all_tiles;
     const bool ring = a.slots < end;
     const uint32_t slots = (uint32_t)a.slots;
     const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
@@ -2308,12 +2325,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             if (row_ok) {
                 raw = *(const uint4 *)(a.q + (((uint64_t)my_row * a.heads + head[h]) * 64u + 16u * ks + 8u * hh) * 2u);
             }
-            // scale * log2(e) goes into the query operand, once: the products then come out of the matrix unit
-            // in the exponent's own units (one more bf16 rounding of q: 2^-9 relative per element, a few 1e-4 on
-            // a score, an order below the rounding of the weights to bf16)
+            // Two heads per wavefront: scale * log2(e) goes into the query operand, once; the products then come out
+            // of the matrix unit in the exponent's own units (one more bf16 rounding of q: 2^-9 relative per element,
+            // a few 1e-4 on a score, an order below the rounding of the weights to bf16), and a pass whose maximum is
+            // fixed at zero has nothing left to do but the exponential. One head per wavefront always tracks the
+            // maximum: there the factor rides in the multiply-add that subtracts the maximum, and the 80
+            // instructions that rescale the queries are saved.
             bf16x8 qv = as_bf16x8(raw);
+            if constexpr (NH == 2) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) qv[e] = (__bf16)((float)qv[e] * sl2);
+                for (int e = 0; e < 8; ++e) qv[e] = (__bf16)((float)qv[e] * sl2);
+            }
             qreg[h][ks] = qv;
         }
     }
@@ -2338,13 +2360,32 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         *(uint4 *)(&s_k[buf][ld_key * PF_KSTRIDE + ld_chunk * 8u]) = kr;
         *(uint4 *)(&s_v[buf][ld_key * PF_VSTRIDE + ld_chunk * 8u]) = vr;
     };
+    // UP: this thread's row of a tile straight into LDS; a wavefront's 64 lanes fill 8 whole rows (1 KiB) of K and of V
+    auto request = [&](uint32_t tile) {
+        uint32_t p = tile0 + tile * PF_BN + ld_key;
+        p = p > pos_last ? pos_last : p;
+        p = p < kfirst ? kfirst : p;
+        const uint32_t r = ring ? p % slots : p;
+        const uint32_t ck = ld_chunk ^ ((ld_key >> 1) & 7u), cv = ld_chunk ^ (((ld_key >> 1) & 1u) << 2);
+        typedef __attribute__((address_space(1))) const void *gptr;
+        typedef __attribute__((address_space(3))) void *lptr;
+        __builtin_amdgcn_global_load_lds((gptr)(a.k + (uint64_t)g * 128u + (uint64_t)r * row_bytes + ck * 16u),
+                                         (lptr)(&s_k[tile][wave * 512u]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(a.v + (uint64_t)g * 128u + (uint64_t)r * row_bytes + cv * 16u),
+                                         (lptr)(&s_v[tile][wave * 512u]), 16, 0, 0);
+    };
 
     // per-lane constant parts of the LDS addresses
-    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
+    // (UP: rows of 64 elements, piece 2 ks + hh at (2 ks + hh) ^ ((n >> 1) & 7): the lane's part of it here, ks as
+    // an exclusive-or of 16 ks elements on top)
+    const uint32_t k_lane_off = UP ? n * 64u + ((hh ^ ((n >> 1) & 7u)) << 3) : n * PF_KSTRIDE + 8u * hh; // + kb*32*KSTRIDE + 16*ks
     const uint32_t L = lane & 15u;
     const uint32_t blk16 = lane >> 4;                                     // 16-lane block 0..3
     // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
-    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+    // (UP: the rows two apart within a group of four have their 64-byte halves exchanged)
+    const uint32_t v_lane_off = UP ? (4u * (blk16 >> 1) + (L >> 2)) * 64u + 16u * (blk16 & 1u) + 4u * (L & 3u)
+                                   : (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+    const uint32_t v_flip = (L >> 3) & 1u;
 
     // With two heads per wavefront (long causal runs) the pass is first made optimistically: once a
     // first interior tile has set the running maximum from real scores, the remaining interior
@@ -2383,7 +2424,11 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
         }
     }
-    if (first_tile < n_tiles) {
+    if constexpr (UP) {
+        const uint32_t up_tiles = all_tiles < PF_UP_TILES ? all_tiles : PF_UP_TILES; // (the host sends no more this way)
+        for (uint32_t i = 0; i < up_tiles; ++i) request(i);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's rows are in LDS (and its queries in registers)
+    } else if (first_tile < n_tiles) {
         fetch(first_tile, kr, vr);
         stash(first_tile & 1u, kr, vr);
     }
@@ -2396,6 +2441,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool FIXED = MODE != 0;
+        constexpr bool RAW = NH == 1; // the products are plain q.k: the factor is applied with the maximum
         const uint32_t buf = tile & 1u;
         const uint32_t kt0 = tile0 + tile * PF_BN; // position of the tile's first key
             {
@@ -2404,7 +2450,11 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                 bf16x8 ka[4];
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
-                    ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
+                    if constexpr (UP) {
+                        ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[0][(k_lane_off ^ (16u * ks)) + kb * 32 * 64]));
+                    } else {
+                        ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
+                    }
                 }
                 floatx16 st[NH];
 #pragma unroll
@@ -2425,8 +2475,13 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                         for (int db = 0; db < 2; ++db) {
-                            const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
-                            va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                            if constexpr (UP) {
+                                const uint16_t *vp = &s_v[0][v_lane_off + (32 * kb + 16 * jj) * 64 + 32 * (db ^ v_flip)];
+                                va[jj][db] = lds_read_tr8(vp, vp + 8 * 64);
+                            } else {
+                                const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                                va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
+                            }
                         }
                     }
                 };
@@ -2442,12 +2497,19 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                     if constexpr (MASK) {
                         // key kp = kt0 + 32 kb + 4 hh + o_i is visible when 0 <= my_pos - kp < window, i.e. when the
                         // constant o_i lies in (dist - window, dist]: two compares against per-block bounds
-                        const int dist = (int)(my_pos - (kt0 + 32u * kb + 4u * hh));
-                        const int below = windowed ? dist - (int)window : -0x40000000;
+                        // With one head per wavefront (windows), a block of an edge tile that every query of the
+                        // workgroup sees whole skips the masks: a uniform branch around them (three of the five
+                        // blocks of a 128-position window).
+                        const uint32_t b0 = kt0 + 32u * kb;
+                        const bool cut = NH == 2 || b0 + 31u > pos_first || (windowed && b0 + window < pos_first + PF_BM);
+                        if (cut) {
+                            const int dist = (int)(my_pos - (b0 + 4u * hh));
+                            const int below = windowed ? dist - (int)window : -0x40000000;
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) {
-                            const int o = 8 * (i >> 2) + (i & 3);
-                            st[h][i] = (o <= dist && o > below) ? st[h][i] : LNG_NEG_INF;
+                            for (int i = 0; i < 16; ++i) {
+                                const int o = 8 * (i >> 2) + (i & 3);
+                                st[h][i] = (o <= dist && o > below) ? st[h][i] : LNG_NEG_INF;
+                            }
                         }
                     }
                     float m_safe = 0.0f;
@@ -2458,6 +2520,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
 #pragma unroll
                         for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[h][i]);
                         tmax = other_half_max(tmax);
+                        if constexpr (RAW) tmax *= sl2; // the host sends only positive factors this way
                         const float m_new = tmax > m[h] + PF_TAU ? tmax : m[h];
                         m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
                         if (__builtin_amdgcn_ballot_w64(m_new != m[h]) != 0) {
@@ -2476,8 +2539,9 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                         for (int e = 0; e < 8; e += 2) {
-                            const float p0 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e] : st[h][8 * jj + e] - m_safe);
-                            const float p1 = __builtin_amdgcn_exp2f(MODE == 2 ? st[h][8 * jj + e + 1] : st[h][8 * jj + e + 1] - m_safe);
+                            const float s0 = st[h][8 * jj + e], s1 = st[h][8 * jj + e + 1];
+                            const float p0 = __builtin_amdgcn_exp2f(RAW ? __builtin_fmaf(s0, sl2, MODE == 2 ? 0.0f : -m_safe) : MODE == 2 ? s0 : s0 - m_safe);
+                            const float p1 = __builtin_amdgcn_exp2f(RAW ? __builtin_fmaf(s1, sl2, MODE == 2 ? 0.0f : -m_safe) : MODE == 2 ? s1 : s1 - m_safe);
                             bf16x2 pr;
                             pr[0] = (__bf16)p0;
                             pr[1] = (__bf16)p1;
@@ -2517,9 +2581,9 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         if (wave_active) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
-                if constexpr (decltype(mask_tag)::value && NH == 1) { // windows: a block no query of the workgroup sees
+                if constexpr (decltype(mask_tag)::value && NH == 1) {
                     const uint32_t b0 = tile0 + tile * PF_BN + 32u * kb;
-                    if (b0 > pos_last || b0 + 31u < kfirst) continue;
+                    if (b0 > pos_last || b0 + 31u < kfirst) continue; // windows: a block no query of the workgroup sees
                 }
                 block(mask_tag, mode_tag, tile, kb);
             }
@@ -2537,7 +2601,17 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     using fixed_at_zero = std::integral_constant<int, 2>;
     uint32_t tile = first_tile;
     bool frozen = false;
-    {
+    if constexpr (UP) {
+        // blocks of 32 keys from the one that holds the first visible key to the one that holds the last
+        // (Measured and not kept: a first pass around zero - weights 2^score, no maxima, the sums on the matrix unit,
+        // a range check and the tracked pass again when it fails: 40 % fewer vector instructions per block, same time.)
+        if (wave_active) {
+            const uint32_t b_end = min((pos_last - tile0) / 32u + 1u, 2u * PF_UP_TILES);
+            for (uint32_t b = (kfirst - tile0) / 32u; b < b_end; ++b) block(std::true_type{}, tracked{}, 0u, (int)b);
+        }
+        __syncthreads(); // the rows are dead: the outputs are laid down over them
+        tile = n_tiles;
+    } else {
     for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tracked{}, tile); // window edge
     if (optimistic) {                                                                      // interior
         bool at_zero = false;
@@ -2690,6 +2764,12 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64(ln
 
 extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1(lng_k_prefill a) {
     prefill_body<1>(a);
+}
+
+// The one-head form with every K and V row requested up front, straight into LDS: windows of at most
+// 64 PF_UP_TILES - 96 positions, no splits (64 KiB of LDS, two workgroups per compute unit).
+extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1w(lng_k_prefill a) {
+    prefill_body<1, true>(a);
 }
 
 // =============================================================================================

@@ -418,6 +418,56 @@ def test_windowed_prefill_with_scores_far_outside_the_usual_range(gpu, case, win
         assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
 
 
+@pytest.mark.parametrize("t,start,window,slots,heads,kv_heads", [
+    (500, 0, 128, 500, 64, 8),      # the usual window, aligned: three tiles of keys per workgroup
+    (333, 4077, 128, 4410, 16, 2),  # an odd start: four tiles
+    (200, 1000, 160, 1300, 6, 2),   # the widest window that goes this way; groups of three heads: idle wavefronts
+    (97, 31, 40, 128, 16, 4), (65, 3, 1, 96, 8, 8), (130, 1000, 128, 320, 4, 1), (40, 97, 7, 64, 10, 2),
+    (31, 900, 100, 160, 64, 8),     # fewer than 32 rows, in a ring that wraps
+])
+def test_narrow_windows_with_every_row_requested_up_front(gpu, t, start, window, slots, heads, kv_heads, monkeypatch):
+    """Windows of up to 160 positions run the kernel that asks for all of a workgroup's K and V rows at its start,
+    by loads that write LDS directly into swizzled rows: it is the kernel the dispatch names, it agrees with the CPU
+    reference, and it gives the bits of the tile-by-tile kernel (same arithmetic in the same order; a wrong swizzle
+    or a row in the wrong place changes them)."""
+    end = start + t
+    q, k, v, sinks = normal_inputs(11 + window + t, t, end, heads, kv_heads, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    # rows the pass may not read are poisoned (NaN bits): positions before the first query's window, rows never written
+    kp, vp = kb.copy(), vb.copy()
+    kp[:max(0, start + 1 - window)] = 0x7FC0
+    vp[:max(0, start + 1 - window)] = 0x7FC0
+    kr, vr = ring_layout(kp, t, start, slots, True, fill=0x7FC0), ring_layout(vp, t, start, slots, True, fill=0x7FC0)
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    want = oracle.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS)
+
+    def run(expect):
+        rows = (t + 31) // 32 * 32
+        qp = np.zeros((rows, heads, 64), dtype=np.uint16)
+        qp[:t] = qb
+        bufs = [gpu.upload(qp), gpu.upload(kr), gpu.upload(vr), gpu.buffer(qp.nbytes), gpu.upload(sinks)]
+        bufs[3].fill(0xFF)
+        batch = gpu.batch(bufs)
+        try:
+            batch.set_timing(True)
+            batch.attention_grouped_tiled_with_sinks((C.Slice(0, 0, qp.nbytes), C.Slice(1, 0, kr.nbytes), C.Slice(2, 0, vr.nbytes)),
+                                                     C.Slice(4, 0, heads * 4), C.Slice(3, 0, qp.nbytes), shape, C.BF16)
+            done = batch.run()
+            assert not isinstance(done.gpu_time, Exception), done.gpu_time
+            assert batch.kernel_seconds(expect)[1] == 1
+            return bufs[3].read(np.uint16).reshape(rows, heads, 64)[:t]
+        finally:
+            batch.drop()
+            for b in bufs:
+                b.free()
+
+    got = run("lng_prefill_bf16_d64_h1w")
+    assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+    monkeypatch.setenv("LNG_PREFILL_UPFRONT", "0")
+    tile_by_tile = run("lng_prefill_bf16_d64_h1")
+    assert np.array_equal(got, tile_by_tile)
+
+
 @pytest.mark.parametrize("t,start,heads,kv_heads,sinks_on", [
     (300, 0, 64, 8, True), (1000, 0, 32, 8, True), (777, 1300, 64, 8, False), (64, 0, 16, 2, True), (65, 63, 8, 1, True),
     (130, 4000, 24, 8, True), (2048, 0, 64, 8, True)])
