@@ -2772,6 +2772,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     prefill_body<1, true>(a);
 }
 
+// (Measured and not kept: workgroups of four wavefronts with two heads each, one after the other, three to a compute
+// unit with 48 KiB of LDS each - the same bits and the same time as the form above.)
+
 // =============================================================================================
 // The long full-causal prompt pass (no window, no ring, keys not split): lng_prefill_bf16_d64's
 // arithmetic, tile for tile, in a workgroup that STAYS on its compute unit and walks several
