@@ -2247,26 +2247,10 @@ __device__ __forceinline__ bf16x8 lds_read_tr8(const uint16_t *p0, const uint16_
 // every K/V operand read from LDS feeds two products, which is what a long causal pass needs.
 // NH = 1: 32 query rows per workgroup, wavefront = head; half the registers, so two workgroups share a
 // compute unit (4 wavefronts per SIMD) and short, latency-bound passes (a 128-token window) overlap.
-//
-// UP (one head per wavefront only; narrow windows, at most PF_UP_TILES key tiles per workgroup, no splits): every
-// K and V row the workgroup needs is requested at the start, together with the queries, by loads that write LDS
-// directly (global_load_lds_dwordx4: no registers in between, so nothing limits how many are in flight), there is
-// one barrier when they have landed, and the blocks of 32 keys then run without any further wait for memory. A
-// pass over a 128-position window otherwise spends a memory round trip per tile: the loads of tile i+1 leave when
-// tile i's arithmetic starts and take longer than it does. Such a load writes the 16 bytes of lane l at
-// base + 16 l, so rows cannot be padded; instead each lane fetches the piece that belongs at its place in a
-// swizzled row: piece c (16 bytes) of K row r sits at c ^ ((r >> 1) & 7) - the 16-byte reads of 16 consecutive
-// rows then fall in 16 different 16-byte bank groups - and piece c of V row r at c ^ (((r >> 1) & 1) << 2): the
-// four rows x 64 bytes that half a wavefront reads transposed fall in four different quarters of the banks.
-#define PF_UP_TILES 4
-template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(const lng_k_prefill &a) {
-    static_assert(!UP || NH == 1, "rows are requested up front in the one-head form only");
+template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefill &a) {
     constexpr uint32_t PF_BM = NH == 2 ? 64u : 32u;
-    constexpr uint32_t K_BUF = UP ? PF_BN * 64u : PF_BN * PF_KSTRIDE; // elements per tile buffer
-    constexpr uint32_t V_BUF = UP ? PF_BN * 64u : PF_BN * PF_VSTRIDE;
-    constexpr uint32_t N_BUF = UP ? PF_UP_TILES : 2;
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[N_BUF][K_BUF];
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[N_BUF][V_BUF];
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
 
     const bool partial = a.splits > 1u;
     const uint32_t g = blockIdx.x % a.kv_heads;
@@ -2360,32 +2344,13 @@ template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(
         *(uint4 *)(&s_k[buf][ld_key * PF_KSTRIDE + ld_chunk * 8u]) = kr;
         *(uint4 *)(&s_v[buf][ld_key * PF_VSTRIDE + ld_chunk * 8u]) = vr;
     };
-    // UP: this thread's row of a tile straight into LDS; a wavefront's 64 lanes fill 8 whole rows (1 KiB) of K and of V
-    auto request = [&](uint32_t tile) {
-        uint32_t p = tile0 + tile * PF_BN + ld_key;
-        p = p > pos_last ? pos_last : p;
-        p = p < kfirst ? kfirst : p;
-        const uint32_t r = ring ? p % slots : p;
-        const uint32_t ck = ld_chunk ^ ((ld_key >> 1) & 7u), cv = ld_chunk ^ (((ld_key >> 1) & 1u) << 2);
-        typedef __attribute__((address_space(1))) const void *gptr;
-        typedef __attribute__((address_space(3))) void *lptr;
-        __builtin_amdgcn_global_load_lds((gptr)(a.k + (uint64_t)g * 128u + (uint64_t)r * row_bytes + ck * 16u),
-                                         (lptr)(&s_k[tile][wave * 512u]), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr)(a.v + (uint64_t)g * 128u + (uint64_t)r * row_bytes + cv * 16u),
-                                         (lptr)(&s_v[tile][wave * 512u]), 16, 0, 0);
-    };
 
     // per-lane constant parts of the LDS addresses
-    // (UP: rows of 64 elements, piece 2 ks + hh at (2 ks + hh) ^ ((n >> 1) & 7): the lane's part of it here, ks as
-    // an exclusive-or of 16 ks elements on top)
-    const uint32_t k_lane_off = UP ? n * 64u + ((hh ^ ((n >> 1) & 7u)) << 3) : n * PF_KSTRIDE + 8u * hh; // + kb*32*KSTRIDE + 16*ks
+    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
     const uint32_t L = lane & 15u;
     const uint32_t blk16 = lane >> 4;                                     // 16-lane block 0..3
     // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
-    // (UP: the rows two apart within a group of four have their 64-byte halves exchanged)
-    const uint32_t v_lane_off = UP ? (4u * (blk16 >> 1) + (L >> 2)) * 64u + 16u * (blk16 & 1u) + 4u * (L & 3u)
-                                   : (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
-    const uint32_t v_flip = (L >> 3) & 1u;
+    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
 
     // With two heads per wavefront (long causal runs) the pass is first made optimistically: once a
     // first interior tile has set the running maximum from real scores, the remaining interior
@@ -2424,11 +2389,7 @@ template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(
             for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
         }
     }
-    if constexpr (UP) {
-        const uint32_t up_tiles = all_tiles < PF_UP_TILES ? all_tiles : PF_UP_TILES; // (the host sends no more this way)
-        for (uint32_t i = 0; i < up_tiles; ++i) request(i);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's rows are in LDS (and its queries in registers)
-    } else if (first_tile < n_tiles) {
+    if (first_tile < n_tiles) {
         fetch(first_tile, kr, vr);
         stash(first_tile & 1u, kr, vr);
     }
@@ -2450,11 +2411,7 @@ template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(
                 bf16x8 ka[4];
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
-                    if constexpr (UP) {
-                        ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[0][(k_lane_off ^ (16u * ks)) + kb * 32 * 64]));
-                    } else {
-                        ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
-                    }
+                    ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[buf][k_lane_off + kb * 32 * PF_KSTRIDE + 16 * ks]));
                 }
                 floatx16 st[NH];
 #pragma unroll
@@ -2475,13 +2432,8 @@ template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(
                     for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
                         for (int db = 0; db < 2; ++db) {
-                            if constexpr (UP) {
-                                const uint16_t *vp = &s_v[0][v_lane_off + (32 * kb + 16 * jj) * 64 + 32 * (db ^ v_flip)];
-                                va[jj][db] = lds_read_tr8(vp, vp + 8 * 64);
-                            } else {
-                                const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
-                                va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
-                            }
+                            const uint16_t *vp = &s_v[buf][v_lane_off + (32 * kb + 16 * jj) * PF_VSTRIDE + 32 * db];
+                            va[jj][db] = lds_read_tr8(vp, vp + 8 * PF_VSTRIDE);
                         }
                     }
                 };
@@ -2601,17 +2553,7 @@ template <int NH, bool UP = false> __device__ __forceinline__ void prefill_body(
     using fixed_at_zero = std::integral_constant<int, 2>;
     uint32_t tile = first_tile;
     bool frozen = false;
-    if constexpr (UP) {
-        // blocks of 32 keys from the one that holds the first visible key to the one that holds the last
-        // (Measured and not kept: a first pass around zero - weights 2^score, no maxima, the sums on the matrix unit,
-        // a range check and the tracked pass again when it fails: 40 % fewer vector instructions per block, same time.)
-        if (wave_active) {
-            const uint32_t b_end = min((pos_last - tile0) / 32u + 1u, 2u * PF_UP_TILES);
-            for (uint32_t b = (kfirst - tile0) / 32u; b < b_end; ++b) block(std::true_type{}, tracked{}, 0u, (int)b);
-        }
-        __syncthreads(); // the rows are dead: the outputs are laid down over them
-        tile = n_tiles;
-    } else {
+    {
     for (; tile < n_tiles && edge(tile); ++tile) step(std::true_type{}, tracked{}, tile); // window edge
     if (optimistic) {                                                                      // interior
         bool at_zero = false;
@@ -2766,14 +2708,195 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     prefill_body<1>(a);
 }
 
-// The one-head form with every K and V row requested up front, straight into LDS: windows of at most
-// 64 PF_UP_TILES - 96 positions, no splits (64 KiB of LDS, two workgroups per compute unit).
+// Windows of at most 160 positions (unsplit passes): lng_prefill_bf16_d64_h1's arithmetic, block for block, with
+// every K and V row of the workgroup requested at its start. A workgroup of eight wavefronts (a head each) takes 32
+// query rows; they see at most 160 + 31 keys, which lie in at most four tiles of 64 rows from a multiple of 64.
+// These rows are asked for together with the queries by loads that write LDS directly (global_load_lds_dwordx4: no registers in between, so nothing limits how
+// many are in flight); there is one barrier when they have landed, and the blocks of 32 keys then run without any
+// further wait for memory - tile by tile, such a pass spends a memory round trip per tile: the loads of tile i+1
+// leave when tile i's arithmetic starts and take longer than it does. A load of this kind puts the 16 bytes of
+// lane l at base + 16 l, so rows cannot be padded; instead each lane fetches the piece that belongs at its place in
+// a swizzled row: piece c (16 bytes) of K row r sits at c ^ ((r >> 1) & 7) - the 16-byte reads of 16 consecutive
+// rows then fall in 16 different 16-byte bank groups - and piece c of V row r at c ^ (((r >> 1) & 1) << 2): the
+// four rows x 64 bytes that half a wavefront reads transposed fall in four different quarters of the banks.
+// After the last block a barrier says that nobody reads K and V any more, and each wavefront lays its rows down
+// there so that eight lanes store a whole 128-byte row. 64 KiB of LDS: two workgroups per compute unit.
+// (Measured and not kept: a first pass around zero - weights 2^score, no maxima, the sums on the matrix unit, a range
+// check and the tracked pass again when it fails: 40 % fewer vector instructions per block, same time; workgroups of
+// four wavefronts with two heads each, three to a compute unit with 48 KiB of LDS each: same time; 64 query rows per
+// workgroup as two blocks of 32, one after the other, over the same K and V rows: 42 against 39 us.)
+#define PW_TILES 4
 extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1w(lng_k_prefill a) {
-    prefill_body<1, true>(a);
-}
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[PW_TILES * 64 * 64];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[PW_TILES * 64 * 64];
+    const uint32_t g = blockIdx.x % a.kv_heads;
+    const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads;
+    const uint32_t group = a.heads / a.kv_heads;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & 63u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n = lane & 31u;  // query within the block of 32
+    const uint32_t hh = lane >> 5;  // which half of the k-slots / of each 8 accumulator rows
+    const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
+    const uint32_t q0 = qtile * 32u;
+    const uint32_t rows_here = t - q0 < 32u ? t - q0 : 32u;
+    const uint32_t end = start + t;
+    const uint32_t pos_first = start + q0;
+    const uint32_t pos_last = pos_first + rows_here - 1u;
+    const uint32_t window = (uint32_t)a.window; // the host sends windows of 1..160 only
+    const uint32_t kfirst = pos_first + 1u > window ? pos_first + 1u - window : 0u;
+    const uint32_t tile0 = kfirst & ~63u;
+    const uint32_t n_tiles = min((pos_last - tile0) / 64u + 1u, (uint32_t)PW_TILES);
+    const bool ring = a.slots < end;
+    const uint32_t slots = (uint32_t)a.slots;
+    const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
+    const float sl2 = a.scale * LNG_LOG2E;
+    const bool wave_active = wave < group; // a wavefront past the group only helps loading
+    const uint32_t head = g * group + (wave_active ? wave : 0u);
 
-// (Measured and not kept: workgroups of four wavefronts with two heads each, one after the other, three to a compute
-// unit with 48 KiB of LDS each - the same bits and the same time as the form above.)
+    // the queries as they are: scale x log2(e) rides with the maximum
+    const uint32_t my_pos = pos_first + n;
+    bf16x8 qreg[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (q0 + n < t) raw = *(const uint4 *)(a.q + (((uint64_t)(q0 + n) * a.heads + head) * 64u + 16u * ks + 8u * hh) * 2u);
+        qreg[ks] = as_bf16x8(raw);
+    }
+    // every K and V row of the workgroup: a wavefront's 64 lanes fill 8 whole rows of a tile
+    {
+        const uint32_t ld_row = 8u * wave + (lane >> 3), ld_chunk = lane & 7u;
+        const uint32_t ck = ld_chunk ^ ((ld_row >> 1) & 7u), cv = ld_chunk ^ (((ld_row >> 1) & 1u) << 2);
+        typedef __attribute__((address_space(1))) const void *gptr;
+        typedef __attribute__((address_space(3))) void *lptr;
+        for (uint32_t i = 0; i < n_tiles; ++i) {
+            uint32_t p = tile0 + 64u * i + ld_row;
+            p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway,
+            p = p < kfirst ? kfirst : p;     // and so are rows before the first one (a ring may not hold them any more)
+            const uint32_t r = ring ? p % slots : p;
+            __builtin_amdgcn_global_load_lds((gptr)(a.k + (uint64_t)g * 128u + (uint64_t)r * row_bytes + ck * 16u),
+                                             (lptr)(s_k + i * 4096u + wave * 512u), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr)(a.v + (uint64_t)g * 128u + (uint64_t)r * row_bytes + cv * 16u),
+                                             (lptr)(s_v + i * 4096u + wave * 512u), 16, 0, 0);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this wavefront's rows are in LDS, its queries in registers
+    __syncthreads();
+
+    const uint32_t k_lane_off = n * 64u + ((hh ^ ((n >> 1) & 7u)) << 3); // ^ 16 ks, + 2048 b
+    const uint32_t L = lane & 15u;
+    const uint32_t blk16 = lane >> 4;
+    // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
+    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * 64u + 16u * (blk16 & 1u) + 4u * (L & 3u);
+    const uint32_t v_flip = (L >> 3) & 1u; // rows two apart within a group of four have their 64-byte halves exchanged
+    bf16x2 ones2;
+    ones2[0] = (__bf16)1.0f;
+    ones2[1] = (__bf16)1.0f;
+    floatx16 ot[2];
+    float l = 0.0f;
+    if (wave_active) {
+        float m = a.sinks ? a.sinks[head] * LNG_LOG2E : LNG_NEG_INF;
+        l = (a.sinks && hh == 0) ? 1.0f : 0.0f;
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) ot[db][i] = 0.0f;
+        }
+        // blocks of 32 keys from the one that holds the first visible key to the one that holds the last
+        const uint32_t b_end = min((pos_last - tile0) / 32u + 1u, 2u * PW_TILES);
+        for (uint32_t b = (kfirst - tile0) / 32u; b < b_end; ++b) {
+            bf16x8 ka[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[(k_lane_off ^ (16u * ks)) + b * 2048u]));
+            floatx16 st;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) st[i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) st = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qreg[ks], st, 0, 0, 0);
+            // V^T operands: issued now, their LDS latency hides behind the softmax arithmetic
+            bf16x8 va[2][2];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+                    const uint16_t *vp = &s_v[v_lane_off + (32u * b + 16 * jj) * 64u + 32 * (db ^ v_flip)];
+                    va[jj][db] = lds_read_tr8(vp, vp + 8 * 64);
+                }
+            }
+            // key kp = b0 + 4 hh + o_i is visible when 0 <= my_pos - kp < window; a block every row sees whole skips it
+            const uint32_t b0 = tile0 + 32u * b;
+            if (b0 + 31u > pos_first || b0 + window < pos_first + 32u) {
+                const int dist = (int)(my_pos - (b0 + 4u * hh));
+                const int below = dist - (int)window;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int o = 8 * (i >> 2) + (i & 3);
+                    st[i] = (o <= dist && o > below) ? st[i] : LNG_NEG_INF;
+                }
+            }
+            // the running maximum only moves when the block's exceeds it by PF_TAU (see prefill_body)
+            float tmax = LNG_NEG_INF;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, st[i]);
+            tmax = other_half_max(tmax) * sl2; // the host sends only positive factors this way
+            const float m_new = tmax > m + PF_TAU ? tmax : m;
+            const float m_safe = m_new == LNG_NEG_INF ? 0.0f : m_new;
+            if (__builtin_amdgcn_ballot_w64(m_new != m) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+                l *= alpha;
+#pragma unroll
+                for (int db = 0; db < 2; ++db) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) ot[db][i] *= alpha;
+                }
+                m = m_new;
+            }
+            bf16x8 pb[2];
+            float psum[2] = {0.0f, 0.0f};
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                for (int e = 0; e < 8; e += 2) {
+                    bf16x2 pr;
+                    pr[0] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(st[8 * jj + e], sl2, -m_safe));
+                    pr[1] = (__bf16)__builtin_amdgcn_exp2f(__builtin_fmaf(st[8 * jj + e + 1], sl2, -m_safe));
+                    pb[jj][e] = pr[0];
+                    pb[jj][e + 1] = pr[1];
+                    psum[jj] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, psum[jj], false); // the sum of the rounded weights
+                }
+            }
+            l += psum[0] + psum[1];
+#pragma unroll
+            for (int jj = 0; jj < 2; ++jj) {
+#pragma unroll
+                for (int db = 0; db < 2; ++db) ot[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[jj][db], pb[jj], ot[db], 0, 0, 0);
+            }
+        }
+    }
+    __syncthreads(); // K and V are dead: the outputs go through their place (32 rows of 144 bytes per wavefront)
+    if (!wave_active) return;
+    const float total = l + __shfl_xor(l, 32, 64);
+    const float inv = total > 0.0f ? 1.0f / total : 0.0f;
+    uint16_t *stage = wave < 4u ? s_k + wave * (32u * 72u) : s_v + (wave - 4u) * (32u * 72u);
+#pragma unroll
+    for (int db = 0; db < 2; ++db) {
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            bf16x4 w; // narrowed by the conversion instruction (round to nearest even)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w[i] = (__bf16)(ot[db][4 * blk + i] * inv);
+            *(bf16x4 *)(stage + n * 72u + 32 * db + 8 * blk + 4 * hh) = w;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const uint32_t r = 8u * pass + (lane >> 3), ch = lane & 7u;
+        const uint4 piece = *(const uint4 *)(stage + r * 72u + 8u * ch);
+        const uint32_t row = q0 + r;
+        if (row < t) *(uint4 *)((uint16_t *)a.out + ((uint64_t)row * a.heads + head) * 64u + 8u * ch) = piece;
+    }
+}
 
 // =============================================================================================
 // The long full-causal prompt pass (no window, no ring, keys not split): lng_prefill_bf16_d64's
