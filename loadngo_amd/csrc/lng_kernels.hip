@@ -2754,6 +2754,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     const bool wave_active = wave < group; // a wavefront past the group only helps loading
     const uint32_t head = g * group + (wave_active ? wave : 0u);
 
+    // the head's sink: asked for here, with everything else (after the barrier it would be a memory round trip of its own)
+    const float sink_l2 = a.sinks ? a.sinks[head] * LNG_LOG2E : LNG_NEG_INF;
     // the queries as they are: scale x log2(e) rides with the maximum
     const uint32_t my_pos = pos_first + n;
     bf16x8 qreg[4];
@@ -2795,7 +2797,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     floatx16 ot[2];
     float l = 0.0f;
     if (wave_active) {
-        float m = a.sinks ? a.sinks[head] * LNG_LOG2E : LNG_NEG_INF;
+        float m = sink_l2;
         l = (a.sinks && hh == 0) ? 1.0f : 0.0f;
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
