@@ -497,11 +497,13 @@ def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, st
     assert np.abs(got - other).max() <= 2.0 ** -7  # a bf16 step or two at |o| < 1
 
 
-@pytest.mark.parametrize("t,start,heads,kv_heads", [(2048, 1000, 64, 8), (1000, 0, 32, 8)])
-def test_long_causal_pass_gives_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, monkeypatch):
+@pytest.mark.parametrize("t,start,heads,kv_heads,window", [(2048, 1000, 64, 8, FULL), (1000, 0, 32, 8, FULL),
+                                                          (2048, 1000, 64, 8, 128), (1000, 37, 24, 4, 100)])
+def test_long_passes_give_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, window, monkeypatch):
     """The resident kernel's wavefronts pass the tile barrier at two different places of their sequence and share
-    three LDS buffers: 256 launches over the same inputs, each into its own output, all bit for bit the first
-    (an LDS row overwritten early or read late would show as a launch that differs)."""
+    three LDS buffers; the kernel for narrow windows reads rows that other wavefronts' loads wrote straight into
+    LDS: 256 launches over the same inputs, each into its own output, all bit for bit the first (an LDS row
+    overwritten early or read late would show as a launch that differs)."""
     monkeypatch.setenv("LNG_PREFILL_STREAM", "1")
     dim, per_batch, end = 64, 32, start + t
     rows, krows = (t + 31) // 32 * 32, (end + 31) // 32 * 32
@@ -514,7 +516,7 @@ def test_long_causal_pass_gives_the_same_bits_every_launch(gpu, t, start, heads,
             fill.fill_synthetic(C.Slice(0, 0, bufs[i].len), C.BF16, 90 + i, 0.5, 0)
             fill.run()
             fill.drop()
-        shape = C.GroupedShape(t, start, heads, kv_heads, dim, FULL, end, 0.125)
+        shape = C.GroupedShape(t, start, heads, kv_heads, dim, window, end, 0.125)
         first = None
         for _ in range(8):
             batch = gpu.batch(bufs)
