@@ -1003,14 +1003,14 @@ def run_wide_heads(gpu, steps, warmup):
         res = {"bytes": nbytes}
         for name, env in (("sliced", None), ("one_wavefront_per_head", "1")):
             if env:
-                os.environ["LNG_WIDE_GENERIC"] = env
+                gpu.debug_set("LNG_WIDE_GENERIC", env)
             try:
                 for _ in range(max(2, warmup)):
                     go()
                 n = max(steps, 9)
                 t = sorted(go() for _ in range(n))[n // 2]
             finally:
-                os.environ.pop("LNG_WIDE_GENERIC", None)
+                gpu.debug_set("LNG_WIDE_GENERIC", None)
             res[name] = {"gpu_us": t * 1e6, "gbs": nbytes / t / 1e9, "hbm_frac": nbytes / t / 1e9 / HBM_PEAK_GBS}
         out["%d_sequences" % n_seq] = res
         for b in (q, o, k, v):

@@ -95,6 +95,26 @@ int lng_hip_open(int device, lng_gpu **gpu);
 void lng_hip_close(lng_gpu *gpu);
 /* Device name (e.g. "gfx950..."), copied into `name` (NUL-terminated, truncated to `cap`). */
 int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
+/* Development switches. No counterpart in the reference and NOT part of the interface: they pick between kernels
+ * that compute the same thing (tests compare them; experiments time them) and may change or go at any time. Each
+ * has the name of an environment variable, which is read ONCE, at lng_hip_open; afterwards only this call changes
+ * it (`value` NULL puts the default back). Nothing on the record path reads the environment. Calls recorded after
+ * the change see it; it is the caller's business not to change switches while other threads record.
+ *   LNG_DECODE_WGS n         workgroups a decode dispatch aims for (default 4096)
+ *   LNG_FUSE_WGS n           largest decode grid that merges its chunks inside the kernel (default 4 x compute units)
+ *   LNG_DECODE_O3            never the four-wavefront build of the decode kernel
+ *   LNG_MERGE_WIDE           always the chunk merge of one workgroup per query head
+ *   LNG_WIDE_GENERIC         head widths 128-512 row by row on the kernel of one workgroup per (row, head)
+ *   LNG_F32_GENERIC          f32 operands on that kernel only
+ *   LNG_PLAIN_ROW_BY_ROW     the row-by-row operator never takes a prompt-pass kernel
+ *   LNG_WIDE_ROW_BY_ROW      prompt passes of head widths 128-512 row by row on the decode kernels
+ *   LNG_PREFILL_STREAM 0|1   never / whenever possible the prompt-pass kernel whose workgroups walk several query tiles
+ *   LNG_PREFILL_UPFRONT 0    narrow windows on the tile-by-tile kernel
+ *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
+ *   LNG_PREFILL_FUSED 0      split prompt passes always merged by a second dispatch
+ *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups
+ * Read at lng_hip_open only: LNG_HSACO (a code object file to load instead of the embedded one). */
+int lng_hip_debug_set(lng_gpu *gpu, const char *name, const char *value);
 
 /* ---- memory --------------------------------------------------------------------------- */
 

@@ -97,6 +97,7 @@ SYMBOLS = {
     "lng_hip_open": (ctypes.c_int, [ctypes.c_int, ctypes.POINTER(_P)]),
     "lng_hip_close": (None, [_P]),
     "lng_hip_device_name": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.c_size_t]),
+    "lng_hip_debug_set": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.c_char_p]),
     "lng_hip_buffer": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.POINTER(_P)]),
     "lng_hip_resident": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.POINTER(_P)]),
     "lng_hip_buffer_free": (ctypes.c_int, [_P]),
@@ -345,6 +346,11 @@ class Gpu:
         buf = ctypes.create_string_buffer(128)
         _check(library().lng_hip_device_name(self._h, buf, 128))
         return buf.value.decode()
+
+    def debug_set(self, name, value):
+        """A development switch by its environment name (``include/lng_hip.h`` lists them; not part of the
+        interface); ``value`` None puts the default back. The environment itself is read once, at open."""
+        _check(library().lng_hip_debug_set(self._h, name.encode(), None if value is None else str(value).encode()))
 
     def buffer(self, len):
         h = _P()

@@ -57,7 +57,23 @@ const char *hip_text(hipError_t e) { return hipGetErrorString(e); }
 
 size_t elem_size(int dtype) { return dtype == LNG_BF16 ? 2 : 4; }
 
-bool env_is(const char *value, const char *what) { return value && strcmp(value, what) == 0; }
+// Development switches (not part of the interface): read from the environment once, at lng_hip_open, and changed
+// afterwards only through lng_hip_debug_set. Nothing on the record path reads the environment.
+struct Knobs {
+    bool wide_generic = false;     // LNG_WIDE_GENERIC: head widths 128-512 row by row on the kernel of one workgroup per (row, head)
+    bool f32_generic = false;      // LNG_F32_GENERIC: f32 operands on the generic kernel only
+    bool plain_row_by_row = false; // LNG_PLAIN_ROW_BY_ROW: the row-by-row operator never takes a prompt-pass kernel
+    bool decode_o3 = false;        // LNG_DECODE_O3: never the four-wavefront build of the decode kernel
+    bool merge_wide = false;       // LNG_MERGE_WIDE: always the merge of one workgroup per query head
+    bool q8_w16 = false;           // LNG_Q8_W16: the one-position Q8_0 kernel always as 16-wavefront workgroups
+    bool wide_row_by_row = false;  // LNG_WIDE_ROW_BY_ROW: prompt passes of head widths 128-512 row by row on the decode kernels
+    int prefill_stream = -1;       // LNG_PREFILL_STREAM: 0 never the resident prompt-pass kernel, 1 whenever it can run, -1 planner
+    int prefill_upfront = -1;      // LNG_PREFILL_UPFRONT: 0 narrow windows on the tile-by-tile kernel
+    int prefill_splits = 0;        // LNG_PREFILL_SPLITS: workgroups per (query tile, kv head) of a split prompt pass; 0 planner
+    int prefill_fused = -1;        // LNG_PREFILL_FUSED: 0 split prompt passes always merged by lng_prefill_merge, -1 planner
+    long decode_wgs = 0;           // LNG_DECODE_WGS: workgroups a decode dispatch aims for; 0 default
+    long fuse_wgs = -1;            // LNG_FUSE_WGS: largest grid that merges inside the decode kernel; -1 default
+};
 
 struct Table { // one pinned-host / device pair holding row tables of batched dispatches
     char *host = nullptr;
@@ -110,10 +126,10 @@ struct lng_gpu {
     char *scratch_x = nullptr;   // bf16 planes of the positions of a Q8_0 product
     size_t scratch_x_len = 0;
     std::vector<void *> retired; // outgrown scratch, freed at close (dispatches may name it)
-    std::atomic<long> live_buffers{0}; // buffers, residents and batches that still name this gpu
-    std::atomic<bool> closed{false};   // lng_hip_close was called while some were alive: the last one to go frees the gpu
+    std::atomic<long> live_buffers{1}; // the open handle, and the buffers, residents and batches that still name this gpu
     unsigned decode_wgs = 4096; // workgroups a decode dispatch aims for
     uint64_t fuse_wgs = 1024;   // decode dispatches of up to this many workgroups merge their chunks in the kernel
+    Knobs knobs;                // development switches, see lng_hip_debug_set
     char *static_scratch = nullptr; // this device's copy of the fixed scratch array (LNG_STATIC_SCRATCH_BYTES)
 
     // completion thread (only for batches committed with a callback)
@@ -240,6 +256,41 @@ int check_shape(const lng_grouped_shape &s, bool tiled) {
     return LNG_OK;
 }
 
+// One development switch by its environment name; value NULL puts the default back. Returns false for an unknown name.
+const char *const knob_names[] = {"LNG_WIDE_GENERIC", "LNG_F32_GENERIC", "LNG_PLAIN_ROW_BY_ROW", "LNG_DECODE_O3", "LNG_MERGE_WIDE",
+                                  "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_UPFRONT",
+                                  "LNG_PREFILL_SPLITS", "LNG_PREFILL_FUSED", "LNG_DECODE_WGS", "LNG_FUSE_WGS"};
+bool set_knob(lng_gpu *g, const char *name, const char *value) {
+    Knobs &k = g->knobs;
+    const Knobs defaults;
+    const long n = value ? atol(value) : 0;
+    auto flag = [&](bool &field) { field = value != nullptr; return true; }; // present, whatever it holds: on
+    auto choice = [&](int &field, int dflt) { field = value ? (int)n : dflt; return true; };
+    if (!strcmp(name, "LNG_WIDE_GENERIC")) return flag(k.wide_generic);
+    if (!strcmp(name, "LNG_F32_GENERIC")) return flag(k.f32_generic);
+    if (!strcmp(name, "LNG_PLAIN_ROW_BY_ROW")) return flag(k.plain_row_by_row);
+    if (!strcmp(name, "LNG_DECODE_O3")) return flag(k.decode_o3);
+    if (!strcmp(name, "LNG_MERGE_WIDE")) return flag(k.merge_wide);
+    if (!strcmp(name, "LNG_Q8_W16")) return flag(k.q8_w16);
+    if (!strcmp(name, "LNG_WIDE_ROW_BY_ROW")) return flag(k.wide_row_by_row);
+    if (!strcmp(name, "LNG_PREFILL_STREAM")) return choice(k.prefill_stream, defaults.prefill_stream);
+    if (!strcmp(name, "LNG_PREFILL_UPFRONT")) return choice(k.prefill_upfront, defaults.prefill_upfront);
+    if (!strcmp(name, "LNG_PREFILL_FUSED")) return choice(k.prefill_fused, defaults.prefill_fused);
+    if (!strcmp(name, "LNG_PREFILL_SPLITS")) {
+        k.prefill_splits = value ? (int)std::max(1l, std::min(n, 64l)) : 0;
+        return true;
+    }
+    if (!strcmp(name, "LNG_DECODE_WGS")) {
+        g->decode_wgs = value && n >= 1 && n <= (1 << 20) ? (unsigned)n : 4096u;
+        return true;
+    }
+    if (!strcmp(name, "LNG_FUSE_WGS")) {
+        g->fuse_wgs = value && n >= 0 ? (uint64_t)n : 4ull * g->cus;
+        return true;
+    }
+    return false;
+}
+
 int need_recording(lng_batch *b) {
     if (!b) return fail(LNG_ERR_DISPATCH, "no batch");
     if (b->state != lng_batch::Recording) return fail(LNG_ERR_DISPATCH, "the batch was already committed");
@@ -253,7 +304,14 @@ template <typename A> void set_args(Cmd &c, const A &a) {
 
 // Device scratch for split-K partials, shared by every dispatch of the gpu: dispatches run
 // in order on one stream, so the next one starts after the previous combine has read it.
-int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats, size_t n_tickets) {
+// The three pointers are handed out as they were under the lock: a batch recorded on another thread may grow and
+// swap them right after (the outgrown ones stay allocated until close, so a dispatch recorded with them is safe).
+struct Scratch {
+    float *o = nullptr;
+    float *ml = nullptr;
+    uint32_t *tickets = nullptr;
+};
+int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats, size_t n_tickets, Scratch *out) {
     std::lock_guard<std::mutex> lock(g->mu);
     if (n_tickets > g->tickets_len) {
         void *p = nullptr;
@@ -285,6 +343,9 @@ int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats, size_t n_tick
         g->scratch_ml = (float *)p;
         g->scratch_ml_len = want;
     }
+    out->o = g->scratch_o;
+    out->ml = g->scratch_ml;
+    out->tickets = g->tickets;
     return LNG_OK;
 }
 
@@ -464,14 +525,14 @@ RowsPlan plan_rows(lng_gpu *g, const lng_k_attn &a, const lng_k_row *host_rows, 
     // Head widths the matrix kernels serve: 64 (gpt-oss), and 128, 256, 512 in slices of 64. Anything else, groups of
     // more than 16 query heads and operands off 16-byte boundaries go to the kernel of one wavefront per (row, head).
     const int wide = a.dim == 128 ? 0 : a.dim == 256 ? 1 : a.dim == 512 ? 2 : -1;
-    const bool dim_ok = a.dim == 64 || (wide >= 0 && !getenv("LNG_WIDE_GENERIC"));
+    const bool dim_ok = a.dim == 64 || (wide >= 0 && !g->knobs.wide_generic);
     const bool fast = a.dtype == LNG_BF16 && dim_ok && group <= 16 && aligned16;
     // f32 (the reference's own element type) at the gpt-oss head width: the same chunks and partials on the f32 matrix instruction
     // (that kernel counts positions in 32 bits and steps by up to 256 chunks x 128 positions past the last one)
     uint64_t latest = t_uniform ? host_rows[0].start + t_uniform - 1 : 0;
     for (size_t i = 0; !t_uniform && i < n_rows; ++i) latest = std::max(latest, host_rows[i].start);
     const bool fast_f32 = a.dtype == LNG_F32 && dim_ok && group <= 16 && aligned16 && latest < 0xffff0000ull &&
-                          a.scale > 0.0f && a.scale <= 3.0e38f && !getenv("LNG_F32_GENERIC");
+                          a.scale > 0.0f && a.scale <= 3.0e38f && !g->knobs.f32_generic;
     p.pairs = n_rows * (size_t)a.kv_heads;
     if (!fast && !fast_f32) return p;
     p.kind = fast ? RowsPlan::Bf16 : RowsPlan::F32;
@@ -537,12 +598,12 @@ int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *
                             p.kind == RowsPlan::Bf16 ? wide_bf16[p.wide] : wide_f32[p.wide], (unsigned)wgs, a};
     } else {
         // (many workgroups of short chunks - a table of sequences: the build of the bf16 kernel with four wavefronts per SIMD)
-        const bool o4 = p.kind == RowsPlan::Bf16 && a.chunk < 2048u && wgs > 3ull * g->cus && !getenv("LNG_DECODE_O3");
+        const bool o4 = p.kind == RowsPlan::Bf16 && a.chunk < 2048u && wgs > 3ull * g->cus && !g->knobs.decode_o3;
         out->l[out->n++] = {p.kind == RowsPlan::Bf16 ? (o4 ? g->decode_bf16_d64_o4 : g->decode_bf16_d64) : g->decode_f32_d64,
                             p.kind == RowsPlan::Bf16 ? (o4 ? "lng_decode_bf16_d64_o4" : "lng_decode_bf16_d64") : "lng_decode_f32_d64", (unsigned)wgs, a};
     }
     if (a.n_chunks > 1 && !a.fused) {
-        if (a.n_chunks <= 8 && !getenv("LNG_MERGE_WIDE")) { // a wavefront per (row, kv head, query head), four to a workgroup
+        if (a.n_chunks <= 8 && !g->knobs.merge_wide) { // a wavefront per (row, kv head, query head), four to a workgroup
             out->l[out->n++] = {g->decode_merge_few, "lng_decode_merge_few", (unsigned)(p.pairs * ((group + 3) / 4)), a};
         } else {                                            // a workgroup per (row, kv head, query head)
             out->l[out->n++] = {g->decode_merge, "lng_decode_merge", (unsigned)(p.pairs * group), a};
@@ -557,10 +618,11 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
     lng_gpu *g = b->gpu;
     const RowsPlan p = plan_rows(g, a, host_rows, n_rows, t_uniform, aligned16);
     if (p.partial_slots) {
-        if (int rc = reserve_scratch(g, p.partial_slots * a.dim, p.partial_slots * 2, p.pairs)) return rc;
-        a.partial_o = g->scratch_o;
-        a.partial_ml = g->scratch_ml;
-        a.tickets = g->tickets;
+        Scratch sc;
+        if (int rc = reserve_scratch(g, p.partial_slots * a.dim, p.partial_slots * 2, p.pairs, &sc)) return rc;
+        a.partial_o = sc.o;
+        a.partial_ml = sc.ml;
+        a.tickets = sc.tickets;
     }
     // Rows of unequal length (a table of sequences): room for the running counts of live workgroups.
     char *work_host = nullptr, *work_dev = nullptr;
@@ -623,13 +685,13 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
     // Measured break-even on 64/8 heads: rows x visible keys of about 32 K at 2,048 keys (16 rows), 16 K from 4,096 keys on.
     const uint64_t seen = std::min<uint64_t>(end, s.window > UINT64_MAX - s.t ? UINT64_MAX : s.window + s.t);
     const bool several_rows = !tiled && s.t >= 4 && seen >= 1024 && (s.t * seen >= 32768 || (seen >= 4096 && s.t * seen >= 16384)) &&
-                              !getenv("LNG_PLAIN_ROW_BY_ROW");
+                              !b->gpu->knobs.plain_row_by_row;
     // (the matrix kernels take the maximum of the raw products and scale it afterwards: scale > 0; any other
     // scale goes to the kernels that scale first)
     const bool scale_positive = s.scale > 0.0f && s.scale <= 3.0e38f;
     // (the prompt-pass kernels compare distances between positions as signed 32-bit numbers)
     if ((tiled || several_rows) && s.dim == 64 && s.heads / s.kv_heads <= 8 && aligned16 && scale_positive && end <= 0x7fffffffull &&
-        (dtype == LNG_BF16 || !getenv("LNG_F32_GENERIC"))) {
+        (dtype == LNG_BF16 || !g->knobs.f32_generic)) {
         const bool f32 = dtype == LNG_F32;
         lng_k_prefill p{};
         p.dtype = (uint32_t)dtype;
@@ -667,21 +729,21 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const uint64_t plain_wgs = (uint64_t)p.q_tiles * s.kv_heads;
         // LNG_PREFILL_STREAM: 0 never takes the kernel of workgroups that walk several query tiles, 1 takes it for
         // every full-causal pass it can run (tests: small shapes), otherwise only when every compute unit has a tile.
-        const char *stream_env = getenv("LNG_PREFILL_STREAM");
-        const bool stream_can = !f32 && !narrow && p.window == LNG_WINDOW_FULL && s.slots >= end && !env_is(stream_env, "0");
-        const bool stream = stream_can && (plain_wgs >= g->cus || env_is(stream_env, "1"));
+        const bool stream_can = !f32 && !narrow && p.window == LNG_WINDOW_FULL && s.slots >= end && g->knobs.prefill_stream != 0;
+        const bool stream = stream_can && (plain_wgs >= g->cus || g->knobs.prefill_stream == 1);
         if (!stream && (!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
             uint64_t want = g->cus / plain_wgs;
             want = std::min<uint64_t>(want, key_tiles / 4);
             want = std::min<uint64_t>(want, 64);
-            if (const char *env = getenv("LNG_PREFILL_SPLITS")) want = std::min<uint64_t>(std::max(1, atoi(env)), 64);
+            if (g->knobs.prefill_splits > 0) want = std::min<uint64_t>(g->knobs.prefill_splits, 64);
             if (want > 1) p.splits = (uint32_t)want;
         }
         if (p.splits > 1) {
             const size_t slots = (size_t)s.t * s.heads * p.splits;
-            if (int rc = reserve_scratch(g, slots * 64, slots * 2, 0)) return rc;
-            p.partial_o = g->scratch_o;
-            p.partial_ml = g->scratch_ml;
+            Scratch sc;
+            if (int rc = reserve_scratch(g, slots * 64, slots * 2, 0, &sc)) return rc;
+            p.partial_o = sc.o;
+            p.partial_ml = sc.ml;
         }
         // The long full-causal pass with every compute unit busy anyway: one workgroup per compute unit that stays
         // there and walks several query tiles (balanced by construction, no per-workgroup start-up between them).
@@ -696,7 +758,7 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const bool f32_two = f32 && c.grid[0] >= 4u * g->cus;
         // Windows of up to 160 positions: the 32 query rows of a workgroup see at most four tiles of 64 keys, and the
         // one-head kernel asks for all of them at its start, straight into LDS (LNG_PREFILL_UPFRONT=0: never).
-        const bool upfront = narrow && p.window != LNG_WINDOW_FULL && p.window <= 160 && p.splits == 1 && !env_is(getenv("LNG_PREFILL_UPFRONT"), "0");
+        const bool upfront = narrow && p.window != LNG_WINDOW_FULL && p.window <= 160 && p.splits == 1 && g->knobs.prefill_upfront != 0;
         c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : upfront ? g->prefill_bf16_d64_h1w : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : g->prefill_bf16_d64;
         c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : upfront ? "lng_prefill_bf16_d64_h1w" : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : "lng_prefill_bf16_d64";
         set_args(c, p);
@@ -842,15 +904,18 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
     }
     g->static_scratch = (char *)lng_static_scratch(device);
     g->fuse_wgs = 4ull * g->cus;
-    if (const char *env = getenv("LNG_FUSE_WGS")) {
-        const long n = atol(env);
-        if (n >= 0) g->fuse_wgs = (uint64_t)n;
-    }
-    if (const char *env = getenv("LNG_DECODE_WGS")) {
-        const long n = atol(env);
-        if (n >= 1 && n <= (1 << 20)) g->decode_wgs = (unsigned)n;
+    // the development switches, read once here
+    for (const char *name : knob_names) {
+        if (const char *value = getenv(name)) set_knob(g, name, value);
     }
     *out = g;
+    return LNG_OK;
+}
+
+extern "C" int lng_hip_debug_set(lng_gpu *g, const char *name, const char *value) {
+    if (!g || !name) return fail(LNG_ERR_DISPATCH, "no gpu or no name");
+    std::lock_guard<std::mutex> lock(g->mu);
+    if (!set_knob(g, name, value)) return fail(LNG_ERR_DISPATCH, "no development switch called %s", name);
     return LNG_OK;
 }
 
@@ -871,9 +936,10 @@ void destroy_gpu(lng_gpu *g) {
     delete g;
 }
 
-// A buffer or batch of `g` went away: the last one after lng_hip_close takes the gpu with it.
+// A buffer, a batch or the open handle of `g` went away: whoever takes the count to zero takes the gpu with it.
+// Nothing of `g` is read after the decrement, so the last two holders may let go on different threads.
 void object_gone(lng_gpu *g) {
-    if (g->live_buffers.fetch_sub(1) == 1 && g->closed.load()) destroy_gpu(g);
+    if (g->live_buffers.fetch_sub(1, std::memory_order_acq_rel) == 1) destroy_gpu(g);
 }
 } // namespace
 
@@ -891,9 +957,7 @@ extern "C" void lng_hip_close(lng_gpu *g) {
     hipStreamSynchronize(g->stream);
     // Buffers, residents and batches keep the gpu alive, as the reference's own do (they borrow or share it): with
     // some still around, the handle stays valid for freeing and dropping them and goes with the last of them.
-    g->live_buffers.fetch_add(1);
-    g->closed.store(true);
-    object_gone(g);
+    object_gone(g); // the handle's own reference, held since lng_hip_open
 }
 
 extern "C" int lng_hip_device_name(lng_gpu *g, char *name, size_t cap) {
@@ -1654,7 +1718,7 @@ int q8_check(lng_batch *b, const lng_slice &codes, const lng_slice &scales, cons
 void q8_record_stream(lng_batch *b, const lng_k_q8 &a, uint64_t row_tiles, bool x_bf16) {
     const bool one = a.n == 1 && a.cols <= 12288 && !x_bf16; // x of a single position is held in LDS (Q8S_X1 floats)
     // more row tiles than compute units (several matrices): 8-wavefront workgroups, two per unit, one round
-    const bool w8 = one && row_tiles > b->gpu->cus && !getenv("LNG_Q8_W16");
+    const bool w8 = one && row_tiles > b->gpu->cus && !b->gpu->knobs.q8_w16;
     Cmd c;
     c.fn = x_bf16 ? b->gpu->q8_stream_bf16 : w8 ? b->gpu->q8_stream_one_w8 : one ? b->gpu->q8_stream_one : b->gpu->q8_stream;
     c.name = x_bf16 ? "lng_q8_stream_bf16" : w8 ? "lng_q8_stream_one_w8" : one ? "lng_q8_stream_one" : "lng_q8_stream";

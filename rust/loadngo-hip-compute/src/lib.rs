@@ -128,6 +128,19 @@ impl Gpu {
         unsafe { CStr::from_ptr(text.as_ptr()) }.to_string_lossy().into_owned()
     }
 
+    /// A development switch by its environment name (the header lists them; not part of the interface, no
+    /// counterpart in metal-compute). `None` puts the default back. The environment itself is read once, in `new`.
+    pub fn debug_set(&self, name: &str, value: Option<&str>) -> Result<(), Error> {
+        let name = CString::new(name).map_err(|_| Error::Dispatch("a switch name holds a NUL".into()))?;
+        let value = match value {
+            Some(v) => Some(CString::new(v).map_err(|_| Error::Dispatch("a switch value holds a NUL".into()))?),
+            None => None,
+        };
+        let value_ptr = value.as_ref().map_or(ptr::null(), |v| v.as_ptr());
+        // SAFETY: both strings are NUL-terminated and outlive the call.
+        check(unsafe { ffi::lng_hip_debug_set(self.raw.as_ptr(), name.as_ptr(), value_ptr) })
+    }
+
     /// Device memory of `len` bytes, contents unspecified (`apple.rs:255`). `len == 0` is `Alloc(0)`.
     pub fn buffer(&self, len: usize) -> Result<Buffer, Error> {
         let mut raw = ptr::null_mut();

@@ -15,6 +15,34 @@ def gpu():
     g.close()
 
 
+class _Knobs:
+    """Development switches of the session's device for one test (``lng_hip_debug_set``); the library reads the
+    environment only when a device is opened, so tests that pick a kernel go through this. Defaults come back at
+    the end of the test."""
+
+    def __init__(self, gpu):
+        self._gpu, self._touched = gpu, set()
+
+    def setenv(self, name, value):
+        self._touched.add(name)
+        self._gpu.debug_set(name, value)
+
+    def delenv(self, name, raising=True):
+        self._touched.add(name)
+        self._gpu.debug_set(name, None)
+
+    def restore(self):
+        for name in self._touched:
+            self._gpu.debug_set(name, None)
+
+
+@pytest.fixture
+def knobs(gpu):
+    k = _Knobs(gpu)
+    yield k
+    k.restore()
+
+
 def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out=True):
     """One dispatch as the reference's test harness lays it out (attention_grouped.rs:102-158):
     five buffers (q, k, v, out, sinks), slices over all of each. q is [t][H][D]; for the tiled

@@ -8,7 +8,7 @@ import pytest
 
 from loadngo_amd import compute as C
 from oracle import oracle
-from tests.gpu_common import THREADS, gpu, max_error, reference_case, run_attention  # noqa: F401
+from tests.gpu_common import THREADS, gpu, knobs, max_error, reference_case, run_attention  # noqa: F401
 from tests.helpers import (FULL, REF_GPT_OSS_CASES, REF_PLAIN_CASES, REF_REJECTED, REF_TILED_CASES,
                            from_bf16_bits, normal_inputs, ring_layout, to_bf16_bits)
 
@@ -317,13 +317,13 @@ def test_prefill_bf16_matches_the_cpu_reference(gpu, t, start, window, slots, he
     # up to 32 rows: the 32-row form of the kernel, with splits
     (32, 4064, FULL, 4096, None), (20, 5000, FULL, 5024, None), (7, 9000, 4000, 4032, "9"),
 ])
-def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots, forced, monkeypatch):
+def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots, forced, knobs):
     """A chunk of a long prompt (the reference passes 512 rows at a time, engine.rs:51), or a few rows late
     in a long context: too few query tiles to fill the device, so the keys of a tile are split between
     workgroups and merged afterwards. Same bound as the unsplit pass; LNG_PREFILL_SPLITS forces split counts
     that leave some workgroups without a tile, or with edge tiles only."""
     if forced:
-        monkeypatch.setenv("LNG_PREFILL_SPLITS", forced)
+        knobs.setenv("LNG_PREFILL_SPLITS", forced)
     heads, kv_heads = 64, 8
     end = start + t
     q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
@@ -338,7 +338,7 @@ def test_prefill_bf16_few_query_rows_over_many_keys(gpu, t, start, window, slots
 
 @pytest.mark.parametrize("t,start,window,slots", [(8, 5000, FULL, 5008), (31, 3000, 2000, 2031), (4, 9000, FULL, 9100),
                                                   (16, 2100, FULL, 2116), (31, 40000, 1100, 1131), (5, 7000, 6999, 7004)])
-def test_several_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, monkeypatch):
+def test_several_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, knobs):
     """attention_grouped with a handful of rows over thousands of keys (the tail of a prompt: gpu.rs:760-806
     takes this operator below 32 rows) is served by the prompt-pass kernel, which reads the cache once instead
     of once per row. Same results as row by row (LNG_PLAIN_ROW_BY_ROW) and as the CPU reference; rows of the
@@ -357,19 +357,19 @@ def test_several_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, s
     want = from_bf16_bits(oracle.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS))
     got = from_bf16_bits(run_attention(gpu, qb, kr, vr, sinks, shape, False, C.BF16))
     assert not np.isnan(got).any() and max_error(got, want) < BF16_TOL
-    monkeypatch.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
+    knobs.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
     rows = from_bf16_bits(run_attention(gpu, qb, kr, vr, sinks, shape, False, C.BF16))
     assert max_error(rows, want) < BF16_TOL and np.abs(rows - got).max() < 2.0 ** -6
 
 
 @pytest.mark.parametrize("stream", ["0", "1"])
 @pytest.mark.parametrize("spike_at,sinks_on", [(300, True), (300, False), (5, True), (5, False), (700, True)])
-def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on, stream, monkeypatch):
+def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on, stream, knobs):
     """Long causal passes first keep the running maximum fixed after one interior tile and check the
     normalisers afterwards. A key whose score is about 10,000 above the rest (2^10000 cannot be held)
     late in the pass must send the workgroup through the pass that tracks the maximum; the same key
     early in the pass, or a cache whose scores all sit far below the first tile's, must not lose anything."""
-    monkeypatch.setenv("LNG_PREFILL_STREAM", stream)  # both kernels of the long causal pass (see the next test)
+    knobs.setenv("LNG_PREFILL_STREAM", stream)  # both kernels of the long causal pass (see the next test)
     t, heads, kv_heads = 1024, 16, 2
     q, k, v, sinks = normal_inputs(91 + spike_at, t, t, heads, kv_heads, 64, scale=0.5)
     q[:] = np.abs(q) + 1.0                      # every query has a large positive overlap with the spike key
@@ -425,7 +425,7 @@ def test_windowed_prefill_with_scores_far_outside_the_usual_range(gpu, case, win
     (97, 31, 40, 128, 16, 4), (65, 3, 1, 96, 8, 8), (130, 1000, 128, 320, 4, 1), (40, 97, 7, 64, 10, 2),
     (31, 900, 100, 160, 64, 8),     # fewer than 32 rows, in a ring that wraps
 ])
-def test_narrow_windows_with_every_row_requested_up_front(gpu, t, start, window, slots, heads, kv_heads, monkeypatch):
+def test_narrow_windows_with_every_row_requested_up_front(gpu, t, start, window, slots, heads, kv_heads, knobs):
     """Windows of up to 160 positions run the kernel that asks for all of a workgroup's K and V rows at its start,
     by loads that write LDS directly into swizzled rows: it is the kernel the dispatch names, it agrees with the CPU
     reference, and it gives the bits of the tile-by-tile kernel (same arithmetic in the same order; a wrong swizzle
@@ -463,7 +463,7 @@ def test_narrow_windows_with_every_row_requested_up_front(gpu, t, start, window,
 
     got = run("lng_prefill_bf16_d64_h1w")
     assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
-    monkeypatch.setenv("LNG_PREFILL_UPFRONT", "0")
+    knobs.setenv("LNG_PREFILL_UPFRONT", "0")
     tile_by_tile = run("lng_prefill_bf16_d64_h1")
     assert np.array_equal(got, tile_by_tile)
 
@@ -471,7 +471,7 @@ def test_narrow_windows_with_every_row_requested_up_front(gpu, t, start, window,
 @pytest.mark.parametrize("t,start,heads,kv_heads,sinks_on", [
     (300, 0, 64, 8, True), (1000, 0, 32, 8, True), (777, 1300, 64, 8, False), (64, 0, 16, 2, True), (65, 63, 8, 1, True),
     (130, 4000, 24, 8, True), (2048, 0, 64, 8, True)])
-def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, start, heads, kv_heads, sinks_on, monkeypatch):
+def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, start, heads, kv_heads, sinks_on, knobs):
     """lng_prefill_bf16_d64_stream (one resident workgroup per compute unit, query tiles dealt out in a snake,
     K/V tiles through three LDS buffers, the interior in matrix and arithmetic phases with the second wavefront of
     every SIMD one phase behind and the normaliser summed by the matrix unit): forced for shapes of every kind it
@@ -484,9 +484,9 @@ def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, st
     kr, vr = ring_layout(kb, t, start, end, True), ring_layout(vb, t, start, end, True)
     shape = C.GroupedShape(t, start, heads, kv_heads, 64, FULL, end, 0.125)
     sk = sinks if sinks_on else None
-    monkeypatch.setenv("LNG_PREFILL_STREAM", "1")
+    knobs.setenv("LNG_PREFILL_STREAM", "1")
     got = from_bf16_bits(run_attention(gpu, qb, kr, vr, sk, shape, True, C.BF16))
-    monkeypatch.setenv("LNG_PREFILL_STREAM", "0")
+    knobs.setenv("LNG_PREFILL_STREAM", "0")
     other = from_bf16_bits(run_attention(gpu, qb, kr, vr, sk, shape, True, C.BF16))
     rows = sorted(set([0, 1, 31, 32, 63, 64, t - 1] + [int(x) for x in np.random.default_rng(t).integers(0, t, 24)]))
     rows = [r for r in rows if r < t]
@@ -499,12 +499,12 @@ def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, st
 
 @pytest.mark.parametrize("t,start,heads,kv_heads,window", [(2048, 1000, 64, 8, FULL), (1000, 0, 32, 8, FULL),
                                                           (2048, 1000, 64, 8, 128), (1000, 37, 24, 4, 100)])
-def test_long_passes_give_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, window, monkeypatch):
+def test_long_passes_give_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, window, knobs):
     """The resident kernel's wavefronts pass the tile barrier at two different places of their sequence and share
     three LDS buffers; the kernel for narrow windows reads rows that other wavefronts' loads wrote straight into
     LDS: 256 launches over the same inputs, each into its own output, all bit for bit the first (an LDS row
     overwritten early or read late would show as a launch that differs)."""
-    monkeypatch.setenv("LNG_PREFILL_STREAM", "1")
+    knobs.setenv("LNG_PREFILL_STREAM", "1")
     dim, per_batch, end = 64, 32, start + t
     rows, krows = (t + 31) // 32 * 32, (end + 31) // 32 * 32
     one = rows * heads * dim * 2
@@ -656,7 +656,7 @@ def test_decode_bf16_one_long_row(gpu, start, window, slots, heads, kv_heads):
     (31, 100, FULL, 131, 5, 1), (2, 9000, 1, 3, 64, 8), (5, 260, 300, 305, 24, 8), (1, 5000, FULL, 5001, 32, 2),
     (3, 700, 100, 128, 12, 1), (2, 40, 17, 19, 16, 1), (1, 31, FULL, 32, 64, 8), (1, 0, FULL, 1, 64, 8),
 ])
-def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_heads, monkeypatch):
+def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_heads, knobs):
     """The row-by-row operator on f32 caches: groupings up to 16 heads per kv head, one chunk and many
     (merged by a second dispatch), rings that have wrapped, windows that start inside a tile, with and without
     sinks; rows the operator must not read hold NaN (attention_grouped.rs:57). Within 1e-5 (relative to
@@ -677,9 +677,9 @@ def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_hea
         want = oracle.attention_f32(q, kz, vz, sinks, start, window=window, slots=None, scale=0.125, threads=THREADS)
         got = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
         assert rel_error(got, want) <= F32_RTOL
-        monkeypatch.setenv("LNG_F32_GENERIC", "1")
+        knobs.setenv("LNG_F32_GENERIC", "1")
         generic = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
-        monkeypatch.delenv("LNG_F32_GENERIC")
+        knobs.delenv("LNG_F32_GENERIC")
         assert rel_error(generic, want) <= F32_RTOL
 
 
@@ -694,13 +694,13 @@ def test_decode_f32_at_head_width_64(gpu, t, start, window, slots, heads, kv_hea
     # a thousand workgroups and more: the build of the kernel with two workgroups per compute unit
     (4096, 0, 128, 4096, 8, 8, None), (4096, 0, FULL, 4096, 8, 8, None), (2080, 3000, 300, 2400, 32, 8, None),
 ])
-def test_prefill_f32_matches_the_cpu_reference(gpu, t, start, window, slots, heads, kv_heads, forced, monkeypatch):
+def test_prefill_f32_matches_the_cpu_reference(gpu, t, start, window, slots, heads, kv_heads, forced, knobs):
     """The tiled operator on f32 operands at head width 64 (the reference's own prompt pass, gpu.rs:760-806):
     within 1e-5 (relative to 1 + |x|) of the CPU reference, with and without sinks, rings, windows, ragged
     last tiles, groupings from 1 to 8, keys split between workgroups (by the library's own choice and forced
     through LNG_PREFILL_SPLITS); the generic kernel (LNG_F32_GENERIC) agrees."""
     if forced:
-        monkeypatch.setenv("LNG_PREFILL_SPLITS", forced)
+        knobs.setenv("LNG_PREFILL_SPLITS", forced)
     end = start + t
     q, k, v, sinks = normal_inputs(t + start, t, end, heads, kv_heads, 64, scale=0.5)
     kr, vr = ring_layout(k, t, start, slots, True), ring_layout(v, t, start, slots, True)
@@ -709,14 +709,14 @@ def test_prefill_f32_matches_the_cpu_reference(gpu, t, start, window, slots, hea
         want = oracle.attention_f32(q, k, v, sk, start, window=window, slots=None, scale=0.125, threads=THREADS)
         got = run_attention(gpu, q, kr, vr, sk, shape, True, C.F32)
         assert rel_error(got, want) <= F32_RTOL
-    monkeypatch.setenv("LNG_F32_GENERIC", "1")
+    knobs.setenv("LNG_F32_GENERIC", "1")
     generic = run_attention(gpu, q, kr, vr, None, shape, True, C.F32)
     assert rel_error(generic, want) <= F32_RTOL
 
 
 @pytest.mark.parametrize("t,start,window,slots", [(8, 5000, FULL, 5008), (31, 3000, 2000, 2031), (16, 2100, FULL, 2116),
                                                   (5, 7000, 6999, 7004)])
-def test_several_f32_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, monkeypatch):
+def test_several_f32_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, start, window, slots, knobs):
     """attention_grouped on f32 caches with a handful of rows over thousands of keys goes through the f32
     prompt-pass kernel; same results as row by row (LNG_PLAIN_ROW_BY_ROW) and as the CPU reference; cache rows
     outside [first visible, last] hold NaN, and rings need not be multiples of 32 rows."""
@@ -732,7 +732,7 @@ def test_several_f32_rows_through_the_row_by_row_operator_over_long_caches(gpu, 
     want = oracle.attention_f32(q, k, v, sinks, start, window=window, slots=None, scale=0.125, threads=THREADS)
     got = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
     assert rel_error(got, want) <= F32_RTOL
-    monkeypatch.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
+    knobs.setenv("LNG_PLAIN_ROW_BY_ROW", "1")
     rows = run_attention(gpu, q, kr, vr, sinks, shape, False, C.F32)
     assert rel_error(rows, want) <= F32_RTOL
 
@@ -774,7 +774,7 @@ WIDE_CASES = [
 
 @pytest.mark.parametrize("dtype", [C.BF16, C.F32])
 @pytest.mark.parametrize("t,start,window,slots,heads,kv_heads,dim", WIDE_CASES)
-def test_decode_at_head_widths_128_256_512(gpu, dtype, t, start, window, slots, heads, kv_heads, dim, monkeypatch):
+def test_decode_at_head_widths_128_256_512(gpu, dtype, t, start, window, slots, heads, kv_heads, dim, knobs):
     """The row-by-row operator at the wider heads: one chunk and many (merged by a second dispatch), rings that
     have wrapped, windows that start inside a tile, groups of 1..16, with and without sinks; rows the operator must
     not read hold NaN (attention_grouped.rs:57). To the bars of the width-64 kernels against the CPU reference, and
@@ -805,9 +805,9 @@ def test_decode_at_head_widths_128_256_512(gpu, dtype, t, start, window, slots, 
             bar = BF16_TOL
         got = run_attention(gpu, q, kr, vr, sinks, shape, False, dtype)
         assert err(got) <= bar
-        monkeypatch.setenv("LNG_WIDE_GENERIC", "1")
+        knobs.setenv("LNG_WIDE_GENERIC", "1")
         generic = run_attention(gpu, q, kr, vr, sinks, shape, False, dtype)
-        monkeypatch.delenv("LNG_WIDE_GENERIC")
+        knobs.delenv("LNG_WIDE_GENERIC")
         assert err(generic) <= bar
 
 

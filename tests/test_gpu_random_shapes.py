@@ -8,7 +8,7 @@ import pytest
 
 from loadngo_amd import compute as C
 from oracle import oracle as orc
-from tests.gpu_common import THREADS, gpu, max_error, run_attention  # noqa: F401
+from tests.gpu_common import THREADS, gpu, knobs, max_error, run_attention  # noqa: F401
 from tests.helpers import FULL, from_bf16_bits, ring_layout, to_bf16_bits
 
 pytestmark = pytest.mark.gpu
@@ -79,7 +79,7 @@ def test_random_shapes_agree_with_the_oracle_or_are_refused(gpu, tiled, dtype):
     assert ran >= 25 and refused >= 1, (ran, refused)
 
 
-def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
+def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, knobs):
     """bf16, head width 64, 32..600 rows after up to 6,000 cached positions, flat caches and rings, full
     attention and windows above 1,024: the calls whose keys the library splits between workgroups, with the
     library's own split count and with forced ones (including more splits than tiles)."""
@@ -98,9 +98,9 @@ def test_random_prompt_passes_with_few_rows_over_long_caches(gpu, monkeypatch):
             slots = ((window if window != FULL else end) + t + int(rng.integers(0, 200)) + 31) // 32 * 32
         forced = rng.choice([None, None, "1", "2", "3", "5", "8", "9", "17", "64"])
         if forced:
-            monkeypatch.setenv("LNG_PREFILL_SPLITS", str(forced))
+            knobs.setenv("LNG_PREFILL_SPLITS", str(forced))
         else:
-            monkeypatch.delenv("LNG_PREFILL_SPLITS", raising=False)
+            knobs.delenv("LNG_PREFILL_SPLITS", raising=False)
         if not orc.accepts(t, start, heads, kv_heads, 64, window, slots, True):
             continue
         qb = to_bf16_bits((rng.standard_normal((t, heads, 64)) * 0.7).astype(np.float32))
