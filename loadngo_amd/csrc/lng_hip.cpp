@@ -109,6 +109,7 @@ struct lng_gpu {
     hipFunction_t decode_bf16_d64 = nullptr, decode_bf16_d64_o4 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr, decode_merge_few = nullptr;
     hipFunction_t decode_bf16_wide[3] = {}, decode_f32_wide[3] = {}; // head widths 128, 256, 512
     hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_h1w = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
+    hipFunction_t prefill_bf16_wide[3] = {}, prefill_f32_wide[3] = {}; // head widths 128, 256, 512
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
     hipFunction_t prepare_v4 = nullptr, prepare_v1 = nullptr;
     hipFunction_t q8_split_x = nullptr, q8_stream = nullptr, q8_stream_one = nullptr, q8_stream_one_w8 = nullptr, q8_stream_bf16 = nullptr, q8_tiled = nullptr,
@@ -780,6 +781,73 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         return LNG_OK;
     }
 
+    // Head widths 128, 256 and 512: the prompt-pass kernels that walk the head in slices of 64 dimensions, groups of
+    // up to 16 query heads. A workgroup of four wavefronts takes 1, 2 or 4 heads of one kv head (as many as the
+    // group has, up to four) and 4, 2 or 1 blocks of 32 query rows.
+    const int wide = s.dim == 128 ? 0 : s.dim == 256 ? 1 : s.dim == 512 ? 2 : -1;
+    if ((tiled || several_rows) && wide >= 0 && s.heads / s.kv_heads <= 16 && aligned16 && scale_positive && end <= 0x7fffffffull &&
+        !g->knobs.wide_row_by_row && !g->knobs.wide_generic && (dtype == LNG_BF16 || !g->knobs.f32_generic)) {
+        const bool f32 = dtype == LNG_F32;
+        const uint64_t group = s.heads / s.kv_heads;
+        const uint64_t hw = group >= 3 ? 4 : group, bm = 32 * (4 / hw), head_blocks = (group + hw - 1) / hw;
+        lng_k_prefill p{};
+        p.dtype = (uint32_t)dtype;
+        p.q = (const char *)oq.buf->ptr + q.offset;
+        p.k = (const char *)ok.buf->ptr + k.offset;
+        p.v = (const char *)ov.buf->ptr + v.offset;
+        p.out = (char *)oo.buf->ptr + out.offset;
+        p.sinks = sinks ? (const float *)((const char *)os.buf->ptr + sinks->offset) : nullptr;
+        p.t = s.t;
+        p.start = s.start;
+        p.window = s.window >= end ? LNG_WINDOW_FULL : s.window;
+        p.slots = s.slots;
+        p.heads = (uint32_t)s.heads;
+        p.kv_heads = (uint32_t)s.kv_heads;
+        p.dim = (uint32_t)s.dim;
+        p.q_tiles = (uint32_t)((s.t + bm - 1) / bm);
+        p.scale = s.scale;
+        // Fewer workgroups than compute units: the key tiles of a query tile are split between up to eight
+        // workgroups (each keeping two tiles or more), merged by lng_prefill_merge.
+        p.splits = 1;
+        const uint64_t visible = p.window == LNG_WINDOW_FULL ? end : std::min<uint64_t>(end, p.window + bm);
+        const uint64_t key_tiles = (visible + 63) / 64;
+        const uint64_t plain_wgs = (uint64_t)p.q_tiles * head_blocks * s.kv_heads;
+        if (plain_wgs < g->cus) {
+            uint64_t want = std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, key_tiles / 2), 8);
+            if (g->knobs.prefill_splits > 0) want = std::min<uint64_t>(g->knobs.prefill_splits, 8);
+            if (want > 1) p.splits = (uint32_t)want;
+        }
+        if ((uint64_t)plain_wgs * p.splits > 0x7fffffffull) return fail(LNG_ERR_DISPATCH, "%llu rows of %llu heads are more workgroups than one dispatch holds", (unsigned long long)s.t, (unsigned long long)s.heads);
+        if (p.splits > 1) {
+            const size_t slots = (size_t)s.t * s.heads * p.splits;
+            Scratch sc;
+            if (int rc = reserve_scratch(g, slots * s.dim, slots * 2, 0, &sc)) return rc;
+            p.partial_o = sc.o;
+            p.partial_ml = sc.ml;
+        }
+        static const char *const names_bf16[3] = {"lng_prefill_bf16_w128", "lng_prefill_bf16_w256", "lng_prefill_bf16_w512"};
+        static const char *const names_f32[3] = {"lng_prefill_f32_w128", "lng_prefill_f32_w256", "lng_prefill_f32_w512"};
+        Cmd c;
+        c.grid[0] = (unsigned)(plain_wgs * p.splits); // kv head fastest: one XCD's L2 per kv head
+        c.block = 256;
+        c.fn = f32 ? g->prefill_f32_wide[wide] : g->prefill_bf16_wide[wide];
+        c.name = f32 ? names_f32[wide] : names_bf16[wide];
+        set_args(c, p);
+        b->cmds.push_back(std::move(c));
+        if (p.splits > 1) {
+            Cmd m;
+            m.fn = g->prefill_merge;
+            m.name = "lng_prefill_merge";
+            const uint64_t pairs_per_wg = 1024 / s.dim; // a thread per (row, head, four dims)
+            m.grid[0] = (unsigned)((s.t * s.heads + pairs_per_wg - 1) / pairs_per_wg);
+            m.block = 256;
+            set_args(m, p);
+            b->cmds.push_back(std::move(m));
+        }
+        b->dispatches += 1;
+        return LNG_OK;
+    }
+
     lng_k_attn a{};
     a.q = (const char *)oq.buf->ptr;
     a.k = (const char *)ok.buf->ptr;
@@ -864,6 +932,12 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
         {"lng_prefill_f32_d64_w4", &g->prefill_f32_d64_w4, true},
         {"lng_prefill_merge", &g->prefill_merge, true},
+        {"lng_prefill_bf16_w128", &g->prefill_bf16_wide[0], true},
+        {"lng_prefill_bf16_w256", &g->prefill_bf16_wide[1], true},
+        {"lng_prefill_bf16_w512", &g->prefill_bf16_wide[2], true},
+        {"lng_prefill_f32_w128", &g->prefill_f32_wide[0], true},
+        {"lng_prefill_f32_w256", &g->prefill_f32_wide[1], true},
+        {"lng_prefill_f32_w512", &g->prefill_f32_wide[2], true},
         {"lng_copy_rows", &g->copy_rows, true},
         {"lng_fill_synthetic", &g->fill_synthetic, true},
         {"lng_add_rows", &g->add_rows, true},

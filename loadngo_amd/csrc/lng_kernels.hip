@@ -3662,17 +3662,19 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_f32_d64_
 extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefill p) {
     const uint32_t group = p.heads / p.kv_heads;
     if (p.splits <= 8u) {
-        const uint64_t pair = (uint64_t)blockIdx.x * 16u + (threadIdx.x >> 4); // row * heads + head
+        // dim / 4 threads per (row, head): 16 at head width 64, so 16 (row, head) pairs per workgroup; 2 at width 512
+        const uint32_t per_pair = p.dim >> 2, pairs_per_wg = 256u / per_pair;
+        const uint64_t pair = (uint64_t)blockIdx.x * pairs_per_wg + threadIdx.x / per_pair; // row * heads + head
         if (pair >= p.t * p.heads) return;
         const uint32_t row = (uint32_t)(pair / p.heads), head = (uint32_t)(pair % p.heads);
-        const uint32_t g = head / group, h = head % group, d4 = (threadIdx.x & 15u) * 4u;
+        const uint32_t g = head / group, h = head % group, d4 = (threadIdx.x % per_pair) * 4u;
         const uint64_t slot0 = (((uint64_t)row * p.kv_heads + g) * p.splits) * group + h;
         float4 o[8];
         float2 ml[8];
 #pragma unroll
         for (int c = 0; c < 8; ++c) {
             if ((uint32_t)c < p.splits) {
-                o[c] = *(const float4 *)(p.partial_o + (slot0 + (uint64_t)c * group) * 64u + d4);
+                o[c] = *(const float4 *)(p.partial_o + (slot0 + (uint64_t)c * group) * p.dim + d4);
                 ml[c] = *(const float2 *)(p.partial_ml + (slot0 + (uint64_t)c * group) * 2u);
             }
         }
@@ -3696,7 +3698,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
             }
         }
         if (p.dtype == LNG_F32) {
-            *(float4 *)((float *)p.out + pair * 64u + d4) = make_float4(sum.x / z, sum.y / z, sum.z / z, sum.w / z);
+            *(float4 *)((float *)p.out + pair * p.dim + d4) = make_float4(sum.x / z, sum.y / z, sum.z / z, sum.w / z);
             return;
         }
         ushort4 r;
@@ -3704,7 +3706,7 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
         r.y = f32_to_bf16_bits(sum.y / z);
         r.z = f32_to_bf16_bits(sum.z / z);
         r.w = f32_to_bf16_bits(sum.w / z);
-        *(ushort4 *)((uint16_t *)p.out + pair * 64u + d4) = r;
+        *(ushort4 *)((uint16_t *)p.out + pair * p.dim + d4) = r;
         return;
     }
     const uint32_t row = blockIdx.y / p.kv_heads;
@@ -3721,3 +3723,5 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     it.sinks_offset = p.sinks ? 0u : LNG_NO_SINKS;
     merge_chunks<false>(a, it, blockIdx.y, g, group, p.splits);
 }
+
+#include "lng_prefill_wide.h"

@@ -43,10 +43,11 @@ def knobs(gpu):
     k.restore()
 
 
-def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out=True):
+def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out=True, expect_kernel=None):
     """One dispatch as the reference's test harness lays it out (attention_grouped.rs:102-158):
     five buffers (q, k, v, out, sinks), slices over all of each. q is [t][H][D]; for the tiled
-    operator it is zero-padded to t rounded up to 32 rows. Returns out[:t] (f32 or bf16 bits)."""
+    operator it is zero-padded to t rounded up to 32 rows. Returns out[:t] (f32 or bf16 bits).
+    ``expect_kernel``: the name of a kernel the dispatch must have launched exactly once."""
     t, heads, dim = q.shape
     es = 4 if dtype == C.F32 else 2
     rows = (t + 31) // 32 * 32 if tiled else t
@@ -58,6 +59,8 @@ def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out
     if poison_out:
         bufs[3].fill(0xFF)  # NaN pattern in both f32 and bf16: unwritten outputs show
     batch = gpu.batch(bufs)
+    if expect_kernel:
+        batch.set_timing(True)
     qs, ks, vs, os_ = (C.Slice(0, 0, qp.nbytes), C.Slice(1, 0, k_ring.nbytes), C.Slice(2, 0, v_ring.nbytes),
                        C.Slice(3, 0, out_len))
     try:
@@ -69,6 +72,8 @@ def run_attention(gpu, q, k_ring, v_ring, sinks, shape, tiled, dtype, poison_out
                 (qs, ks, vs), ss, os_, shape, dtype)
         done = batch.run()
         assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        if expect_kernel:
+            assert batch.kernel_seconds(expect_kernel)[1] == 1, expect_kernel
         out = bufs[3].read(np.float32 if dtype == C.F32 else np.uint16)
     finally:
         batch.drop()

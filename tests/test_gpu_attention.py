@@ -35,7 +35,9 @@ def test_plain_matches_the_float64_definition(gpu, case, sharp):
 @pytest.mark.parametrize("case,sharp", REF_TILED_CASES)
 def test_tiled_matches_the_float64_definition(gpu, case, sharp):
     q, k, v, kr, vr, shape = reference_case(oracle, case, sharp, True, None, 1.0, C.F32)
-    got = run_attention(gpu, q, kr, vr, None, shape, True, C.F32)
+    # widths 256 and 512 (the reference's tiled kernel is generic in the width): the prompt-pass kernel of that width
+    kernel = {256: "lng_prefill_f32_w256", 512: "lng_prefill_f32_w512", 64: None}[shape.dim]
+    got = run_attention(gpu, q, kr, vr, None, shape, True, C.F32, expect_kernel=kernel)
     want = oracle.attention_f64(q, k, v, None, shape.start, window=shape.window, scale=1.0, threads=THREADS)
     assert max_error(got, want) < 1e-4, case  # attention_grouped.rs:224
 
