@@ -1047,6 +1047,61 @@ def run_wide_heads(gpu, steps, warmup):
     return out
 
 
+def run_gemma(gpu, steps, warmup):
+    """The reference's own timing harness (metal-compute/tests/attention_grouped.rs:281-358 `gemma_shapes_timing`):
+    five attention shapes of its other model (32 heads over 16 kv heads of width 256 with a 1024-token window in a ring
+    of 1536; 32 over 4 of width 512, full), the tiled operator from 32 positions on and the row-by-row one below, f32
+    as the reference times them, scale 1, no sinks; bf16 beside. Median GPU time of one dispatch. `m4_pro_gpu_ms` is the
+    figure docs/NPU_ACCELERATION.md:202-208 publishes for the Metal kernel on an M4 Pro (context, not a baseline on this
+    hardware). FLOPs = 4 * dim * heads * (unmasked query-key pairs)."""
+    full = C.FULL
+    cases = [("sliding_512_pass_wrapped", (512, 2600, 32, 16, 256, 1024, 1536), 21.9),
+             ("sliding_first_512", (512, 0, 32, 16, 256, 1024, 1536), 6.1),
+             ("sliding_one_token_at_3000", (1, 3000, 32, 16, 256, 1024, 1536), 0.6),
+             ("full_77_after_700", (77, 700, 32, 4, 512, full, 32768), 8.1),
+             ("full_one_token_at_1500", (1, 1500, 32, 4, 512, full, 32768), 1.7)]
+    out = {"workload": "attention_grouped.rs:286-306, five shapes, scale 1, no sinks; synthetic fill (centred sum of four uniforms, std 0.5)"}
+    for name, (t, start, heads, kv_heads, dim, window, slots), m4 in cases:
+        tiled = t >= 32
+        end = start + t
+        rows = (t + 31) // 32 * 32 if tiled else t
+        kv_rows = min(slots, end) if not tiled else (slots if slots < end else (end + 31) // 32 * 32)
+        pairs = sum(min(start + i + 1, window) for i in range(t))
+        flops = 4 * dim * heads * pairs
+        res = {"shape": [t, start, heads, kv_heads, dim, "full" if window == full else window, slots], "operator": "tiled" if tiled else "plain",
+               "pairs": pairs, "flops": flops, "m4_pro_gpu_ms": m4}
+        for label, dtype, es in (("f32", C.F32, 4), ("bf16", C.BF16, 2)):
+            q, o = gpu.buffer(rows * heads * dim * es), gpu.buffer(rows * heads * dim * es)
+            k, v = gpu.buffer(kv_rows * kv_heads * dim * es), gpu.buffer(kv_rows * kv_heads * dim * es)
+            for i, b in enumerate((q, k, v)):
+                batch = gpu.batch([b])
+                batch.fill_synthetic(C.Slice(0, 0, b.len), dtype, 70 + i, 0.5, 0)
+                batch.run()
+                batch.drop()
+            shape = C.GroupedShape(t, start, heads, kv_heads, dim, window, slots, 1.0)
+            sl = (C.Slice(0, 0, q.len), C.Slice(1, 0, k.len), C.Slice(2, 0, v.len), C.Slice(3, 0, o.len))
+
+            def go():
+                batch = gpu.batch([q, k, v, o])
+                (batch.attention_grouped_tiled if tiled else batch.attention_grouped)(*sl, shape, dtype)
+                done = batch.run()
+                batch.drop()
+                return done.gpu_time
+
+            for _ in range(max(warmup, 3)):
+                go()
+            n = max(steps, 15)
+            g = sorted(go() for _ in range(n))[n // 2]
+            nbytes = (2 * rows * heads * dim + 2 * min(kv_rows, min(end, window + t)) * kv_heads * dim) * es
+            peak = MFMA_F32_PEAK_TFLOPS if dtype == C.F32 else MFMA_BF16_PEAK_TFLOPS
+            res[label] = {"gpu_ms": g * 1e3, "tflops": flops / g / 1e12, "mfma_frac": flops / g / 1e12 / peak,
+                          "bytes": nbytes, "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS}
+            for b in (q, o, k, v):
+                b.free()
+        out[name] = res
+    return out
+
+
 def oracle_threads():
     """Threads the oracle is timed on: the cores this process may use (its affinity mask, and OMP_NUM_THREADS when
     the environment sets it: the GPU boxes grant a one-GPU job 16 of the host's cores), never more than the host has."""
@@ -1100,7 +1155,7 @@ def main():
     ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
                     "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block,wide: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block,wide,gemma: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--record-traffic", metavar="DIR", default="", help="no GPU work: turn the rocprofv3 counter runs under DIR "
@@ -1117,7 +1172,7 @@ def main():
     extra = {}
     if args.only:
         runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare, "block": run_block,
-                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads}
+                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads, "gemma": run_gemma}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -1138,6 +1193,8 @@ def main():
         extra["c1_fp32"] = run_config1(gpu, args.steps, args.warmup)
         extra["head_width_256"] = run_wide_heads(gpu, args.steps, args.warmup)
         log("wide", extra["head_width_256"])
+        extra["reference_timing_shapes"] = run_gemma(gpu, args.steps, args.warmup)
+        log("gemma", extra["reference_timing_shapes"])
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)
     log("c5", r)
     gpu.close()
