@@ -113,8 +113,13 @@ int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
  *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
  *   LNG_PREFILL_FUSED 0      split prompt passes always merged by a second dispatch
  *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups
+ *   LNG_COUNT_SECOND_PASSES  long causal prompt passes count the query tiles whose fixed-maximum pass failed its range
+ *                            check and was made again with the maximum tracked (read with lng_hip_debug_get)
  * Read at lng_hip_open only: LNG_HSACO (a code object file to load instead of the embedded one). */
 int lng_hip_debug_set(lng_gpu *gpu, const char *name, const char *value);
+/* Development counters, no more part of the interface than the switches: waits for everything submitted so far,
+ * hands out the counter called `name` (LNG_COUNT_SECOND_PASSES) and puts it back to zero. */
+int lng_hip_debug_get(lng_gpu *gpu, const char *name, uint64_t *value);
 
 /* ---- memory --------------------------------------------------------------------------- */
 

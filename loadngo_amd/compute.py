@@ -98,6 +98,7 @@ SYMBOLS = {
     "lng_hip_close": (None, [_P]),
     "lng_hip_device_name": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.c_size_t]),
     "lng_hip_debug_set": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.c_char_p]),
+    "lng_hip_debug_get": (ctypes.c_int, [_P, ctypes.c_char_p, ctypes.POINTER(ctypes.c_uint64)]),
     "lng_hip_buffer": (ctypes.c_int, [_P, ctypes.c_size_t, ctypes.POINTER(_P)]),
     "lng_hip_resident": (ctypes.c_int, [_P, _P, ctypes.c_size_t, ctypes.POINTER(_P)]),
     "lng_hip_buffer_free": (ctypes.c_int, [_P]),
@@ -351,6 +352,12 @@ class Gpu:
         """A development switch by its environment name (``include/lng_hip.h`` lists them; not part of the
         interface); ``value`` None puts the default back. The environment itself is read once, at open."""
         _check(library().lng_hip_debug_set(self._h, name.encode(), None if value is None else str(value).encode()))
+
+    def debug_get(self, name):
+        """A development counter by name (waits for submitted work; the counter goes back to zero)."""
+        value = ctypes.c_uint64()
+        _check(library().lng_hip_debug_get(self._h, name.encode(), ctypes.byref(value)))
+        return value.value
 
     def buffer(self, len):
         h = _P()

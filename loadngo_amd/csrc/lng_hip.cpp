@@ -71,6 +71,7 @@ struct Knobs {
     int prefill_upfront = -1;      // LNG_PREFILL_UPFRONT: 0 narrow windows on the tile-by-tile kernel
     int prefill_splits = 0;        // LNG_PREFILL_SPLITS: workgroups per (query tile, kv head) of a split prompt pass; 0 planner
     int prefill_fused = -1;        // LNG_PREFILL_FUSED: 0 split prompt passes always merged by lng_prefill_merge, -1 planner
+    bool count_second_passes = false; // LNG_COUNT_SECOND_PASSES: long causal passes count the query tiles they repeat
     long decode_wgs = 0;           // LNG_DECODE_WGS: workgroups a decode dispatch aims for; 0 default
     long fuse_wgs = -1;            // LNG_FUSE_WGS: largest grid that merges inside the decode kernel; -1 default
 };
@@ -132,6 +133,7 @@ struct lng_gpu {
     uint64_t fuse_wgs = 1024;   // decode dispatches of up to this many workgroups merge their chunks in the kernel
     Knobs knobs;                // development switches, see lng_hip_debug_set
     char *static_scratch = nullptr; // this device's copy of the fixed scratch array (LNG_STATIC_SCRATCH_BYTES)
+    uint32_t *second_passes = nullptr; // device counter of repeated query tiles (LNG_COUNT_SECOND_PASSES), else NULL
 
     // completion thread (only for batches committed with a callback)
     std::thread worker;
@@ -260,7 +262,7 @@ int check_shape(const lng_grouped_shape &s, bool tiled) {
 // One development switch by its environment name; value NULL puts the default back. Returns false for an unknown name.
 const char *const knob_names[] = {"LNG_WIDE_GENERIC", "LNG_F32_GENERIC", "LNG_PLAIN_ROW_BY_ROW", "LNG_DECODE_O3", "LNG_MERGE_WIDE",
                                   "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_UPFRONT",
-                                  "LNG_PREFILL_SPLITS", "LNG_PREFILL_FUSED", "LNG_DECODE_WGS", "LNG_FUSE_WGS"};
+                                  "LNG_PREFILL_SPLITS", "LNG_PREFILL_FUSED", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES"};
 bool set_knob(lng_gpu *g, const char *name, const char *value) {
     Knobs &k = g->knobs;
     const Knobs defaults;
@@ -274,6 +276,7 @@ bool set_knob(lng_gpu *g, const char *name, const char *value) {
     if (!strcmp(name, "LNG_MERGE_WIDE")) return flag(k.merge_wide);
     if (!strcmp(name, "LNG_Q8_W16")) return flag(k.q8_w16);
     if (!strcmp(name, "LNG_WIDE_ROW_BY_ROW")) return flag(k.wide_row_by_row);
+    if (!strcmp(name, "LNG_COUNT_SECOND_PASSES")) return flag(k.count_second_passes);
     if (!strcmp(name, "LNG_PREFILL_STREAM")) return choice(k.prefill_stream, defaults.prefill_stream);
     if (!strcmp(name, "LNG_PREFILL_UPFRONT")) return choice(k.prefill_upfront, defaults.prefill_upfront);
     if (!strcmp(name, "LNG_PREFILL_FUSED")) return choice(k.prefill_fused, defaults.prefill_fused);
@@ -719,6 +722,7 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const unsigned rows_per_wg = narrow || f32 ? 32 : 64;
         p.q_tiles = (uint32_t)((s.t + rows_per_wg - 1) / rows_per_wg);
         p.scale = s.scale;
+        p.second_passes = g->knobs.count_second_passes ? g->second_passes : nullptr;
         // Few query tiles over many keys (a chunk of a long prompt, a handful of rows late in a long
         // context) would leave most compute units idle with one workgroup per (query tile, kv head):
         // the keys of a tile are then split between several workgroups and lng_prefill_merge combines
@@ -977,6 +981,14 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         return code;
     }
     g->static_scratch = (char *)lng_static_scratch(device);
+    if (hipMalloc((void **)&g->second_passes, sizeof(uint32_t)) != hipSuccess || hipMemset(g->second_passes, 0, sizeof(uint32_t)) != hipSuccess) {
+        const int code = fail(LNG_ERR_ALLOC, "could not allocate a 4-byte counter");
+        if (g->second_passes) hipFree(g->second_passes);
+        hipStreamDestroy(g->stream);
+        hipModuleUnload(g->module);
+        delete g;
+        return code;
+    }
     g->fuse_wgs = 4ull * g->cus;
     // the development switches, read once here
     for (const char *name : knob_names) {
@@ -1005,6 +1017,7 @@ void destroy_gpu(lng_gpu *g) {
     if (g->scratch_ml) hipFree(g->scratch_ml);
     if (g->tickets) hipFree(g->tickets);
     if (g->scratch_x) hipFree(g->scratch_x);
+    if (g->second_passes) hipFree(g->second_passes);
     hipStreamDestroy(g->stream);
     hipModuleUnload(g->module);
     delete g;
@@ -1016,6 +1029,20 @@ void object_gone(lng_gpu *g) {
     if (g->live_buffers.fetch_sub(1, std::memory_order_acq_rel) == 1) destroy_gpu(g);
 }
 } // namespace
+
+extern "C" int lng_hip_debug_get(lng_gpu *g, const char *name, uint64_t *value) {
+    if (!g || !name || !value) return fail(LNG_ERR_DISPATCH, "no gpu, no name or no place for the value");
+    if (strcmp(name, "LNG_COUNT_SECOND_PASSES") != 0) return fail(LNG_ERR_DISPATCH, "no development counter called %s", name);
+    // waits for everything submitted so far, reads the counter and puts it back to zero
+    hipSetDevice(g->device);
+    uint32_t n = 0;
+    hipError_t e = hipStreamSynchronize(g->stream);
+    if (e == hipSuccess) e = hipMemcpy(&n, g->second_passes, sizeof n, hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemset(g->second_passes, 0, sizeof n);
+    if (e != hipSuccess) return fail(LNG_ERR_GPU, "could not read the counter: %s", hip_text(e));
+    *value = n;
+    return LNG_OK;
+}
 
 extern "C" void lng_hip_close(lng_gpu *g) {
     if (!g) return;

@@ -63,6 +63,8 @@ typedef struct lng_k_prefill {
     uint32_t dtype;     /* LNG_F32 / LNG_BF16: element type of q, k, v and out */
     float *partial_o;   /* splits > 1: [row][kv_head][split][group][dim] f32, unnormalised */
     float *partial_ml;  /* splits > 1: [row][kv_head][split][group][2] f32 (max in the log2 domain, sum) */
+    uint32_t *second_passes; /* NULL, or a counter: +1 for every query tile of a long causal pass whose fixed-maximum
+                                pass failed its range check and was made again with the maximum tracked */
 } lng_k_prefill;
 
 typedef struct lng_k_copy {

@@ -2624,6 +2624,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             bad = row_ok ? bad : 0;
         }
         again = __syncthreads_or(bad) != 0;
+        if (again && a.second_passes && threadIdx.x == 0) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!again) {
         for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile);                    // diagonal
@@ -3404,6 +3405,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                     bad = row_ok ? bad : 0;
                 }
                 again = __syncthreads_or(bad) != 0;
+                if (again && a.second_passes && threadIdx.x == 0) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             if (!again) {
                 for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile); // the diagonal, where not done yet

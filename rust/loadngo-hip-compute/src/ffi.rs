@@ -132,6 +132,8 @@ extern "C" {
     pub fn lng_hip_device_name(gpu: *mut LngGpu, name: *mut c_char, cap: usize) -> c_int;
     /// Development switches (not part of the interface); `value` null puts the default back.
     pub fn lng_hip_debug_set(gpu: *mut LngGpu, name: *const c_char, value: *const c_char) -> c_int;
+    /// Development counters (not part of the interface): read and reset.
+    pub fn lng_hip_debug_get(gpu: *mut LngGpu, name: *const c_char, value: *mut u64) -> c_int;
 
     // ---- memory ----
     pub fn lng_hip_buffer(gpu: *mut LngGpu, len: usize, buffer: *mut *mut LngBuffer) -> c_int;

@@ -141,6 +141,15 @@ impl Gpu {
         check(unsafe { ffi::lng_hip_debug_set(self.raw.as_ptr(), name.as_ptr(), value_ptr) })
     }
 
+    /// A development counter by name (not part of the interface): waits for submitted work, reads it and resets it.
+    pub fn debug_get(&self, name: &str) -> Result<u64, Error> {
+        let name = CString::new(name).map_err(|_| Error::Dispatch("a counter name holds a NUL".into()))?;
+        let mut value = 0u64;
+        // SAFETY: the name is NUL-terminated and `value` is a valid place for the result.
+        check(unsafe { ffi::lng_hip_debug_get(self.raw.as_ptr(), name.as_ptr(), &mut value) })?;
+        Ok(value)
+    }
+
     /// Device memory of `len` bytes, contents unspecified (`apple.rs:255`). `len == 0` is `Alloc(0)`.
     pub fn buffer(&self, len: usize) -> Result<Buffer, Error> {
         let mut raw = ptr::null_mut();

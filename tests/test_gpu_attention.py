@@ -389,6 +389,42 @@ def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sin
     assert np.abs(late - from_bf16_bits(vb)[spike_at][None, :, None, :].repeat(heads // kv_heads, 2).reshape(1, heads, 64)).max() < BF16_TOL
 
 
+@pytest.mark.parametrize("stream", ["0", "1"])
+@pytest.mark.parametrize("case", ["all_far_below", "all_far_above", "huge_sink", "std4", "far_above_then_usual"])
+def test_long_causal_passes_with_every_score_far_outside_the_usual_range(gpu, case, stream, knobs):
+    """The long causal kernels (both: workgroups that walk several query tiles, and one tile per workgroup) fold
+    scale * log2(e) into the queries with one more bf16 rounding and first run with the maximum fixed; with every
+    score of a row below -600 or above 600, with sinks of +-300, with Gaussian scores of standard deviation 4
+    (sixteen times the benign fills'), and with scores that sit near +600 for the first tiles and near zero after
+    them, the range check must send the rows that need it through the tracked pass and the result must stay
+    within the bf16 bar of the CPU reference, with and without sinks."""
+    knobs.setenv("LNG_PREFILL_STREAM", stream)
+    t, heads, kv_heads = 1024, 16, 2
+    q, k, v, sinks = normal_inputs(17 + len(case), t, t, heads, kv_heads, 64, scale=0.5)
+    if case == "all_far_below":   # q . k about -64 * 1.4 * 9 * 8 * 0.125 = -800
+        q[:] = np.abs(q) + 1.0
+        k[:] = -np.abs(k) * 8.0 - 5.0
+    elif case == "all_far_above":
+        q[:] = np.abs(q) + 1.0
+        k[:] = np.abs(k) * 8.0 + 5.0
+    elif case == "huge_sink":
+        sinks[:] = 300.0
+        sinks[::3] = -300.0
+    elif case == "std4":          # q . k * 0.125 has standard deviation 4: q, k of standard deviation 2
+        q *= 4.0
+        k *= 4.0
+    elif case == "far_above_then_usual":
+        q[:] = np.abs(q) + 1.0
+        k[:192] = np.abs(k[:192]) * 8.0 + 5.0
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    shape = C.GroupedShape(t, 0, heads, kv_heads, 64, FULL, t, 0.125)
+    for sk in (sinks, None):
+        want = oracle.attention_bf16(qb, kb, vb, sk, 0, scale=0.125, threads=THREADS)
+        got = run_attention(gpu, qb, kb, vb, sk, shape, True, C.BF16,
+                            expect_kernel="lng_prefill_bf16_d64_stream" if stream == "1" else "lng_prefill_bf16_d64")
+        assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
+
+
 @pytest.mark.parametrize("case", ["spike", "all_far_below", "all_far_above", "huge_sink", "usual"])
 @pytest.mark.parametrize("window,start", [(128, 0), (100, 777), (33, 64)])
 def test_windowed_prefill_with_scores_far_outside_the_usual_range(gpu, case, window, start):
