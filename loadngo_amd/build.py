@@ -3,6 +3,7 @@
 csrc/lng_static.hip (the fixed device scratch array and the host code that finds it).
 
     python -m loadngo_amd.build
+    python -m loadngo_amd.build --null-device   # the host library alone, against csrc/null_device, with sanitizers
 """
 import os
 import subprocess
@@ -54,5 +55,26 @@ def build(verbose=False):
     return LIB
 
 
+NULL_LIB = os.path.join(HERE, "liblng_hip_null.so")
+
+
+def build_null_device(verbose=False):
+    """The host library (csrc/lng_hip.cpp) against the null device of csrc/null_device - host memory for device
+    memory, launches recorded instead of run - under AddressSanitizer and UndefinedBehaviorSanitizer. For the CPU
+    tests of the host logic (tests/test_null_device.py); no GPU code, no ROCm needed."""
+    null = os.path.join(CSRC, "null_device")
+    out = _run([
+        "g++", "-std=c++17", "-O1", "-g", "-fPIC", "-shared", "-Wall", "-Wextra", "-pthread", "-fno-omit-frame-pointer",
+        "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-DLNG_NULL_DEVICE", "-I" + null,
+        os.path.join(CSRC, "lng_hip.cpp"), os.path.join(null, "null_hip.cpp"), "-o", NULL_LIB,
+    ])
+    if verbose and out:
+        print(out)
+    return NULL_LIB
+
+
 if __name__ == "__main__":
-    print(build(verbose=True))
+    if "--null-device" in sys.argv[1:]:
+        print(build_null_device(verbose=True))
+    else:
+        print(build(verbose=True))

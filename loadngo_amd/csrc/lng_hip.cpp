@@ -23,6 +23,10 @@
 #include "lng_kernel_args.h"
 #include "lng_static.h"
 
+#ifdef LNG_NULL_DEVICE
+// The host-only build (csrc/null_device): launches are recorded, not run, and there is no code object to embed.
+extern "C" const char lng_hsaco_begin[1] = {0};
+#else
 // The code object, placed in .rodata by the assembler (path given by the build).
 #ifndef LNG_HSACO_PATH
 #error "LNG_HSACO_PATH must name the gfx950 code object to embed"
@@ -38,6 +42,7 @@ __asm__(".section .rodata\n"
         ".previous\n");
 extern "C" const char lng_hsaco_begin[];
 extern "C" const char lng_hsaco_end[];
+#endif
 
 namespace {
 
