@@ -209,7 +209,9 @@ int lng_hip_attention_grouped_tiled(lng_batch *batch, lng_slice q, lng_slice k, 
  * allocation and keeps nothing on the host heap. q, out: [t][heads][dim]; k, v: [min(slots, start + t)]
  * [kv_heads][dim]; sinks: [heads] f32 or NULL; every row is computed as the plain operator computes it
  * (same shape rules and refusals; operands aligned to their element size; the output may not overlap an
- * input). The caller vouches for the sizes behind the addresses.
+ * input). The caller vouches for the sizes behind the addresses, and for `stream` being a stream of the device
+ * `gpu` was opened on; the calling thread's current device is the same after the call as before it. Up to 32
+ * rows per call run row by row on the decode kernels (the cache is read once per row).
  *
  * Split-K partials go to a fixed array of LNG_STATIC_SCRATCH_SLOTS x 264 bytes (16.5 MiB) that every GPU the
  * library is opened on holds until the process ends. The limit: t x heads x ceil(dim / 64) <=

@@ -1392,15 +1392,20 @@ extern "C" int lng_hip_attention_grouped_static(lng_gpu *g, void *stream, const 
     }
     RowsLaunches launches;
     if (int rc = rows_launches(g, a, p, &a.first, s.t, nullptr, nullptr, &launches)) return rc;
-    if (hipSetDevice(g->device) != hipSuccess) return fail(LNG_ERR_NO_DEVICE, "cannot select HIP device %d", g->device);
-    for (int i = 0; i < launches.n; ++i) {
+    // The calling thread's current device is the caller's business (it made `stream` on one): it is put back.
+    int before = g->device;
+    if (hipGetDevice(&before) != hipSuccess) before = g->device;
+    if (before != g->device && hipSetDevice(g->device) != hipSuccess) return fail(LNG_ERR_NO_DEVICE, "cannot select HIP device %d", g->device);
+    int rc = LNG_OK;
+    for (int i = 0; i < launches.n && rc == LNG_OK; ++i) {
         size_t size = sizeof(lng_k_attn);
         void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &launches.l[i].args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                           HIP_LAUNCH_PARAM_END};
         const hipError_t e = hipModuleLaunchKernel(launches.l[i].fn, launches.l[i].grid, 1, 1, 256, 1, 1, 0, (hipStream_t)stream, nullptr, config);
-        if (e != hipSuccess) return fail(LNG_ERR_GPU, "%s did not launch: %s", launches.l[i].name, hip_text(e));
+        if (e != hipSuccess) rc = fail(LNG_ERR_GPU, "%s did not launch: %s", launches.l[i].name, hip_text(e));
     }
-    return LNG_OK;
+    if (before != g->device) hipSetDevice(before);
+    return rc;
 }
 
 extern "C" int lng_hip_copy_rows(lng_batch *b, lng_slice src, uint64_t src_stride, int src_dtype, lng_slice dst,

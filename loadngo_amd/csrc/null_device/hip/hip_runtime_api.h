@@ -51,6 +51,7 @@ hipError_t hipGetLastError(void);
 hipError_t hipInit(unsigned flags);
 hipError_t hipGetDeviceCount(int *count);
 hipError_t hipSetDevice(int device);
+hipError_t hipGetDevice(int *device);
 hipError_t hipGetDeviceProperties(hipDeviceProp_t *prop, int device);
 hipError_t hipDeviceSynchronize(void);
 

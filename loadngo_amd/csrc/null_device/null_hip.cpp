@@ -74,6 +74,10 @@ hipError_t hipGetDeviceCount(int *count) {
     return hipSuccess;
 }
 hipError_t hipSetDevice(int device) { return device == 0 ? hipSuccess : hipErrorInvalidDevice; }
+hipError_t hipGetDevice(int *device) {
+    *device = 0;
+    return hipSuccess;
+}
 hipError_t hipGetDeviceProperties(hipDeviceProp_t *prop, int) {
     memset(prop, 0, sizeof *prop);
     strcpy(prop->gcnArchName, "null-device");

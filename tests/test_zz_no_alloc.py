@@ -3,6 +3,8 @@ the existing entry point it is a variant of (lng_hip_attention_grouped) and agai
 
 Bars: bf16 in/out within 2e-2 max-abs; f32 within 1e-5 relative. Two calls in a row share the fixed
 scratch array, the second with a smaller input: what the first one left there must not show."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -22,15 +24,25 @@ def rel_error(got, want):
     return np.inf if np.isnan(e).any() else float(e.max())
 
 
-def static_call(gpu, q, k, v, sinks, shape, dtype):
-    """Uploads, calls the static entry point on the default stream, downloads (the blocking copy is
-    ordered after the kernels on that stream). Returns out [t][H][D]."""
+def _hip():
+    """The HIP runtime itself, for a stream of the caller's own (the library never makes one for this entry point)."""
+    return ctypes.CDLL("libamdhip64.so")
+
+
+def static_call(gpu, q, k, v, sinks, shape, dtype, stream=None, q_shift=0):
+    """Uploads, calls the static entry point on the default stream (or on `stream`, a hipStream_t), downloads (the
+    blocking copy is ordered after the kernels on the default stream; the caller synchronises its own). `q_shift`
+    puts the queries that many bytes into their buffer. Returns out [t][H][D]."""
     es = 4 if dtype == C.F32 else 2
-    bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.buffer(q.size * es), gpu.upload(sinks)]
+    qb = gpu.buffer(q.nbytes + q_shift)
+    qb.write(q, offset=q_shift)
+    bufs = [qb, gpu.upload(k), gpu.upload(v), gpu.buffer(q.size * es), gpu.upload(sinks)]
     bufs[3].fill(0xFF)
     try:
-        gpu.attention_grouped_static(bufs[0].device_ptr(), bufs[1].device_ptr(), bufs[2].device_ptr(),
-                                     bufs[3].device_ptr(), bufs[4].device_ptr(), shape, dtype)
+        gpu.attention_grouped_static(bufs[0].device_ptr() + q_shift, bufs[1].device_ptr(), bufs[2].device_ptr(),
+                                     bufs[3].device_ptr(), bufs[4].device_ptr(), shape, dtype, stream=stream)
+        if stream is not None:
+            assert _hip().hipStreamSynchronize(ctypes.c_void_p(stream)) == 0
         out = bufs[3].read(np.float32 if dtype == C.F32 else np.uint16)
     finally:
         for b in bufs:
@@ -82,6 +94,33 @@ def test_static_entry_point_takes_other_head_widths(gpu, dtype):
             got = static_call(gpu, q, k, v, sinks, shape, dtype)
             want = oracle.attention_f32(q, k, v, sinks, ctx - t, window=FULL, scale=0.1, threads=THREADS)
             assert rel_error(got, want.astype(np.float64)) < F32_RTOL, (t, ctx, dim)
+
+
+@pytest.mark.parametrize("dtype", [C.BF16, C.F32])
+def test_static_entry_point_on_every_kernel_family_and_on_a_stream_of_the_callers(gpu, dtype):
+    """Widths 128 and 512 in many chunks, a group of 32 query heads (the kernel of one workgroup per (row, head)), queries
+    off a 16-byte boundary (the same kernel), then two calls in a row on a stream the caller made, the second with the
+    smaller input; each against the CPU oracle."""
+    stream = ctypes.c_void_p()
+    assert _hip().hipStreamCreate(ctypes.byref(stream)) == 0
+    try:
+        cases = [(1, 9000, 8, 2, 128, None, 0), (2, 5000, 16, 4, 512, None, 0), (1, 600, 32, 1, 64, None, 0),
+                 (1, 3000, 64, 8, 64, None, 4), (1, 12000, 64, 8, 64, stream.value, 0), (1, 500, 64, 8, 64, stream.value, 0)]
+        for n, (t, ctx, heads, kv_heads, dim, on, shift) in enumerate(cases):
+            scale = float(1.0 / np.sqrt(np.float32(dim)))
+            q, k, v, sinks = normal_inputs(40 + n, t, ctx, heads, kv_heads, dim, scale=0.5)
+            shape = C.GroupedShape(t, ctx - t, heads, kv_heads, dim, FULL, ctx, scale)
+            if dtype == C.BF16:
+                qd, kd, vd = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+                got = static_call(gpu, qd, kd, vd, sinks, shape, dtype, stream=on, q_shift=shift)
+                want = oracle.attention_bf16(qd, kd, vd, sinks, ctx - t, window=FULL, scale=scale, threads=THREADS)
+                assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL, (t, ctx, heads, dim)
+            else:
+                got = static_call(gpu, q, k, v, sinks, shape, dtype, stream=on, q_shift=shift)
+                want = oracle.attention_f32(q, k, v, sinks, ctx - t, window=FULL, scale=scale, threads=THREADS)
+                assert rel_error(got, want.astype(np.float64)) < F32_RTOL, (t, ctx, heads, dim)
+    finally:
+        assert _hip().hipStreamDestroy(stream) == 0
 
 
 def test_static_entry_point_refuses_what_does_not_fit_or_is_malformed(gpu):
