@@ -612,7 +612,7 @@ int rows_launches(lng_gpu *g, lng_k_attn a, const RowsPlan &p, const lng_k_row *
                             p.kind == RowsPlan::Bf16 ? (o4 ? "lng_decode_bf16_d64_o4" : "lng_decode_bf16_d64") : "lng_decode_f32_d64", (unsigned)wgs, a};
     }
     if (a.n_chunks > 1 && !a.fused) {
-        if (a.n_chunks <= 8 && !g->knobs.merge_wide) { // a wavefront per (row, kv head, query head), four to a workgroup
+        if (a.n_chunks <= 32 && !g->knobs.merge_wide) { // a wavefront per (row, kv head, query head), four to a workgroup (LNG_MERGE_FEW)
             out->l[out->n++] = {g->decode_merge_few, "lng_decode_merge_few", (unsigned)(p.pairs * ((group + 3) / 4)), a};
         } else {                                            // a workgroup per (row, kv head, query head)
             out->l[out->n++] = {g->decode_merge, "lng_decode_merge", (unsigned)(p.pairs * group), a};

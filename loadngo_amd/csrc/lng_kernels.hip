@@ -1356,11 +1356,12 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_merge(lng_k_attn a)
     }
 }
 
-// The same merge when no row has more than eight chunks (many rows in the dispatch: a table of sequences): a
-// wavefront per (row, kv head, query head), four to a workgroup, no LDS and no barrier - eight lanes hold the
-// chunks' (max, sum), a lane per dimension adds the up to eight partial outputs with all its loads in flight.
-// A quarter of the workgroups of lng_decode_merge, which at thousands of rows costs more to launch than to run
-// (128 sequences: 5.5 us against 17 us; the same for up to sixteen chunks: 7.3 us).
+// The same merge when no row has more than LNG_MERGE_FEW chunks (many rows in the dispatch: a table of sequences): a
+// wavefront per (row, kv head, query head), four to a workgroup, no LDS and no barrier - the lanes hold the
+// chunks' (max, sum), a lane per dimension adds the partial outputs, asked for eight at a time before the weights
+// are known. A quarter of the workgroups of lng_decode_merge, which at thousands of rows costs more to launch than
+// to run (128 sequences, up to eight chunks: 5.5 us against 17 us).
+#define LNG_MERGE_FEW 32u
 extern "C" __global__ __launch_bounds__(256) void lng_decode_merge_few(lng_k_attn a) {
     const uint32_t group = a.heads / a.kv_heads;
     const uint32_t per_pair = (group + 3u) / 4u; // workgroups per (row, kv head)
@@ -1373,18 +1374,18 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_merge_few(lng_k_att
     const lng_k_row it = row_of(a, row);
     const uint64_t last = it.start;
     const uint64_t base = first_visible(last, it.window) & ~(uint64_t)31;
-    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk); // <= n_chunks <= 8
+    const uint32_t row_chunks = (uint32_t)((last + 1 - base + a.chunk - 1) / a.chunk); // <= n_chunks <= LNG_MERGE_FEW
     if (row_chunks == 1) return; // the decode kernel already wrote this row
     const uint64_t step = (uint64_t)group * a.dim;
     const uint32_t head = g * group + h;
     const uint64_t slot0 = ((uint64_t)pair * a.n_chunks) * group + h;
     const float *po = a.partial_o + slot0 * a.dim + lane;
-    float x[8]; // the first 64 dimensions' partial outputs, asked for before the weights are known
+    float x[8]; // the first 64 dimensions' partial outputs of the first eight chunks, asked for before the weights are known
 #pragma unroll
     for (int u = 0; u < 8; ++u) x[u] = (uint32_t)u < row_chunks ? po[(uint64_t)u * step] : 0.0f;
     const float sink2 = it.sinks_offset != LNG_NO_SINKS ? ((const float *)(a.sinks + it.sinks_offset))[head] * LNG_LOG2E
                                                          : LNG_NEG_INF;
-    const uint32_t c = lane & 7u; // every group of eight lanes holds the same eight chunks
+    const uint32_t c = lane & (LNG_MERGE_FEW - 1u); // both halves of the wavefront hold the same chunks
     float mc = LNG_NEG_INF, lc = 0.0f;
     if (c < row_chunks) {
         const float2 ml = *(const float2 *)(a.partial_ml + (slot0 + (uint64_t)c * group) * 2u);
@@ -1393,25 +1394,24 @@ extern "C" __global__ __launch_bounds__(256) void lng_decode_merge_few(lng_k_att
     }
     float top = fmaxf(mc, sink2);
 #pragma unroll
-    for (int s = 4; s >= 1; s >>= 1) top = fmaxf(top, __shfl_xor(top, s, 64));
+    for (int s = 16; s >= 1; s >>= 1) top = fmaxf(top, __shfl_xor(top, s, 64));
     const float wt = mc == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(mc - top);
     float z = lc * wt;
 #pragma unroll
-    for (int s = 4; s >= 1; s >>= 1) z += __shfl_xor(z, s, 64);
+    for (int s = 16; s >= 1; s >>= 1) z += __shfl_xor(z, s, 64);
     z += sink2 == LNG_NEG_INF ? 0.0f : __builtin_amdgcn_exp2f(sink2 - top);
-    float w[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) w[u] = __shfl(wt, u, 64);
     for (uint32_t db = 0; db < a.dim; db += 64u) {
-        if (db) {
-#pragma unroll
-            for (int u = 0; u < 8; ++u) x[u] = (uint32_t)u < row_chunks ? po[db + (uint64_t)u * step] : 0.0f;
-        }
         float o0 = 0.0f, o1 = 0.0f;
+        for (uint32_t c0 = 0; c0 < row_chunks; c0 += 8u) { // uniform: one turn up to eight chunks
+            if (db || c0) {
 #pragma unroll
-        for (int u = 0; u < 8; u += 2) {
-            o0 += x[u] * w[u];
-            o1 += x[u + 1] * w[u + 1];
+                for (int u = 0; u < 8; ++u) x[u] = c0 + (uint32_t)u < row_chunks ? po[db + (uint64_t)(c0 + u) * step] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; u += 2) {
+                o0 += x[u] * __shfl(wt, (int)(c0 + u), 64);
+                o1 += x[u + 1] * __shfl(wt, (int)(c0 + u + 1), 64);
+            }
         }
         const float res = (o0 + o1) / z;
         const uint64_t at = (uint64_t)head * a.dim + db + lane;

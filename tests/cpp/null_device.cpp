@@ -387,7 +387,7 @@ static void check_rows_dispatch(const std::vector<lng_k_row> &rows, uint32_t hea
             const std::string m = merge;
             CHECK(m == "lng_decode_merge" || m == "lng_decode_merge_few");
             CHECK(mgrid[0] == (m == "lng_decode_merge" ? pairs * group : pairs * ((group + 3) / 4)));
-            if (m == "lng_decode_merge_few") CHECK(a.n_chunks <= 8);
+            if (m == "lng_decode_merge_few") CHECK(a.n_chunks <= 32);
         }
     } else {
         CHECK(n_launches == 1 && !a.fused);
