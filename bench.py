@@ -889,6 +889,31 @@ def run_copy(gpu, steps, warmup, nbytes=1 << 30):
             "gpu_ms": g * 1e3, "gbs": 2 * nbytes / g / 1e9}
 
 
+def run_read(gpu, steps, warmup, nbytes=4 << 30):
+    """A plain streaming read of 4 GiB (lng_checksum: nothing but whole-line loads and an XOR): what the memory system
+    of this box delivers to a kernel that only reads, the yardstick beside the decode kernels' rate."""
+    src, dst = gpu.buffer(nbytes), gpu.buffer(16)
+    fill(gpu, src, 98)
+
+    def go():
+        batch = gpu.batch([src, dst])
+        batch.set_timing(True)
+        batch.checksum(C.Slice(0, 0, nbytes), C.Slice(1, 0, 16))
+        batch.run()
+        t = batch.kernel_seconds("lng_checksum")[0]
+        batch.drop()
+        return t
+
+    for _ in range(max(warmup, 2)):
+        go()
+    runs = sorted(go() for _ in range(max(steps, 7)))
+    src.free()
+    dst.free()
+    g = runs[len(runs) // 2]
+    return {"workload": "streaming read of %d bytes (lng_checksum)" % nbytes, "read_bytes": nbytes, "gpu_ms": g * 1e3,
+            "gbs": nbytes / g / 1e9, "hbm_frac": nbytes / g / 1e9 / HBM_PEAK_GBS}
+
+
 def run_block(gpu, steps, warmup, ctx=4096, layers=24):
     """One decoding token through the attention block of gpt-oss/src/gpu.rs:703-827 at gpt-oss-20b's sizes (hidden
     2880, 64 q / 8 kv heads of 64, Q8_0 projections), `layers` times in one batch over a bf16 cache of `ctx` tokens:
@@ -1188,7 +1213,7 @@ def main():
     ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
                     "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,prep,q8,block,wide,gemma: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,read,prep,q8,block,wide,gemma: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--record-traffic", metavar="DIR", default="", help="no GPU work: turn the rocprofv3 counter runs under DIR "
@@ -1205,7 +1230,7 @@ def main():
     extra = {}
     if args.only:
         runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare, "block": run_block,
-                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads, "gemma": run_gemma}
+                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads, "gemma": run_gemma, "read": run_read}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -1226,6 +1251,8 @@ def main():
         extra["c1_fp32"] = run_config1(gpu, args.steps, args.warmup)
         extra["head_width_256"] = run_wide_heads(gpu, args.steps, args.warmup)
         log("wide", extra["head_width_256"])
+        extra["streaming_read"] = run_read(gpu, args.steps, args.warmup)
+        log("read", extra["streaming_read"])
         extra["reference_timing_shapes"] = run_gemma(gpu, args.steps, args.warmup)
         log("gemma", extra["reference_timing_shapes"])
     r = run_stack(gpu, args.steps, args.warmup, args.batch, args.ctx, kv_gap_gib=args.kv_gap_gib)

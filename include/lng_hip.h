@@ -113,6 +113,7 @@ int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
  *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
  *   LNG_PREFILL_FUSED 0      split prompt passes always merged by a second dispatch
  *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups
+ *   LNG_CHECKSUM_WGS n       workgroups per compute unit of lng_hip_checksum's streaming read (default 2)
  *   LNG_COUNT_SECOND_PASSES  long causal prompt passes count the query tiles whose fixed-maximum pass failed its range
  *                            check and was made again with the maximum tracked (read with lng_hip_debug_get)
  * Read at lng_hip_open only: LNG_HSACO (a code object file to load instead of the embedded one). */
@@ -382,6 +383,12 @@ int lng_hip_gemm_q8_0_residual(lng_batch *batch, lng_slice codes, lng_slice scal
  * same integers are documented in the library source so a host can reproduce any element. */
 int lng_hip_fill_synthetic(lng_batch *batch, lng_slice dst, int dtype, uint64_t seed, float scale,
                            uint64_t period);
+
+/* No counterpart in the reference (benchmarks and tests): the XOR of every 16-byte word of `src` (a whole number of
+ * them, on a 16-byte boundary), written to the 16 bytes of `dst`. A kernel that only reads, whole 128-byte lines per
+ * wavefront instruction: what the memory system delivers to a plain streaming read, beside the decode kernels; and a
+ * cheap way for a host to tell whether a 96 GiB cache holds what it should. */
+int lng_hip_checksum(lng_batch *batch, lng_slice src, lng_slice dst);
 
 #ifdef __cplusplus
 }

@@ -128,6 +128,7 @@ SYMBOLS = {
                                                         ctypes.c_size_t, _U64, _U64, _U64, ctypes.c_float,
                                                         ctypes.c_int]),
     "lng_hip_fill_synthetic": (ctypes.c_int, [_P, _Slice, ctypes.c_int, _U64, ctypes.c_float, _U64]),
+    "lng_hip_checksum": (ctypes.c_int, [_P, _Slice, _Slice]),
     "lng_hip_rmsnorm_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, ctypes.c_float]),
     "lng_hip_add_rows": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64]),
     "lng_hip_rotate_halves": (ctypes.c_int, [_P, _Slice, _Slice, _U64, _U64, _U64, _U64]),
@@ -537,6 +538,10 @@ class Batch:
 
     def fill_synthetic(self, dst, dtype, seed, scale=1.0, period=0):
         _check(library().lng_hip_fill_synthetic(self._h, dst._c(), dtype, seed, scale, period))
+
+    def checksum(self, src, dst):
+        """XOR of every 16-byte word of ``src`` into the 16 bytes of ``dst`` (a plain streaming read)."""
+        _check(library().lng_hip_checksum(self._h, src._c(), dst._c()))
 
     def set_timing(self, enabled=True):
         """Record an event after every kernel so ``kernel_seconds`` can report per-kernel time."""

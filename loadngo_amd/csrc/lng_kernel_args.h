@@ -87,6 +87,17 @@ typedef struct lng_k_fill {
     uint32_t dtype;
 } lng_k_fill;
 
+/* XOR of every 16-byte word of src[0 .. n16): lng_checksum leaves one 16-byte word per workgroup in `parts`,
+ * lng_checksum_fold (one workgroup) folds the n_parts of them into dst. */
+typedef struct lng_k_checksum {
+    const char *src;
+    uint32_t *parts;
+    uint32_t *dst;
+    uint64_t n16; /* 16-byte words */
+    uint32_t n_parts;
+    uint32_t pad_;
+} lng_k_checksum;
+
 /* dst[r][i] += src[r * src_stride + i], f32. */
 typedef struct lng_k_add {
     float *dst;

@@ -2176,6 +2176,67 @@ extern "C" __global__ __launch_bounds__(512) void lng_q8_tiled_bf16(lng_k_q8 a) 
 }
 
 // Synthetic data (see LNG_SYNTH_STD in lng_kernel_args.h for the exact integers).
+// A plain streaming read: the XOR of every 16-byte word of a buffer. Consecutive lanes read consecutive 16-byte
+// words (a wavefront instruction = eight whole 128-byte lines), four loads in flight per lane and turn; the yardstick
+// for what the memory system delivers to a kernel that does nothing but read.
+extern "C" __global__ __launch_bounds__(256) void lng_checksum(lng_k_checksum a) {
+    const uint64_t stride = (uint64_t)gridDim.x * 256u;
+    uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    const uint4 *src = (const uint4 *)a.src;
+    uint4 x = make_uint4(0, 0, 0, 0);
+    for (; i + 3u * stride < a.n16; i += 4u * stride) {
+        const uint4 p0 = src[i], p1 = src[i + stride], p2 = src[i + 2u * stride], p3 = src[i + 3u * stride];
+        x.x ^= p0.x ^ p1.x ^ p2.x ^ p3.x;
+        x.y ^= p0.y ^ p1.y ^ p2.y ^ p3.y;
+        x.z ^= p0.z ^ p1.z ^ p2.z ^ p3.z;
+        x.w ^= p0.w ^ p1.w ^ p2.w ^ p3.w;
+    }
+    for (; i < a.n16; i += stride) {
+        const uint4 p = src[i];
+        x.x ^= p.x, x.y ^= p.y, x.z ^= p.z, x.w ^= p.w;
+    }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        x.x ^= __shfl_xor(x.x, s, 64);
+        x.y ^= __shfl_xor(x.y, s, 64);
+        x.z ^= __shfl_xor(x.z, s, 64);
+        x.w ^= __shfl_xor(x.w, s, 64);
+    }
+    __shared__ uint4 s_x[4];
+    if ((threadIdx.x & 63u) == 0) s_x[threadIdx.x >> 6] = x;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint4 r = s_x[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) r.x ^= s_x[w].x, r.y ^= s_x[w].y, r.z ^= s_x[w].z, r.w ^= s_x[w].w;
+        ((uint4 *)a.parts)[blockIdx.x] = r;
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void lng_checksum_fold(lng_k_checksum a) {
+    uint4 x = make_uint4(0, 0, 0, 0);
+    for (uint32_t i = threadIdx.x; i < a.n_parts; i += 256u) {
+        const uint4 p = ((const uint4 *)a.parts)[i];
+        x.x ^= p.x, x.y ^= p.y, x.z ^= p.z, x.w ^= p.w;
+    }
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) {
+        x.x ^= __shfl_xor(x.x, s, 64);
+        x.y ^= __shfl_xor(x.y, s, 64);
+        x.z ^= __shfl_xor(x.z, s, 64);
+        x.w ^= __shfl_xor(x.w, s, 64);
+    }
+    __shared__ uint4 s_x[4];
+    if ((threadIdx.x & 63u) == 0) s_x[threadIdx.x >> 6] = x;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint4 r = s_x[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) r.x ^= s_x[w].x, r.y ^= s_x[w].y, r.z ^= s_x[w].z, r.w ^= s_x[w].w;
+        *(uint4 *)a.dst = r;
+    }
+}
+
 extern "C" __global__ __launch_bounds__(256) void lng_fill_synthetic(lng_k_fill a) {
     const uint64_t stride = (uint64_t)gridDim.x * 256u;
     for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < a.n; i += stride) {

@@ -214,5 +214,6 @@ extern "C" {
         h: LngSlice, rows: u64, cols: u64, n: u64, x_stride: u64, h_stride: u64,
     ) -> c_int;
 
+    pub fn lng_hip_checksum(batch: *mut LngBatch, src: LngSlice, dst: LngSlice) -> c_int;
     pub fn lng_hip_fill_synthetic(batch: *mut LngBatch, dst: LngSlice, dtype: c_int, seed: u64, scale: f32, period: u64) -> c_int;
 }

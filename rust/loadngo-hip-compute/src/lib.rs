@@ -880,6 +880,13 @@ impl<'g> Batch<'g> {
         })
     }
 
+    /// The XOR of every 16-byte word of `src`, written to the 16 bytes of `dst`: a plain streaming read (benchmarks
+    /// and tests; no counterpart in metal-compute).
+    pub fn checksum(&mut self, src: Slice, dst: Slice) -> Result<(), Error> {
+        // SAFETY: plain call; the library validates the slices.
+        check(unsafe { ffi::lng_hip_checksum(self.handle(), src.into(), dst.into()) })
+    }
+
     /// Deterministic synthetic values written on the device (benchmarks and full-size tests).
     pub fn fill_synthetic(&mut self, dst: Slice, dtype: DType, seed: u64, scale: f32, period: u64) -> Result<(), Error> {
         // SAFETY: plain call; the library validates the slice.

@@ -217,3 +217,30 @@ def test_buffers_outlive_a_closed_gpu():
     assert np.array_equal(a.read(np.float32), np.arange(16, dtype=np.float32))
     a.free()
     b.free()
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 + 16, 1 << 20, (1 << 24) + 48])
+def test_checksum_is_the_xor_of_every_16_byte_word(gpu, nbytes):
+    """lng_hip_checksum (the plain streaming read the decode kernels are measured beside) against numpy, at sizes of
+    one word, a ragged number of words and many workgroups' worth; the slice may start inside its buffer."""
+    rng = np.random.default_rng(nbytes)
+    data = rng.integers(0, 2**32, size=nbytes // 4 + 8, dtype=np.uint32)
+    src, dst = gpu.upload(data), gpu.buffer(64)
+    dst.fill(0xFF)
+    batch = gpu.batch([src, dst])
+    try:
+        batch.checksum(C.Slice(0, 32, nbytes), C.Slice(1, 16, 16))
+        with pytest.raises(C.Dispatch):
+            batch.checksum(C.Slice(0, 32, nbytes - 8), C.Slice(1, 16, 16))  # not whole 16-byte words
+        with pytest.raises(C.Dispatch):
+            batch.checksum(C.Slice(0, 0, 64), C.Slice(0, 16, 16))           # the sum over its own source
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception), done.gpu_time
+        got = dst.read(np.uint32)
+    finally:
+        batch.drop()
+        src.free()
+        dst.free()
+    want = np.bitwise_xor.reduce(data[8:8 + nbytes // 4].reshape(-1, 4), axis=0)
+    assert (got[4:8] == want).all()
+    assert (got[:4] == 0xFFFFFFFF).all() and (got[8:] == 0xFFFFFFFF).all()
