@@ -126,3 +126,44 @@ def test_a_pass_in_chunks_equals_the_pass_in_one_call(gpu):
         assert rel_error(got, want[done:done + n]) <= F32_RTOL
         done += n
     assert done == t
+
+
+@pytest.mark.parametrize("dtype", [C.F32, C.BF16])
+def test_random_prompt_passes_at_the_wider_heads(gpu, dtype, knobs):
+    """Seeded random shapes at widths 128, 256 and 512: groups of 1..16 (one, two and four heads per workgroup, idle
+    wavefronts, several workgroups per kv head), 1..300 rows after up to 3,000 cached positions, windows of every size
+    against flat caches and rings that wrap at every phase, the library's own split count and forced ones. Every shape
+    the reference's rules accept must run on the kernel of its width and meet the bar."""
+    rng = np.random.default_rng(4242 + dtype)
+    ran = 0
+    for _ in range(36):
+        dim = int(rng.choice([128, 256, 512]))
+        kv_heads = int(rng.choice([1, 2, 3, 4] if dim < 512 else [1, 2]))
+        group = int(rng.choice([1, 2, 3, 4, 5, 8, 16]))
+        heads = kv_heads * group
+        t = int(rng.choice([32, 33, 63, 64, 65, 100, 129, 300]))
+        start = int(rng.choice([0, 1, 31, 64, 500, 1000, 3000]))
+        window = [FULL, FULL, 1, 33, 64, 100, 1025][int(rng.integers(7))]
+        end = start + t
+        if rng.integers(0, 2):
+            slots = end + int(rng.integers(0, 70))
+        else:
+            slots = ((window if window != FULL else end) + t + int(rng.integers(0, 100)) + 31) // 32 * 32
+        forced = [None, None, "2", "3", "8"][int(rng.integers(5))]
+        if forced:
+            knobs.setenv("LNG_PREFILL_SPLITS", forced)
+        else:
+            knobs.delenv("LNG_PREFILL_SPLITS", raising=False)
+        if not oracle.accepts(t, start, heads, kv_heads, dim, window, slots, True):
+            continue
+        scale = float(1.0 / np.sqrt(np.float32(dim)))
+        q, kr, vr, kz, vz, sinks = inputs(t, start, window, slots, heads, kv_heads, dim, True, 9000 + ran)
+        shape = C.GroupedShape(t, start, heads, kv_heads, dim, window, slots, scale)
+        kernel = "lng_prefill_%s_w%d" % ("f32" if dtype == C.F32 else "bf16", dim)
+        try:
+            check(gpu, dtype, q, kr, vr, kz, vz, sinks if rng.integers(0, 3) else None, shape, True, kernel)
+        except AssertionError as e:
+            raise AssertionError(f"t={t} start={start} H={heads} G={kv_heads} D={dim} window={window} slots={slots} "
+                                 f"splits={forced}: {e}") from e
+        ran += 1
+    assert ran >= 25, ran
