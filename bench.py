@@ -636,6 +636,54 @@ def run_prefill(gpu, steps, warmup, t=8192):
     return res
 
 
+def run_prefill_lengths(gpu, steps, warmup):
+    """The full-causal prompt pass at three lengths, split into what a query tile costs however many key tiles it
+    walks and what a key tile costs. The resident kernel runs one workgroup per compute unit; a workgroup's time is
+    (query tiles it takes) * a + (key tiles it walks) * b, and the three lengths give a and b by least squares."""
+    cus = 256
+    rows = []
+    for t in (8192, 12288, 16384):
+        q, out = gpu.buffer(t * QO), gpu.buffer(t * QO)
+        k, v = gpu.buffer(t * ROW), gpu.buffer(t * ROW)
+        sinks = gpu.upload(np.random.default_rng(4).standard_normal(H).astype(np.float32))
+        for i, b in enumerate((q, k, v)):
+            fill(gpu, b, 30 + i)
+        bufs = [q, k, v, out, sinks]
+        sl = (C.Slice(0, 0, t * QO), C.Slice(1, 0, t * ROW), C.Slice(2, 0, t * ROW))
+        shape = C.GroupedShape(t, 0, H, G, D, C.FULL, t, SCALE)
+
+        def go(n=20):
+            batch = gpu.batch(bufs)
+            for _ in range(n):
+                batch.attention_grouped_tiled_with_sinks(sl, C.Slice(4, 0, H * 4), C.Slice(3, 0, t * QO), shape, C.BF16)
+            done = batch.run()
+            batch.drop()
+            return done.gpu_time / n
+
+        last = go()
+        for _ in range(12):
+            cur = go()
+            if cur > 0.99 * last:
+                break
+            last = cur
+        sec = sorted(go() for _ in range(5))[2]
+        n = t // 64
+        rows.append({"positions": t, "back_to_back_ms": sec * 1e3, "query_tiles_per_workgroup": n * G / cus,
+                     "key_tiles_per_workgroup": G * n * (n + 1) / 2 / cus,
+                     "mfma_frac": 4 * D * H * (t * (t + 1) // 2) / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+        for b in bufs:
+            b.free()
+    a_mat = np.array([[r["query_tiles_per_workgroup"], r["key_tiles_per_workgroup"]] for r in rows])
+    y = np.array([r["back_to_back_ms"] * 1e3 for r in rows])
+    (per_query_tile, per_key_tile), *_ = np.linalg.lstsq(a_mat, y, rcond=None)
+    first = rows[0]
+    return {"kernel": "lng_prefill_bf16_d64_stream", "workgroups": cus, "lengths": rows,
+            "us_per_query_tile_beyond_its_key_tiles": float(per_query_tile), "us_per_key_tile": float(per_key_tile),
+            "share_outside_the_key_tiles_at_8192": float(per_query_tile * first["query_tiles_per_workgroup"] /
+                                                         (first["back_to_back_ms"] * 1e3)),
+            "residual_us": [float(x) for x in (a_mat @ np.array([per_query_tile, per_key_tile]) - y)]}
+
+
 def run_prefill_activity(gpu, steps, warmup, t=8192):
     """The full-causal prompt pass of configuration 4 on all-zero inputs and on random inputs of two
     magnitudes, one launch at a time and 50 launches back to back in one batch. Same instructions, same
@@ -1213,7 +1261,7 @@ def main():
     ap.add_argument("--kv-gap-gib", type=int, default=None, help="allocate all K caches, this many GiB unused, then "
                     "all V caches, instead of K and V layer by layer (placement experiment)")
     ap.add_argument("--no-extras", action="store_true", help="skip configurations 2, 3 and 4")
-    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,copy,read,prep,q8,block,wide,gemma: run just these and print their results "
+    ap.add_argument("--only", default="", help="comma list of c2,c3,c4,c4act,c4fit,copy,read,prep,q8,block,wide,gemma: run just these and print their results "
                     "(a development aid; no headline line)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--record-traffic", metavar="DIR", default="", help="no GPU work: turn the rocprofv3 counter runs under DIR "
@@ -1230,7 +1278,7 @@ def main():
     extra = {}
     if args.only:
         runs = {"c2": run_single_decode, "c3": run_ragged, "c4": run_prefill, "copy": run_copy, "prep": run_prepare, "block": run_block,
-                "c4act": run_prefill_activity, "q8": run_q8, "wide": run_wide_heads, "gemma": run_gemma, "read": run_read}
+                "c4act": run_prefill_activity, "c4fit": run_prefill_lengths, "q8": run_q8, "wide": run_wide_heads, "gemma": run_gemma, "read": run_read}
         for name in args.only.split(","):
             print(json.dumps({name: runs[name](gpu, args.steps, args.warmup)}))
         gpu.close()
@@ -1241,6 +1289,7 @@ def main():
         extra["c3_ragged_batch"] = run_ragged(gpu, args.steps, args.warmup)
         log("c3", extra["c3_ragged_batch"])
         extra["c4_prefill"] = run_prefill(gpu, args.steps, args.warmup)
+        extra["c4_prefill"]["full_by_length"] = run_prefill_lengths(gpu, args.steps, args.warmup)
         log("c4", extra["c4_prefill"])
         extra["pre_attention_step"] = run_prepare(gpu, args.steps, args.warmup)
         log("prep", extra["pre_attention_step"])
