@@ -4,7 +4,8 @@ The reference's tiled kernel is generic in the head width (kernels.metal:588-720
 widths 256 and 512 (attention_grouped.rs:210-221; run in tests/test_gpu_attention.py with the kernel's name
 asserted). Here: seeded random shapes at every width, both element types, groups of 1..16, windows, rings that
 have wrapped, passes split between workgroups, and the row-by-row operator with several rows over a long cache.
-Tolerances: f32 1e-5 relative (|err| / (|want| + 1)); bf16 2e-2 max-abs."""
+Tolerances: f32 1e-5 relative (|err| / (|want| + 1)); bf16 2e-2 max-abs, or one bf16 step of the expected value where
+that is more (values of 4 and above, which windows of one or two keys over N(0,1) values do produce)."""
 import numpy as np
 import pytest
 
@@ -51,7 +52,9 @@ def check(gpu, dtype, q, kr, vr, kz, vz, sinks, shape, tiled, kernel):
         want = from_bf16_bits(oracle.attention_bf16(qb, kzb, vzb, sinks, shape.start, window=shape.window, scale=shape.scale,
                                                     threads=THREADS))
         got = run_attention(gpu, qb, krb, vrb, sinks, shape, tiled, C.BF16, expect_kernel=kernel)
-        assert max_error(from_bf16_bits(got), want) <= BF16_TOL
+        have = from_bf16_bits(got).astype(np.float64)
+        assert not np.isnan(have).any()
+        assert (np.abs(have - want) <= np.maximum(BF16_TOL, np.abs(want) * 2.0 ** -7)).all(), max_error(from_bf16_bits(got), want)
     return got
 
 
