@@ -95,7 +95,7 @@ def record_traffic(root, ctx, batch):
     total = 0.0
     detail = {}
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        for kernel in DECODE_KERNELS + ("lng_decode_merge",):
+        for kernel in DECODE_KERNELS + ("lng_decode_merge", "lng_decode_merge_few"):
             for grid, kib in per_dispatch("pmc_c5_" + counter, kernel).items():
                 nbytes = kib * 1024.0 * scale[counter]
                 detail["%s grid %d %s" % (kernel, grid, counter)] = {"kib_per_dispatch": kib, "bytes": nbytes}
