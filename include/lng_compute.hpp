@@ -317,6 +317,9 @@ class Batch {
         detail::check(lng_hip_prepare_attention(h_, &buffers, items.data(), items.size(), heads, kv_heads, dim, rotary,
                                                 (int)out_dtype));
     }
+    // No counterpart in the reference: the XOR of every 16-byte word of `src`, written to the 16 bytes of `dst` (a plain
+    // streaming read: a yardstick for the memory system and a cheap check of what a large cache holds).
+    void checksum(Slice src, Slice dst) { detail::check(lng_hip_checksum(h_, src.c(), dst.c())); }
     // apple.rs:2194
     void barrier() { detail::check(lng_hip_batch_barrier(h_)); }
 
@@ -391,6 +394,14 @@ class Gpu {
     // apple.rs:302
     std::shared_ptr<Resident> resident_words(const std::vector<uint16_t> &words) const {
         return resident(words.data(), words.size() * 2);
+    }
+    // Development switches and counters (no counterpart in the reference, not part of the interface: see lng_hip.h).
+    // `value` nullptr puts the switch's default back.
+    void debug_set(const char *name, const char *value) const { detail::check(lng_hip_debug_set(h_, name, value)); }
+    uint64_t debug_get(const char *name) const {
+        uint64_t value = 0;
+        detail::check(lng_hip_debug_get(h_, name, &value));
+        return value;
     }
     // apple.rs:365 Gpu::batch(buffers, dispatch): the batch owns `buffers` until it completes or is dropped.
     Batch batch(std::vector<Buffer> buffers, Dispatch = Dispatch::Serial) const {

@@ -2,7 +2,8 @@
 // against the sequence of reference operators it stands for:
 //   * attention_decode_batched == one attention_grouped_with_sinks (t = 1) per sequence (gpt-oss/src/gpu.rs:794-805);
 //   * prepare_attention == add_rows x 3, rotate_halves x 2 and copy_rows into the ring (gpu.rs:733-759), bit for bit in f32;
-//   * gemm_q8_0_bf16 == gemm_q8_0 on positions that are exact in bf16; gemm_q8_0_many == one gemm_q8_0 per matrix.
+//   * gemm_q8_0_bf16 == gemm_q8_0 on positions that are exact in bf16; gemm_q8_0_many == one gemm_q8_0 per matrix;
+//   * checksum == the XOR of the words on the host; debug_set / debug_get.
 //
 // Prints one line per test and exits with the number of failures.
 #include <cmath>
@@ -252,6 +253,38 @@ void decoding_products_fold_their_neighbours_in(const Gpu &gpu) {
     std::printf("done decoding_products_fold_their_neighbours_in\n");
 }
 
+void checksum_is_the_xor_of_the_words_and_switches_pick_kernels(const Gpu &gpu) {
+    const size_t n = 3 * 65536 + 4; // floats: a whole number of 16-byte words, several workgroups and a ragged end
+    const std::vector<float> data = values(41, n);
+    uint32_t want[4] = {0, 0, 0, 0};
+    for (size_t i = 0; i < n; ++i) {
+        uint32_t bits;
+        std::memcpy(&bits, &data[i], 4);
+        want[i & 3] ^= bits;
+    }
+    std::vector<Buffer> buffers;
+    buffers.push_back(upload(gpu, data));
+    buffers.push_back(gpu.buffer(32));
+    Batch batch = gpu.batch(std::move(buffers));
+    batch.checksum(f32s(0, n), Slice(1, 0, 16));
+    gpu.debug_set("LNG_CHECKSUM_WGS", "7"); // another number of workgroups, the same sum
+    batch.checksum(f32s(0, n), Slice(1, 16, 16));
+    gpu.debug_set("LNG_CHECKSUM_WGS", nullptr);
+    Completed done = std::move(batch).run();
+    done.gpu_time();
+    const std::vector<float> got = done.buffers[1].to_f32();
+    expect(std::memcmp(got.data(), want, 16) == 0 && std::memcmp(got.data() + 4, want, 16) == 0, "checksum: the XOR of every 16-byte word");
+    bool refused = false;
+    try {
+        gpu.debug_set("LNG_NO_SUCH_SWITCH", "1");
+    } catch (const lng::Error &) {
+        refused = true;
+    }
+    expect(refused, "an unknown switch is refused");
+    expect(gpu.debug_get("LNG_COUNT_SECOND_PASSES") == 0, "no long causal pass has been made again");
+    std::printf("done checksum_is_the_xor_of_the_words_and_switches_pick_kernels\n");
+}
+
 } // namespace
 
 int main() {
@@ -261,6 +294,7 @@ int main() {
         prepare_attention_is_the_reference_sequence_of_dispatches(gpu);
         q8_product_of_bf16_positions_is_the_f32_product(gpu);
         decoding_products_fold_their_neighbours_in(gpu);
+        checksum_is_the_xor_of_the_words_and_switches_pick_kernels(gpu);
     } catch (const lng::Error &e) {
         std::printf("FAILED with %s\n", e.what());
         return 100;

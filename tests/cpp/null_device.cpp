@@ -5,6 +5,8 @@
 //    wrong length, outside their buffer or off their element size (apple.rs:860-887), outputs in resident memory or
 //    over an input (apple.rs:889-906), buffers that belong to a batch in flight, and the refusals of copy_rows,
 //    prepare_attention and the Q8_0 products; a refused call records nothing.
+//  - the development switches (environment at open, lng_hip_debug_set afterwards) and lng_hip_checksum: refusals and
+//    what is recorded.
 //  - ownership: batches hand their buffers back; close with buffers alive; the last buffer freed on one thread while
 //    the handle is closed on another.
 //  - allocation failures while recording: reported, nothing recorded, nothing leaked.
@@ -194,6 +196,94 @@ static void refusals() {
     f.rebatch();
     CHECK(lng_hip_buffer_free(res) == LNG_OK);
     lng_null_clear();
+}
+
+// The development switches (read from the environment once, at open; afterwards only lng_hip_debug_set) and the
+// streaming read: refusals, and what the planner records under a switch.
+static void switches_and_checksum() {
+    const size_t MB = 1 << 20;
+    setenv("LNG_PREFILL_SPLITS", "3", 1); // read at open ...
+    Fixture f(5, MB);
+    unsetenv("LNG_PREFILL_SPLITS"); // ... and never again
+    lng_batch *b = f.batch;
+    lng_null_clear();
+    auto prefill_splits = [&]() { // a prompt pass of 64 rows over 1,024 cached positions: one query tile per kv head
+        const lng_grouped_shape s = shape(64, 960, 8, 2, 64, LNG_WINDOW_FULL, 1024, 0.125f);
+        const lng_slice q{0, 0, 64 * 8 * 64 * 2}, k{1, 0, 1024 * 2 * 64 * 2}, v{2, 0, 1024 * 2 * 64 * 2}, o{3, 0, 64 * 8 * 64 * 2};
+        CHECK(lng_hip_attention_grouped_tiled(f.batch, q, k, v, o, nullptr, &s, LNG_BF16) == LNG_OK);
+        CHECK(lng_hip_batch_commit(f.batch, nullptr, nullptr) == LNG_OK);
+        CHECK(lng_hip_batch_wait(f.batch, nullptr) == LNG_OK);
+        const char *name = nullptr;
+        const void *args = nullptr;
+        size_t args_size = 0;
+        unsigned grid[3], block[3];
+        CHECK(lng_null_launch_count() >= 1 && lng_null_launch(0, &name, grid, block, &args, &args_size) == 0);
+        lng_k_prefill p{};
+        CHECK(args_size == sizeof p);
+        memcpy(&p, args, sizeof p);
+        CHECK(grid[0] == p.q_tiles * p.kv_heads * p.splits);
+        CHECK(p.splits == 1 || lng_null_launch_count() == 2);
+        lng_null_clear();
+        f.rebatch();
+        return p.splits;
+    };
+    CHECK(prefill_splits() == 3); // the environment's value at open
+    CHECK(lng_hip_debug_set(f.gpu, "LNG_PREFILL_SPLITS", "5") == LNG_OK);
+    CHECK(prefill_splits() == 5);
+    CHECK(lng_hip_debug_set(f.gpu, "LNG_PREFILL_SPLITS", nullptr) == LNG_OK);
+    const uint32_t planned = prefill_splits(); // the planner's own: one workgroup per compute unit, four key tiles each at least
+    CHECK(planned >= 1 && planned <= 4);
+    CHECK(refused(lng_hip_debug_set(f.gpu, "LNG_NO_SUCH_SWITCH", "1"), "no development switch"));
+    CHECK(refused(lng_hip_debug_set(f.gpu, nullptr, "1"), "no name"));
+    CHECK(lng_hip_debug_set(nullptr, "LNG_PREFILL_SPLITS", "1") != LNG_OK);
+    uint64_t n = 99;
+    CHECK(lng_hip_debug_get(f.gpu, "LNG_COUNT_SECOND_PASSES", &n) == LNG_OK && n == 0);
+    CHECK(refused(lng_hip_debug_get(f.gpu, "LNG_PREFILL_SPLITS", &n), "no development counter"));
+    CHECK(lng_hip_debug_get(f.gpu, "LNG_COUNT_SECOND_PASSES", nullptr) != LNG_OK);
+
+    // the streaming read: whole 16-byte words on a 16-byte boundary, 16 bytes out, not over its input
+    b = f.batch;
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 0, 100}, lng_slice{1, 0, 16}), "16-byte words"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 0, 0}, lng_slice{1, 0, 16}), "16-byte words"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 8, 160}, lng_slice{1, 0, 16}), "not a multiple"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 0, 160}, lng_slice{1, 0, 32}), "the shape needs"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 0, 160}, lng_slice{1, 4, 16}), "not a multiple"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, 0, 160}, lng_slice{0, 32, 16}), "overlaps"));
+    CHECK(refused(lng_hip_checksum(b, lng_slice{0, MB - 16, 32}, lng_slice{1, 0, 16}), "outside"));
+    CHECK(lng_hip_batch_dispatches(b) == 0);
+    CHECK(lng_hip_checksum(b, lng_slice{0, 0, 160}, lng_slice{1, 0, 16}) == LNG_OK);       // ten words: one workgroup
+    CHECK(lng_hip_checksum(b, lng_slice{0, 0, MB}, lng_slice{1, 16, 16}) == LNG_OK);        // 65,536 words: 256 workgroups
+    CHECK(lng_hip_debug_set(f.gpu, "LNG_CHECKSUM_WGS", "1") == LNG_OK);
+    CHECK(lng_hip_checksum(b, lng_slice{2, 0, MB}, lng_slice{1, 32, 16}) == LNG_OK);
+    CHECK(lng_hip_batch_dispatches(b) == 3);
+    CHECK(lng_hip_batch_commit(b, nullptr, nullptr) == LNG_OK);
+    CHECK(lng_hip_batch_wait(b, nullptr) == LNG_OK);
+    CHECK(lng_null_launch_count() == 6);
+    for (size_t i = 0; i < 6; i += 2) {
+        const char *name = nullptr, *fold = nullptr;
+        const void *args = nullptr;
+        size_t args_size = 0;
+        unsigned grid[3], fgrid[3];
+        CHECK(lng_null_launch(i, &name, grid, nullptr, &args, &args_size) == 0 && std::string(name) == "lng_checksum");
+        CHECK(lng_null_launch(i + 1, &fold, fgrid, nullptr, nullptr, nullptr) == 0 && std::string(fold) == "lng_checksum_fold" && fgrid[0] == 1);
+        lng_k_checksum a{};
+        CHECK(args_size == sizeof a);
+        memcpy(&a, args, sizeof a);
+        CHECK(grid[0] == a.n_parts && a.n_parts >= 1 && a.n_parts <= (a.n16 + 255) / 256);
+        CHECK(a.n16 == (i == 0 ? 10u : MB / 16));
+        CHECK(lng_null_bytes_from(a.parts) >= (size_t)a.n_parts * 16); // a 16-byte word per workgroup, in the library's scratch
+        CHECK(lng_null_bytes_from(a.src) >= a.n16 * 16 && lng_null_bytes_from(a.dst) >= 16);
+        if (i == 0) CHECK(a.n_parts == 1);
+        if (i == 4) { // one workgroup per compute unit instead of two
+            lng_k_checksum two{};
+            const void *args2 = nullptr;
+            CHECK(lng_null_launch(2, nullptr, nullptr, nullptr, &args2, nullptr) == 0);
+            memcpy(&two, args2, sizeof two);
+            CHECK(two.n_parts == 256 ? a.n_parts <= 256 : a.n_parts * 2 == two.n_parts);
+        }
+    }
+    lng_null_clear();
+    f.rebatch();
 }
 
 static void on_done_count(const lng_completed *done, void *user) {
@@ -491,6 +581,7 @@ static void planner_fuzz(size_t dispatches) {
 int main(int argc, char **argv) {
     const size_t dispatches = argc > 1 ? (size_t)strtoull(argv[1], nullptr, 10) : 100000;
     refusals();
+    switches_and_checksum();
     lifetimes();
     allocation_failures();
     planner_fuzz(dispatches);

@@ -13,7 +13,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_DIR = os.path.join(ROOT, "loadngo_amd")
 PROGRAMS = {
     "additions": ("batched_decode_is_one_plain_call_per_sequence", "prepare_attention_is_the_reference_sequence_of_dispatches",
-                  "q8_product_of_bf16_positions_is_the_f32_product", "decoding_products_fold_their_neighbours_in"),
+                  "q8_product_of_bf16_positions_is_the_f32_product", "decoding_products_fold_their_neighbours_in",
+                  "checksum_is_the_xor_of_the_words_and_switches_pick_kernels"),
     "attention_grouped": ("matches_the_float64_definition", "tiled_matches_the_float64_definition",
                           "sinks_take_probability_without_value_on_gpt_oss_shapes", "rejects_shapes_it_cannot_run",
                           "ownership_residents_and_bf16"),

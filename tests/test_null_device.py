@@ -5,7 +5,8 @@ loadngo_amd/csrc/null_device (host memory for device memory, launches recorded i
 tests/cpp/null_device.cpp then drives the C ABI: the refusals of metal-compute/src/apple.rs:860-906 and
 1243-1277 (the reference's rejected shapes, slices of the wrong length, outside their buffer or off their
 element size, outputs in resident memory or over an input, buffers of a batch in flight), the refusals of
-copy_rows, prepare_attention and the Q8_0 products, ownership and lifetimes (close racing the last free on two
+copy_rows, prepare_attention and the Q8_0 products, the development switches (environment at open,
+lng_hip_debug_set afterwards) and lng_hip_checksum, ownership and lifetimes (close racing the last free on two
 threads), allocation failures while recording, and 100,000 random dispatches through the decode planner with
 every grid, work table, chunk and scratch size checked on the host. Any sanitizer report fails the run."""
 import os
