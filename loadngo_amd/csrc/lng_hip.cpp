@@ -819,13 +819,15 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         p.q_tiles = (uint32_t)((s.t + bm - 1) / bm);
         p.scale = s.scale;
         // Fewer workgroups than compute units: the key tiles of a query tile are split between up to eight
-        // workgroups (each keeping two tiles or more), merged by lng_prefill_merge.
+        // workgroups, merged by lng_prefill_merge; each keeps two tiles or more in bf16, where a tile is short
+        // against what a workgroup pays to start and to write its partial rows, and one or more in f32, where a
+        // tile is sixteen times the matrix work (77 rows of width 512 over 777 keys: 141 us in six splits, 112 in eight).
         p.splits = 1;
         const uint64_t visible = p.window == LNG_WINDOW_FULL ? end : std::min<uint64_t>(end, p.window + bm);
         const uint64_t key_tiles = (visible + 63) / 64;
         const uint64_t plain_wgs = (uint64_t)p.q_tiles * head_blocks * s.kv_heads;
         if (plain_wgs < g->cus) {
-            uint64_t want = std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, key_tiles / 2), 8);
+            uint64_t want = std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, f32 ? key_tiles : key_tiles / 2), 8);
             if (g->knobs.prefill_splits > 0) want = std::min<uint64_t>(g->knobs.prefill_splits, 8);
             if (want > 1) p.splits = (uint32_t)want;
         }
