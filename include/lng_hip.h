@@ -111,7 +111,6 @@ int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
  *   LNG_PREFILL_STREAM 0|1   never / whenever possible the prompt-pass kernel whose workgroups walk several query tiles
  *   LNG_PREFILL_UPFRONT 0    narrow windows on the tile-by-tile kernel
  *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
- *   LNG_PREFILL_FUSED 0      split prompt passes always merged by a second dispatch
  *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups
  *   LNG_CHECKSUM_WGS n       workgroups per compute unit of lng_hip_checksum's streaming read (default 2)
  *   LNG_COUNT_SECOND_PASSES  long causal prompt passes count the query tiles whose fixed-maximum pass failed its range

@@ -75,7 +75,6 @@ struct Knobs {
     int prefill_stream = -1;       // LNG_PREFILL_STREAM: 0 never the resident prompt-pass kernel, 1 whenever it can run, -1 planner
     int prefill_upfront = -1;      // LNG_PREFILL_UPFRONT: 0 narrow windows on the tile-by-tile kernel
     int prefill_splits = 0;        // LNG_PREFILL_SPLITS: workgroups per (query tile, kv head) of a split prompt pass; 0 planner
-    int prefill_fused = -1;        // LNG_PREFILL_FUSED: 0 split prompt passes always merged by lng_prefill_merge, -1 planner
     int checksum_wgs = 0;          // LNG_CHECKSUM_WGS: workgroups per compute unit of the streaming read; 0 default (2)
     bool count_second_passes = false; // LNG_COUNT_SECOND_PASSES: long causal passes count the query tiles they repeat
     long decode_wgs = 0;           // LNG_DECODE_WGS: workgroups a decode dispatch aims for; 0 default
@@ -269,7 +268,7 @@ int check_shape(const lng_grouped_shape &s, bool tiled) {
 // One development switch by its environment name; value NULL puts the default back. Returns false for an unknown name.
 const char *const knob_names[] = {"LNG_WIDE_GENERIC", "LNG_F32_GENERIC", "LNG_PLAIN_ROW_BY_ROW", "LNG_DECODE_O3", "LNG_MERGE_WIDE",
                                   "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_UPFRONT",
-                                  "LNG_PREFILL_SPLITS", "LNG_PREFILL_FUSED", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES", "LNG_CHECKSUM_WGS"};
+                                  "LNG_PREFILL_SPLITS", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES", "LNG_CHECKSUM_WGS"};
 bool set_knob(lng_gpu *g, const char *name, const char *value) {
     Knobs &k = g->knobs;
     const Knobs defaults;
@@ -286,7 +285,6 @@ bool set_knob(lng_gpu *g, const char *name, const char *value) {
     if (!strcmp(name, "LNG_COUNT_SECOND_PASSES")) return flag(k.count_second_passes);
     if (!strcmp(name, "LNG_PREFILL_STREAM")) return choice(k.prefill_stream, defaults.prefill_stream);
     if (!strcmp(name, "LNG_PREFILL_UPFRONT")) return choice(k.prefill_upfront, defaults.prefill_upfront);
-    if (!strcmp(name, "LNG_PREFILL_FUSED")) return choice(k.prefill_fused, defaults.prefill_fused);
     if (!strcmp(name, "LNG_CHECKSUM_WGS")) return choice(k.checksum_wgs, defaults.checksum_wgs);
     if (!strcmp(name, "LNG_PREFILL_SPLITS")) {
         k.prefill_splits = value ? (int)std::max(1l, std::min(n, 64l)) : 0;
@@ -748,6 +746,9 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             uint64_t want = g->cus / plain_wgs;
             want = std::min<uint64_t>(want, key_tiles / 4);
             want = std::min<uint64_t>(want, 64);
+            // (under a dozen key tiles the partial rows and the merge cost what two splits save: the first 512 rows of a
+            // prompt 24.5 us unsplit, 30.8 us in two)
+            if (key_tiles < 12) want = 1;
             if (g->knobs.prefill_splits > 0) want = std::min<uint64_t>(g->knobs.prefill_splits, 64);
             if (want > 1) p.splits = (uint32_t)want;
         }
