@@ -2993,16 +2993,38 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
     constexpr int LD = (int)SBN / (32 * QB); // keys of a tile each thread loads
     __shared__ __attribute__((aligned(16))) uint16_t s_k[3][SBN * PF_KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t s_v[3][SBN * PF_VSTRIDE];
+    __shared__ uint32_t s_again; // the range check's verdict, see below
 
-    const uint32_t g = blockIdx.x % a.kv_heads;
     const uint32_t c = blockIdx.x / a.kv_heads;   // this workgroup among the C of its kv head
     const uint32_t C = gridDim.x / a.kv_heads;
     const uint32_t group = a.heads / a.kv_heads;
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t n = lane & 31u;
-    const uint32_t hh = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // What a lane derives from its number (its query, its half, its LDS and cache offsets) is cheap to work out and
+    // expensive to keep: registers that live across the interior loop without being used in it are spilled, a spill
+    // goes out to memory, and its reload waits for every load in flight. These are therefore worked out again at the
+    // top of a query tile, after its interior loop and before its outputs, from a lane number the compiler cannot
+    // follow (so that it does not keep the first copy instead).
+    uint32_t lane, tid, n, hh, ld_key, ld_chunk, k_lane_off, v_lane_off;
+    const char *kbase, *vbase;
+    const uint32_t g = blockIdx.x % a.kv_heads;
+    auto lane_values = [&]() {
+        uint32_t z = 0u;
+        asm volatile("" : "+v"(z));
+        lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
+        tid = wave * 64u + lane;
+        n = lane & 31u;
+        hh = lane >> 5;
+        ld_key = tid >> 3; // a thread's further keys are 32 * QB apart
+        ld_chunk = tid & 7u;
+        kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
+        vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
+        k_lane_off = n * PF_KSTRIDE + 8u * hh;
+        const uint32_t L = lane & 15u;
+        const uint32_t blk16 = lane >> 4;
+        v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+    };
+    lane_values();
+    s_again = 0u; // (every thread, the same value; the first barrier below is ahead of its first use)
     const uint32_t qb = QB == 2 ? (wave & 1u) : 0u;
     const uint32_t hp = QB == 2 ? (wave >> 1) : wave;
     const uint32_t t = (uint32_t)a.t, start = (uint32_t)a.start;
@@ -3014,21 +3036,20 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
     head[0] = g * group + (wave_active ? hp * NH : 0u);
     head[1] = second_ok ? head[0] + 1u : head[0];
     const float sl2 = a.scale * LNG_LOG2E;
-    float sink2[NH]; // read once, not per query tile
+    float sink2[NH]; // read once, not per query tile (and both in one trip)
 #pragma unroll
-    for (int h = 0; h < NH; ++h) sink2[h] = a.sinks ? a.sinks[head[h]] * LNG_LOG2E : LNG_NEG_INF;
+    for (int h = 0; h < NH; ++h) sink2[h] = LNG_NEG_INF;
+    if (a.sinks) {
+        float raw[NH];
+#pragma unroll
+        for (int h = 0; h < NH; ++h) raw[h] = a.sinks[head[h]];
+#pragma unroll
+        for (int h = 0; h < NH; ++h) sink2[h] = raw[h] * LNG_LOG2E;
+    }
     bf16x2 ones2;
     ones2[0] = (__bf16)1.0f;
     ones2[1] = (__bf16)1.0f;
 
-    const uint32_t ld_key = tid >> 3; // a thread's further keys are 32 * QB apart
-    const uint32_t ld_chunk = tid & 7u;
-    const char *kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
-    const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
-    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;
-    const uint32_t L = lane & 15u;
-    const uint32_t blk16 = lane >> 4;
-    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
 
     using tracked = std::integral_constant<int, 0>;
     using fixed_at_m = std::integral_constant<int, 1>;
@@ -3044,9 +3065,15 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
         const uint32_t pos_last = pos_first + rows_here - 1;
         const uint32_t n_tiles = pos_last / SBN + 1;
         const uint32_t n_interior = (pos_first + 1u) / SBN; // tiles whose every key every query of the tile sees
-        const uint32_t my_row = q0 + 32u * qb + n;
-        const uint32_t my_pos = start + my_row;
-        const bool row_ok = my_row < t;
+        uint32_t my_row, my_pos;
+        bool row_ok;
+        auto row_values = [&]() {
+            lane_values();
+            my_row = q0 + 32u * qb + n;
+            my_pos = start + my_row;
+            row_ok = my_row < t;
+        };
+        row_values();
 
         auto fetch = [&](uint32_t tile, uint4 (&kr)[LD], uint4 (&vr)[LD]) {
 #pragma unroll
@@ -3337,6 +3364,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                 __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
                 __builtin_amdgcn_s_barrier();
             };
+            // (the first operands are read here again rather than taken from the step before: carried across the
+            // rescaling to zero they were spilled and reloaded, sixteen registers per query tile)
+            read_k(buf, 0, ka0);
             fetch(tile + 2, kr, vr);
             auto loop = [&](auto active_tag) {
                 constexpr bool ACTIVE = decltype(active_tag)::value;
@@ -3440,6 +3470,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                 }
                 if (at_zero) {
                     pipe(tile);
+                    row_values();
                     // the diagonal at the same fixed reference point (a masked score is 2^-inf = 0), before the check
                     for (; tile < n_tiles; ++tile) step(std::true_type{}, fixed_at_zero{}, tile);
                 } else {
@@ -3465,8 +3496,15 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
                     }
                     bad = row_ok ? bad : 0;
                 }
-                again = __syncthreads_or(bad) != 0;
-                if (again && a.second_passes && threadIdx.x == 0) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // (the workgroup's OR through a word of LDS: the library routine works out a thread number from the
+                // three thread indices, which live in registers from the kernel's start and had been spilled by now -
+                // two trips to memory per query tile)
+                if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) s_again = 1u;
+                __syncthreads();
+                again = s_again != 0u;
+                __syncthreads(); // everyone has read it
+                s_again = 0u;    // for the next query tile: its first barrier is ahead of the next check
+                if (again && a.second_passes && wave == 0u && lane == 0u) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             if (!again) {
                 for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile); // the diagonal, where not done yet
@@ -3474,6 +3512,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
             }
         }
 
+        row_values();
         // ---- normalise and store: lane holds dims 32db + 8blk + 4hh + i of its query ------------------
         if (wave_active && row_ok) {
 #pragma unroll
