@@ -2312,6 +2312,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     constexpr uint32_t PF_BM = NH == 2 ? 64u : 32u;
     __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
+    __shared__ uint32_t s_again; // the range check's verdict (two heads per wavefront)
 
     const bool partial = a.splits > 1u;
     const uint32_t g = blockIdx.x % a.kv_heads;
@@ -2319,11 +2320,35 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     const uint32_t split = partial ? above % a.splits : 0u;        // an unsplit pass pays for no division by splits
     const uint32_t qtile = a.q_tiles - 1u - (partial ? above / a.splits : above);
     const uint32_t group = a.heads / a.kv_heads;
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & 63u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6); // scalar: branches on it are uniform
-    const uint32_t n = lane & 31u;  // query within the wave's block
-    const uint32_t hh = lane >> 5;  // which half of the k-slots / of each 8 accumulator rows
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // scalar: branches on it are uniform
+    // What a lane derives from its number: n = query within the wave's block, hh = which half of the k-slots / of each
+    // 8 accumulator rows, the chunk of a tile it loads, its LDS offsets. With two heads per wavefront (256 registers
+    // in use in the loops) these are worked out again after the loops instead of kept: a register that lives across a
+    // loop without being used in it is spilled, a spill goes out to memory and its reload waits for every load in
+    // flight. The lane number comes from mbcnt behind an empty asm statement, which the compiler cannot trace back
+    // to the first copy.
+    uint32_t lane, tid, n, hh, ld_key, ld_chunk, k_lane_off, v_lane_off;
+    const char *kbase, *vbase;
+    auto lane_values = [&]() {
+        uint32_t z = 0u;
+        asm volatile("" : "+v"(z));
+        lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, z));
+        tid = wave * 64u + lane;
+        n = lane & 31u;
+        hh = lane >> 5;
+        ld_key = tid >> 3;  // 0..63
+        ld_chunk = tid & 7u;
+        kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
+        vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
+        // per-lane constant parts of the LDS addresses
+        k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
+        const uint32_t L = lane & 15u;
+        const uint32_t blk16 = lane >> 4;                                     // 16-lane block 0..3
+        // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
+        v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
+    };
+    lane_values();
+    if constexpr (NH == 2) s_again = 0u; // (every thread, the same value; the first barrier is ahead of its first use)
     const uint32_t qb = NH == 2 ? (wave & 1u) : 0u;
     const uint32_t hp = NH == 2 ? (wave >> 1) : wave; // first head slot of the wavefront is hp * NH
 
@@ -2350,9 +2375,14 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     // ---- this wavefront's queries and its two heads -------------------------------------------
     // A wavefront whose second head slot is past the group computes its first head twice and
     // stores it once; one whose first slot is past the group only helps loading tiles.
-    const uint32_t my_row = q0 + 32u * qb + n;      // query row of this lane
-    const uint32_t my_pos = start + my_row;         // its absolute position
-    const bool row_ok = my_row < t;
+    uint32_t my_row, my_pos;
+    bool row_ok;
+    auto row_values = [&]() {
+        my_row = q0 + 32u * qb + n;      // query row of this lane
+        my_pos = start + my_row;         // its absolute position
+        row_ok = my_row < t;
+    };
+    row_values();
     const bool wave_active = hp * NH < group;
     const bool second_ok = NH == 2 && hp * 2u + 1u < group;
     uint32_t head[NH];
@@ -2389,10 +2419,6 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     ones2[1] = (__bf16)1.0f;
 
     // ---- tile loader: one 16-byte chunk of K and of V per thread --------------------------------
-    const uint32_t ld_key = tid >> 3;  // 0..63
-    const uint32_t ld_chunk = tid & 7u;
-    const char *kbase = a.k + (uint64_t)g * 128u + ld_chunk * 16u;
-    const char *vbase = a.v + (uint64_t)g * 128u + ld_chunk * 16u;
     auto fetch = [&](uint32_t tile, uint4 &kr, uint4 &vr) {
         uint32_t p = tile0 + tile * PF_BN + ld_key;
         p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway,
@@ -2406,12 +2432,6 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         *(uint4 *)(&s_v[buf][ld_key * PF_VSTRIDE + ld_chunk * 8u]) = vr;
     };
 
-    // per-lane constant parts of the LDS addresses
-    const uint32_t k_lane_off = n * PF_KSTRIDE + 8u * hh;                 // + kb*32*KSTRIDE + 16*ks
-    const uint32_t L = lane & 15u;
-    const uint32_t blk16 = lane >> 4;                                     // 16-lane block 0..3
-    // transposing read: source lane L names key (L>>2) of its group and dims 4*(L&3).. of the block's 16
-    const uint32_t v_lane_off = (4u * (blk16 >> 1) + (L >> 2)) * PF_VSTRIDE + 16u * (blk16 & 1u) + 4u * (L & 3u);
 
     // With two heads per wavefront (long causal runs) the pass is first made optimistically: once a
     // first interior tile has set the running maximum from real scores, the remaining interior
@@ -2655,6 +2675,10 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
         for (; tile < n_tiles && !edge(tile); ++tile) step(std::false_type{}, tracked{}, tile);
     }
     }
+    if constexpr (NH == 2) {
+        lane_values();
+        row_values();
+    }
     bool again = false;
     if (NH == 2 && frozen) { // frozen is uniform over the workgroup
         if (wave_active) {
@@ -2684,8 +2708,14 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
             }
             bad = row_ok ? bad : 0;
         }
-        again = __syncthreads_or(bad) != 0;
-        if (again && a.second_passes && threadIdx.x == 0) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // (the workgroup's OR through a word of LDS: the library routine works out a thread number from the three
+        // thread indices, which live in registers from the kernel's start and are spilled by now)
+        if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) s_again = 1u;
+        __syncthreads();
+        again = s_again != 0u;
+        __syncthreads(); // everyone has read it
+        s_again = 0u;    // for the second attempt's check: its barriers lie between
+        if (again && a.second_passes && wave == 0u && lane == 0u) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!again) {
         for (; tile < n_tiles; ++tile) step(std::true_type{}, tracked{}, tile);                    // diagonal
@@ -2694,6 +2724,10 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     }
 
 
+    if constexpr (NH == 2) {
+        lane_values();
+        row_values();
+    }
     // ---- with splits: leave the partial state, lane holds dims 32db + 8blk + 4hh + i of its query. Through LDS
     // like the outputs below, 32 dimensions (128 bytes of f32) of 32 rows at a time: eight lanes store a whole line.
     if (partial) {
