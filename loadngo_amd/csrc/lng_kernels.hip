@@ -2312,7 +2312,7 @@ template <int NH> __device__ __forceinline__ void prefill_body(const lng_k_prefi
     constexpr uint32_t PF_BM = NH == 2 ? 64u : 32u;
     __shared__ __attribute__((aligned(16))) uint16_t s_k[2][PF_BN * PF_KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t s_v[2][PF_BN * PF_VSTRIDE];
-    __shared__ uint32_t s_again; // the range check's verdict (two heads per wavefront)
+    __shared__ uint32_t s_again; // the outcome of the range check (two heads per wavefront)
 
     const bool partial = a.splits > 1u;
     const uint32_t g = blockIdx.x % a.kv_heads;
@@ -3027,7 +3027,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_st
     constexpr int LD = (int)SBN / (32 * QB); // keys of a tile each thread loads
     __shared__ __attribute__((aligned(16))) uint16_t s_k[3][SBN * PF_KSTRIDE];
     __shared__ __attribute__((aligned(16))) uint16_t s_v[3][SBN * PF_VSTRIDE];
-    __shared__ uint32_t s_again; // the range check's verdict, see below
+    __shared__ uint32_t s_again; // the outcome of the range check, see below
 
     const uint32_t c = blockIdx.x / a.kv_heads;   // this workgroup among the C of its kv head
     const uint32_t C = gridDim.x / a.kv_heads;
