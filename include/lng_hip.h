@@ -113,6 +113,8 @@ int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
  *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
  *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups
  *   LNG_CHECKSUM_WGS n       workgroups per compute unit of lng_hip_checksum's streaming read (default 2)
+ *   LNG_TABLE_IN_PLACE n     row tables of n bytes or more stay in pinned host memory, where the kernels read them,
+ *                            instead of being copied to the device ahead of the batch (default 8192; 0: always copied)
  *   LNG_COUNT_SECOND_PASSES  long causal prompt passes count the query tiles whose fixed-maximum pass failed its range
  *                            check and was made again with the maximum tracked (read with lng_hip_debug_get)
  * Read at lng_hip_open only: LNG_HSACO (a code object file to load instead of the embedded one). */

@@ -74,6 +74,7 @@ struct Knobs {
     bool wide_row_by_row = false;  // LNG_WIDE_ROW_BY_ROW: prompt passes of head widths 128-512 row by row on the decode kernels
     int prefill_stream = -1;       // LNG_PREFILL_STREAM: 0 never the resident prompt-pass kernel, 1 whenever it can run, -1 planner
     int prefill_upfront = -1;      // LNG_PREFILL_UPFRONT: 0 narrow windows on the tile-by-tile kernel
+    int table_in_place = 8192;     // LNG_TABLE_IN_PLACE: row tables of this many bytes or more are read from pinned host memory; 0 never
     int prefill_splits = 0;        // LNG_PREFILL_SPLITS: workgroups per (query tile, kv head) of a split prompt pass; 0 planner
     int checksum_wgs = 0;          // LNG_CHECKSUM_WGS: workgroups per compute unit of the streaming read; 0 default (2)
     bool count_second_passes = false; // LNG_COUNT_SECOND_PASSES: long causal passes count the query tiles they repeat
@@ -81,11 +82,12 @@ struct Knobs {
     long fuse_wgs = -1;            // LNG_FUSE_WGS: largest grid that merges inside the decode kernel; -1 default
 };
 
-struct Table { // one pinned-host / device pair holding row tables of batched dispatches
+struct Table { // row tables of batched dispatches: a pinned-host block and its device twin, or (in_place) a pinned-host block the kernels read
     char *host = nullptr;
-    char *dev = nullptr;
+    char *dev = nullptr; // == host when in_place
     size_t cap = 0;
     size_t used = 0;
+    bool in_place = false;
 };
 
 struct Cmd {
@@ -269,7 +271,7 @@ int check_shape(const lng_grouped_shape &s, bool tiled) {
 // One development switch by its environment name; value NULL puts the default back. Returns false for an unknown name.
 const char *const knob_names[] = {"LNG_WIDE_GENERIC", "LNG_F32_GENERIC", "LNG_PLAIN_ROW_BY_ROW", "LNG_DECODE_O3", "LNG_MERGE_WIDE",
                                   "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_UPFRONT",
-                                  "LNG_PREFILL_SPLITS", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES", "LNG_CHECKSUM_WGS"};
+                                  "LNG_PREFILL_SPLITS", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES", "LNG_CHECKSUM_WGS", "LNG_TABLE_IN_PLACE"};
 bool set_knob(lng_gpu *g, const char *name, const char *value) {
     Knobs &k = g->knobs;
     const Knobs defaults;
@@ -287,6 +289,10 @@ bool set_knob(lng_gpu *g, const char *name, const char *value) {
     if (!strcmp(name, "LNG_PREFILL_STREAM")) return choice(k.prefill_stream, defaults.prefill_stream);
     if (!strcmp(name, "LNG_PREFILL_UPFRONT")) return choice(k.prefill_upfront, defaults.prefill_upfront);
     if (!strcmp(name, "LNG_CHECKSUM_WGS")) return choice(k.checksum_wgs, defaults.checksum_wgs);
+    if (!strcmp(name, "LNG_TABLE_IN_PLACE")) {
+        k.table_in_place = value ? (int)std::max(0l, std::min(n, 1l << 30)) : defaults.table_in_place;
+        return true;
+    }
     if (!strcmp(name, "LNG_PREFILL_SPLITS")) {
         k.prefill_splits = value ? (int)std::max(1l, std::min(n, 64l)) : 0;
         return true;
@@ -361,14 +367,29 @@ int reserve_scratch(lng_gpu *g, size_t o_floats, size_t ml_floats, size_t n_tick
 }
 
 // Space for a row table: pinned host memory now, its device twin filled at commit.
-int reserve_table(lng_batch *b, size_t bytes, char **host, char **dev) {
+// A table of up to a few kilobytes is copied to the device ahead of the batch's kernels (one copy per block of
+// tables: about 3 us and a dependency); a larger one stays in pinned host memory and the kernels read it there - the
+// copy of a 17 KB table took 10 us of a 217 us dispatch of 128 sequences, and a workgroup reads only its own row and
+// a few running counts (LNG_TABLE_IN_PLACE: the size in bytes from which tables stay; 0 never).
+// `decides`: the size that says where the table goes, when it is not the table's own (the running counts of a row
+// table go where the rows went).
+int reserve_table(lng_batch *b, size_t bytes, char **host, char **dev, size_t decides = 0) {
     lng_gpu *g = b->gpu;
-    if (b->tables.empty() || b->tables.back().cap - b->tables.back().used < bytes) {
+    const bool in_place = g->knobs.table_in_place > 0 && (decides ? decides : bytes) >= (size_t)g->knobs.table_in_place;
+    Table *block = nullptr;
+    for (size_t i = b->tables.size(); i-- > 0;) { // the newest block of the kind that has room
+        Table &t = b->tables[i];
+        if (t.in_place == in_place) {
+            if (t.cap - t.used >= bytes) block = &t;
+            break;
+        }
+    }
+    if (!block) {
         Table t;
         {
             std::lock_guard<std::mutex> lock(g->mu);
             for (size_t i = 0; i < g->free_tables.size(); ++i) {
-                if (g->free_tables[i].cap >= bytes) {
+                if (g->free_tables[i].cap >= bytes && g->free_tables[i].in_place == in_place) {
                     t = g->free_tables[i];
                     g->free_tables.erase(g->free_tables.begin() + i);
                     break;
@@ -377,16 +398,20 @@ int reserve_table(lng_batch *b, size_t bytes, char **host, char **dev) {
         }
         if (!t.host) {
             t.cap = std::max<size_t>(bytes, 64 * 1024);
+            t.in_place = in_place;
             if (hipHostMalloc((void **)&t.host, t.cap, hipHostMallocDefault) != hipSuccess) return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte pinned table", t.cap);
-            if (hipMalloc((void **)&t.dev, t.cap) != hipSuccess) {
+            if (in_place) {
+                t.dev = t.host; // (pinned host memory has the same address on the device)
+            } else if (hipMalloc((void **)&t.dev, t.cap) != hipSuccess) {
                 hipHostFree(t.host);
                 return fail(LNG_ERR_ALLOC, "could not allocate a %zu-byte device table", t.cap);
             }
         }
         t.used = 0;
         b->tables.push_back(t);
+        block = &b->tables.back();
     }
-    Table &t = b->tables.back();
+    Table &t = *block;
     *host = t.host + t.used;
     *dev = t.dev + t.used;
     t.used += (bytes + 255) / 256 * 256;
@@ -669,7 +694,7 @@ int record_rows(lng_batch *b, lng_k_attn a, const lng_k_row *host_rows, size_t n
         uint64_t live = 0;
         for (size_t r = 0; r < n_rows; ++r) live += (visible_from_tile(host_rows[r]) + p.chunks.chunk - 1) / p.chunks.chunk;
         if (live < (uint64_t)n_rows * p.chunks.n_chunks && live * a.kv_heads <= 0x7fffffffull) {
-            if (int rc = reserve_table(b, (n_rows + 1) * 4, &work_host, &work_dev)) return rc;
+            if (int rc = reserve_table(b, (n_rows + 1) * 4, &work_host, &work_dev, n_rows * sizeof(lng_k_row))) return rc;
         }
     }
     RowsLaunches launches;
@@ -1052,7 +1077,7 @@ void destroy_gpu(lng_gpu *g) {
     hipSetDevice(g->device);
     for (Table &t : g->free_tables) {
         hipHostFree(t.host);
-        hipFree(t.dev);
+        if (!t.in_place) hipFree(t.dev);
     }
     for (void *p : g->retired) hipFree(p);
     for (hipEvent_t ev : g->spare_events) hipEventDestroy(ev);
@@ -1248,7 +1273,7 @@ extern "C" int lng_hip_batch_commit(lng_batch *b, lng_on_done on_done, void *use
     // the row tables of every batched dispatch, one copy per table block, ahead of the kernels
     for (size_t i = 0; e == hipSuccess && i < b->tables.size(); ++i) {
         const Table &t = b->tables[i];
-        if (t.used) e = hipMemcpyAsync(t.dev, t.host, t.used, hipMemcpyHostToDevice, g->stream);
+        if (t.used && !t.in_place) e = hipMemcpyAsync(t.dev, t.host, t.used, hipMemcpyHostToDevice, g->stream);
     }
     for (size_t i = 0; e == hipSuccess && i < b->cmds.size(); ++i) {
         Cmd &c = b->cmds[i];
