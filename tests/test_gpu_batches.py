@@ -9,7 +9,7 @@ import pytest
 
 from loadngo_amd import compute as C
 from oracle import oracle as orc
-from tests.gpu_common import THREADS, gpu  # noqa: F401
+from tests.gpu_common import THREADS, gpu, knobs  # noqa: F401
 from tests.helpers import from_bf16_bits, normal_inputs, to_bf16_bits
 
 pytestmark = pytest.mark.gpu
@@ -121,6 +121,50 @@ def test_a_dispatch_of_more_rows_than_one_grid_dimension_holds(gpu):
     for i in list(rng.integers(0, n, 60)) + [0, n - 1, 17, 4000, 4001, 4002, 8999, 8998, int(np.argmin(lens))]:
         want = orc.attention_bf16(q[i:i + 1], k[:lens[i]], v[:lens[i]], sinks, int(lens[i]) - 1, scale=0.125)
         assert np.abs(got[i] - from_bf16_bits(want[0])).max() < 2e-2, (i, lens[i])
+
+
+def test_a_row_table_read_from_host_memory_and_one_copied_to_the_device_give_the_same_rows(gpu, knobs):
+    """A table of 8 KB or more stays in pinned host memory, where the kernels read it; smaller ones are copied to the
+    device ahead of the batch. 300 sequences of unequal length (a 19 KB table and its running counts) both ways, and
+    with every table left in host memory (LNG_TABLE_IN_PLACE=1): the same bits, and right against the oracle."""
+    n, ctx = 300, 6000
+    rng = np.random.default_rng(78)
+    k = to_bf16_bits((rng.standard_normal((ctx, G, D)) * 0.5).astype(np.float32))
+    v = to_bf16_bits((rng.standard_normal((ctx, G, D)) * 0.5).astype(np.float32))
+    q = to_bf16_bits((rng.standard_normal((n, H, D)) * 0.5).astype(np.float32))
+    sinks = rng.standard_normal(H).astype(np.float32)
+    lens = rng.integers(1, ctx + 1, size=n)
+    items = [C.DecodeItem(i * H * D * 2, i * H * D * 2, 0, 0, 0, int(lens[i]) - 1, C.FULL if i % 3 else 128, int(lens[i])) for i in range(n)]
+    few = items[:40] # a 2.5 KB table: copied unless every table stays
+    results = {}
+    for mode in (None, "0", "1"):
+        if mode is None:
+            knobs.delenv("LNG_TABLE_IN_PLACE", raising=False)
+        else:
+            knobs.setenv("LNG_TABLE_IN_PLACE", mode)
+        bufs = [gpu.upload(q), gpu.upload(k), gpu.upload(v), gpu.buffer(2 * q.nbytes), gpu.upload(sinks)]
+        bufs[3].fill(0xFF)
+        batch = gpu.batch(bufs)
+        batch.attention_decode_batched(0, 1, 2, 3, 4, items, H, G, D, 0.125, C.BF16)
+        shifted = [C.DecodeItem(it.q_offset, q.nbytes + it.out_offset, it.k_offset, it.v_offset, it.sinks_offset, it.start, it.window, it.slots)
+                   for it in few]
+        batch.attention_decode_batched(0, 1, 2, 3, 4, shifted, H, G, D, 0.125, C.BF16)
+        done = batch.run()
+        assert not isinstance(done.gpu_time, Exception)
+        results[mode] = bufs[3].read(np.uint16).reshape(2, n, H, D).copy()
+        batch.drop()
+        for b in bufs:
+            b.free()
+    got = results[None]
+    assert np.array_equal(got, results["0"]) and np.array_equal(got, results["1"])
+    rows = from_bf16_bits(got[0])
+    assert np.abs(rows[:40] - from_bf16_bits(got[1, :40])).max() < 2e-2  # split differently, so not the same bits
+    assert not np.isnan(rows).any()
+    for i in list(rng.integers(0, n, 25)) + [0, n - 1]:
+        window = None if i % 3 else 128
+        want = orc.attention_bf16(q[i:i + 1], k[:lens[i]], v[:lens[i]], sinks, int(lens[i]) - 1, scale=0.125,
+                                  **({} if window is None else {"window": window}))
+        assert np.abs(rows[i] - from_bf16_bits(want[0])).max() < 2e-2, (i, lens[i])
 
 
 def test_many_small_decodes_merged_inside_the_kernel(gpu):
