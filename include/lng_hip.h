@@ -109,6 +109,7 @@ int lng_hip_device_name(lng_gpu *gpu, char *name, size_t cap);
  *   LNG_PLAIN_ROW_BY_ROW     the row-by-row operator never takes a prompt-pass kernel
  *   LNG_WIDE_ROW_BY_ROW      prompt passes of head widths 128-512 row by row on the decode kernels
  *   LNG_PREFILL_STREAM 0|1   never / whenever possible the prompt-pass kernel whose workgroups walk several query tiles
+ *   LNG_PREFILL_PAIR 0|1     never / whenever possible the prompt-pass kernel of one workgroup per (query tile, kv head, pair of heads)
  *   LNG_PREFILL_UPFRONT 0    narrow windows on the tile-by-tile kernel
  *   LNG_PREFILL_SPLITS n     workgroups per (query tile, kv head) of a prompt pass with fewer workgroups than compute units
  *   LNG_Q8_W16               the one-position Q8_0 kernel always as 16-wavefront workgroups

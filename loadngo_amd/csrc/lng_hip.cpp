@@ -73,6 +73,7 @@ struct Knobs {
     bool q8_w16 = false;           // LNG_Q8_W16: the one-position Q8_0 kernel always as 16-wavefront workgroups
     bool wide_row_by_row = false;  // LNG_WIDE_ROW_BY_ROW: prompt passes of head widths 128-512 row by row on the decode kernels
     int prefill_stream = -1;       // LNG_PREFILL_STREAM: 0 never the resident prompt-pass kernel, 1 whenever it can run, -1 planner
+    int prefill_pair = -1;         // LNG_PREFILL_PAIR: 0 never the head-pair prompt-pass kernel, 1 whenever it can run, -1 planner
     int prefill_upfront = -1;      // LNG_PREFILL_UPFRONT: 0 narrow windows on the tile-by-tile kernel
     int table_in_place = 8192;     // LNG_TABLE_IN_PLACE: row tables of this many bytes or more are read from pinned host memory; 0 never
     int prefill_splits = 0;        // LNG_PREFILL_SPLITS: workgroups per (query tile, kv head) of a split prompt pass; 0 planner
@@ -116,7 +117,7 @@ struct lng_gpu {
     hipFunction_t generic_f32 = nullptr, generic_bf16 = nullptr;
     hipFunction_t decode_bf16_d64 = nullptr, decode_bf16_d64_o4 = nullptr, decode_f32_d64 = nullptr, decode_merge = nullptr, decode_merge_few = nullptr;
     hipFunction_t decode_bf16_wide[3] = {}, decode_f32_wide[3] = {}; // head widths 128, 256, 512
-    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_h1w = nullptr, prefill_bf16_d64_stream = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
+    hipFunction_t prefill_bf16_d64 = nullptr, prefill_bf16_d64_h1 = nullptr, prefill_bf16_d64_h1w = nullptr, prefill_bf16_d64_stream = nullptr, prefill_bf16_d64_pair = nullptr, prefill_f32_d64 = nullptr, prefill_f32_d64_w4 = nullptr, prefill_merge = nullptr;
     hipFunction_t prefill_bf16_wide[3] = {}, prefill_f32_wide[3] = {}; // head widths 128, 256, 512
     hipFunction_t checksum = nullptr, checksum_fold = nullptr;
     hipFunction_t copy_rows = nullptr, fill_synthetic = nullptr, add_rows = nullptr, rotate_halves = nullptr, rmsnorm_rows = nullptr, rmsnorm_row_wg = nullptr;
@@ -270,7 +271,7 @@ int check_shape(const lng_grouped_shape &s, bool tiled) {
 
 // One development switch by its environment name; value NULL puts the default back. Returns false for an unknown name.
 const char *const knob_names[] = {"LNG_WIDE_GENERIC", "LNG_F32_GENERIC", "LNG_PLAIN_ROW_BY_ROW", "LNG_DECODE_O3", "LNG_MERGE_WIDE",
-                                  "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_UPFRONT",
+                                  "LNG_Q8_W16", "LNG_WIDE_ROW_BY_ROW", "LNG_PREFILL_STREAM", "LNG_PREFILL_PAIR", "LNG_PREFILL_UPFRONT",
                                   "LNG_PREFILL_SPLITS", "LNG_DECODE_WGS", "LNG_FUSE_WGS", "LNG_COUNT_SECOND_PASSES", "LNG_CHECKSUM_WGS", "LNG_TABLE_IN_PLACE"};
 bool set_knob(lng_gpu *g, const char *name, const char *value) {
     Knobs &k = g->knobs;
@@ -287,6 +288,7 @@ bool set_knob(lng_gpu *g, const char *name, const char *value) {
     if (!strcmp(name, "LNG_WIDE_ROW_BY_ROW")) return flag(k.wide_row_by_row);
     if (!strcmp(name, "LNG_COUNT_SECOND_PASSES")) return flag(k.count_second_passes);
     if (!strcmp(name, "LNG_PREFILL_STREAM")) return choice(k.prefill_stream, defaults.prefill_stream);
+    if (!strcmp(name, "LNG_PREFILL_PAIR")) return choice(k.prefill_pair, defaults.prefill_pair);
     if (!strcmp(name, "LNG_PREFILL_UPFRONT")) return choice(k.prefill_upfront, defaults.prefill_upfront);
     if (!strcmp(name, "LNG_CHECKSUM_WGS")) return choice(k.checksum_wgs, defaults.checksum_wgs);
     if (!strcmp(name, "LNG_TABLE_IN_PLACE")) {
@@ -796,7 +798,28 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         // every full-causal pass it can run (tests: small shapes), otherwise only when every compute unit has a tile.
         const bool stream_can = !f32 && !narrow && p.window == LNG_WINDOW_FULL && s.slots >= end && g->knobs.prefill_stream != 0;
         const bool stream = stream_can && (plain_wgs >= g->cus || g->knobs.prefill_stream == 1);
-        if (!stream && (!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
+        // Between the two - 64-row tiles, but fewer (query tile, kv head) pairs than compute units (a prompt fed 512 rows
+        // at a time) - a workgroup per (query tile, kv head, PAIR of heads) that deals the keys out among its own
+        // wavefronts: four times the workgroups and nothing to merge afterwards. From half the units busy on
+        // (LNG_PREFILL_PAIR: 0 never, 1 whenever it can run).
+        const uint64_t head_pairs = (s.heads / s.kv_heads + 1) / 2;
+        const bool pair_can = !f32 && !narrow && !stream && g->knobs.prefill_pair != 0 && g->knobs.prefill_splits == 0;
+        bool pair = pair_can && g->knobs.prefill_pair == 1;
+        if (pair_can && g->knobs.prefill_pair < 0 && plain_wgs < g->cus && head_pairs > 1) {
+            // Which is faster depends on how many keys a call walks: a head-pair workgroup walks all of them (measured
+            // on 64/8 heads: 15 us + 1.9 us per 256 keys, half as much again per key beyond 6,656, where a kv head's K
+            // and V no longer stay in its XCD's L2; as many rounds as the workgroups need on the device's units), a
+            // split workgroup only its share (25 us + 1.6 us per 64 keys of it, and 8 us for the merge dispatch).
+            // 8,192 positions in calls of 512 rows: 857 -> 735 us; 4,096 in calls of 256: 508 -> 451 us; 2,048 in calls
+            // of 128: 385 -> 313 us; but calls of 256 rows at 8,192 positions and of 512 rows at 16,384 are slower.
+            const double keys = (double)visible;
+            const uint64_t rounds = (plain_wgs * head_pairs + g->cus - 1) / g->cus;
+            const double pair_us = 15.0 + (double)rounds * (1.9 / 256.0) * (keys + (keys > 6656.0 ? 0.5 * (keys - 6656.0) : 0.0));
+            const uint64_t would_split = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, key_tiles / 4), 64));
+            const double split_us = 25.0 + (would_split > 1 && key_tiles >= 12 ? 8.0 + (1.6 / 64.0) * keys / (double)would_split : (1.6 / 64.0) * keys);
+            pair = pair_us < split_us;
+        }
+        if (!stream && !pair && (!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
             uint64_t want = g->cus / plain_wgs;
             want = std::min<uint64_t>(want, key_tiles / 4);
             want = std::min<uint64_t>(want, 64);
@@ -822,13 +845,14 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             const uint64_t per_head = std::min<uint64_t>(p.q_tiles, std::max<uint64_t>(1, g->cus / s.kv_heads));
             c.grid[0] = (unsigned)(per_head * s.kv_heads);
         }
+        if (pair) c.grid[0] = (unsigned)(plain_wgs * head_pairs);
         // f32: two workgroups per compute unit only when there are four rounds of them or more (see the kernels)
         const bool f32_two = f32 && c.grid[0] >= 4u * g->cus;
         // Windows of up to 160 positions: the 32 query rows of a workgroup see at most four tiles of 64 keys, and the
         // one-head kernel asks for all of them at its start, straight into LDS (LNG_PREFILL_UPFRONT=0: never).
         const bool upfront = narrow && p.window != LNG_WINDOW_FULL && p.window <= 160 && p.splits == 1 && g->knobs.prefill_upfront != 0;
-        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : upfront ? g->prefill_bf16_d64_h1w : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : g->prefill_bf16_d64;
-        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : upfront ? "lng_prefill_bf16_d64_h1w" : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : "lng_prefill_bf16_d64";
+        c.fn = f32 ? (f32_two ? g->prefill_f32_d64_w4 : g->prefill_f32_d64) : upfront ? g->prefill_bf16_d64_h1w : narrow ? g->prefill_bf16_d64_h1 : stream ? g->prefill_bf16_d64_stream : pair ? g->prefill_bf16_d64_pair : g->prefill_bf16_d64;
+        c.name = f32 ? (f32_two ? "lng_prefill_f32_d64_w4" : "lng_prefill_f32_d64") : upfront ? "lng_prefill_bf16_d64_h1w" : narrow ? "lng_prefill_bf16_d64_h1" : stream ? "lng_prefill_bf16_d64_stream" : pair ? "lng_prefill_bf16_d64_pair" : "lng_prefill_bf16_d64";
         set_args(c, p);
         b->cmds.push_back(std::move(c));
         if (p.splits > 1) {
@@ -998,6 +1022,7 @@ extern "C" int lng_hip_open(int device, lng_gpu **out) {
         {"lng_prefill_bf16_d64_h1", &g->prefill_bf16_d64_h1, true},
         {"lng_prefill_bf16_d64_h1w", &g->prefill_bf16_d64_h1w, true},
         {"lng_prefill_bf16_d64_stream", &g->prefill_bf16_d64_stream, true},
+        {"lng_prefill_bf16_d64_pair", &g->prefill_bf16_d64_pair, true},
         {"lng_prefill_f32_d64", &g->prefill_f32_d64, true},
         {"lng_prefill_f32_d64_w4", &g->prefill_f32_d64_w4, true},
         {"lng_prefill_merge", &g->prefill_merge, true},

@@ -3860,4 +3860,5 @@ extern "C" __global__ __launch_bounds__(256) void lng_prefill_merge(lng_k_prefil
     merge_chunks<false>(a, it, blockIdx.y, g, group, p.splits);
 }
 
+#include "lng_prefill_pair.h"
 #include "lng_prefill_wide.h"

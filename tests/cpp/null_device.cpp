@@ -221,7 +221,10 @@ static void switches_and_checksum() {
         lng_k_prefill p{};
         CHECK(args_size == sizeof p);
         memcpy(&p, args, sizeof p);
-        CHECK(grid[0] == p.q_tiles * p.kv_heads * p.splits);
+        // (the kernel of a workgroup per pair of heads never splits: its grid has the pairs instead)
+        const bool pairs = !strcmp(name, "lng_prefill_bf16_d64_pair");
+        CHECK(grid[0] == p.q_tiles * p.kv_heads * (pairs ? (p.heads / p.kv_heads + 1) / 2 : p.splits));
+        CHECK(!pairs || p.splits == 1);
         CHECK(p.splits == 1 || lng_null_launch_count() == 2);
         lng_null_clear();
         f.rebatch();
@@ -233,6 +236,36 @@ static void switches_and_checksum() {
     CHECK(lng_hip_debug_set(f.gpu, "LNG_PREFILL_SPLITS", nullptr) == LNG_OK);
     const uint32_t planned = prefill_splits(); // the planner's own: one workgroup per compute unit, four key tiles each at least
     CHECK(planned >= 1 && planned <= 4);
+    // a prompt fed 512 rows at a time (64 heads over 8): 64 (query tile, kv head) pairs on 256 units go to the kernel of a
+    // workgroup per pair of heads while a call walks few enough keys, and to split keys plus a merge beyond that
+    {
+        Fixture big(5, 40 * MB);
+        auto chunk_call = [&](uint64_t start, const char *want_kernel, unsigned want_grid, size_t want_launches) {
+            const lng_grouped_shape s = shape(512, start, 64, 8, 64, LNG_WINDOW_FULL, start + 512, 0.125f);
+            const lng_slice q{0, 0, 512 * 64 * 64 * 2}, k{1, 0, (start + 512) * 8 * 64 * 2}, v{2, 0, (start + 512) * 8 * 64 * 2}, o{3, 0, 512 * 64 * 64 * 2};
+            lng_null_clear();
+            CHECK(lng_hip_attention_grouped_tiled(big.batch, q, k, v, o, nullptr, &s, LNG_BF16) == LNG_OK);
+            CHECK(lng_hip_batch_commit(big.batch, nullptr, nullptr) == LNG_OK);
+            CHECK(lng_hip_batch_wait(big.batch, nullptr) == LNG_OK);
+            const char *name = nullptr;
+            const void *args = nullptr;
+            size_t args_size = 0;
+            unsigned grid[3], block[3];
+            CHECK(lng_null_launch_count() == want_launches && lng_null_launch(0, &name, grid, block, &args, &args_size) == 0);
+            CHECK(!strcmp(name, want_kernel) && grid[0] == want_grid && block[0] == 512);
+            big.rebatch();
+        };
+        const unsigned cus = 256; // the null device's
+        chunk_call(3584, "lng_prefill_bf16_d64_pair", 8 * 8 * 4, 1);
+        chunk_call(0, "lng_prefill_bf16_d64_pair", 8 * 8 * 4, 1);
+        chunk_call(15872, "lng_prefill_bf16_d64", cus, 2);
+        CHECK(lng_hip_debug_set(big.gpu, "LNG_PREFILL_PAIR", "0") == LNG_OK);
+        chunk_call(3584, "lng_prefill_bf16_d64", cus, 2);
+        CHECK(lng_hip_debug_set(big.gpu, "LNG_PREFILL_PAIR", "1") == LNG_OK);
+        chunk_call(15872, "lng_prefill_bf16_d64_pair", 8 * 8 * 4, 1);
+        CHECK(lng_hip_debug_set(big.gpu, "LNG_PREFILL_PAIR", nullptr) == LNG_OK);
+        lng_null_clear();
+    }
     CHECK(refused(lng_hip_debug_set(f.gpu, "LNG_NO_SUCH_SWITCH", "1"), "no development switch"));
     CHECK(refused(lng_hip_debug_set(f.gpu, nullptr, "1"), "no name"));
     CHECK(lng_hip_debug_set(nullptr, "LNG_PREFILL_SPLITS", "1") != LNG_OK);

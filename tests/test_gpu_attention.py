@@ -364,14 +364,21 @@ def test_several_rows_through_the_row_by_row_operator_over_long_caches(gpu, t, s
     assert max_error(rows, want) < BF16_TOL and np.abs(rows - got).max() < 2.0 ** -6
 
 
-@pytest.mark.parametrize("stream", ["0", "1"])
+def long_causal_kernel(knobs, which):
+    """"0": one workgroup per (query tile, kv head); "1": workgroups that walk several query tiles; "pair": one
+    workgroup per (query tile, kv head, pair of heads), its wavefronts sharing out the keys."""
+    knobs.setenv("LNG_PREFILL_STREAM", "0" if which == "pair" else which)
+    knobs.setenv("LNG_PREFILL_PAIR", "1" if which == "pair" else "0")
+
+
+@pytest.mark.parametrize("stream", ["0", "1", "pair"])
 @pytest.mark.parametrize("spike_at,sinks_on", [(300, True), (300, False), (5, True), (5, False), (700, True)])
 def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sinks_on, stream, knobs):
     """Long causal passes first keep the running maximum fixed after one interior tile and check the
     normalisers afterwards. A key whose score is about 10,000 above the rest (2^10000 cannot be held)
     late in the pass must send the workgroup through the pass that tracks the maximum; the same key
     early in the pass, or a cache whose scores all sit far below the first tile's, must not lose anything."""
-    knobs.setenv("LNG_PREFILL_STREAM", stream)  # both kernels of the long causal pass (see the next test)
+    long_causal_kernel(knobs, stream)  # every kernel of the long causal pass (see the next test)
     t, heads, kv_heads = 1024, 16, 2
     q, k, v, sinks = normal_inputs(91 + spike_at, t, t, heads, kv_heads, 64, scale=0.5)
     q[:] = np.abs(q) + 1.0                      # every query has a large positive overlap with the spike key
@@ -389,7 +396,7 @@ def test_prefill_bf16_with_scores_far_outside_the_usual_range(gpu, spike_at, sin
     assert np.abs(late - from_bf16_bits(vb)[spike_at][None, :, None, :].repeat(heads // kv_heads, 2).reshape(1, heads, 64)).max() < BF16_TOL
 
 
-@pytest.mark.parametrize("stream", ["0", "1"])
+@pytest.mark.parametrize("stream", ["0", "1", "pair"])
 @pytest.mark.parametrize("case", ["all_far_below", "all_far_above", "huge_sink", "std4", "far_above_then_usual"])
 def test_long_causal_passes_with_every_score_far_outside_the_usual_range(gpu, case, stream, knobs):
     """The long causal kernels (both: workgroups that walk several query tiles, and one tile per workgroup) fold
@@ -397,8 +404,9 @@ def test_long_causal_passes_with_every_score_far_outside_the_usual_range(gpu, ca
     score of a row below -600 or above 600, with sinks of +-300, with Gaussian scores of standard deviation 4
     (sixteen times the benign fills'), and with scores that sit near +600 for the first tiles and near zero after
     them, the range check must send the rows that need it through the tracked pass and the result must stay
-    within the bf16 bar of the CPU reference, with and without sinks."""
-    knobs.setenv("LNG_PREFILL_STREAM", stream)
+    within the bf16 bar of the CPU reference, with and without sinks. The kernel of a workgroup per pair of heads
+    (calls of few rows) runs the same scheme and is put through the same cases."""
+    long_causal_kernel(knobs, stream)
     t, heads, kv_heads = 1024, 16, 2
     q, k, v, sinks = normal_inputs(17 + len(case), t, t, heads, kv_heads, 64, scale=0.5)
     if case == "all_far_below":   # q . k about -64 * 1.4 * 9 * 8 * 0.125 = -800
@@ -421,7 +429,7 @@ def test_long_causal_passes_with_every_score_far_outside_the_usual_range(gpu, ca
     for sk in (sinks, None):
         want = oracle.attention_bf16(qb, kb, vb, sk, 0, scale=0.125, threads=THREADS)
         got = run_attention(gpu, qb, kb, vb, sk, shape, True, C.BF16,
-                            expect_kernel="lng_prefill_bf16_d64_stream" if stream == "1" else "lng_prefill_bf16_d64")
+                            expect_kernel={"0": "lng_prefill_bf16_d64", "1": "lng_prefill_bf16_d64_stream", "pair": "lng_prefill_bf16_d64_pair"}[stream])
         assert max_error(from_bf16_bits(got), from_bf16_bits(want)) < BF16_TOL
 
 
@@ -535,14 +543,16 @@ def test_long_causal_pass_on_workgroups_that_walk_several_query_tiles(gpu, t, st
     assert np.abs(got - other).max() <= 2.0 ** -7  # a bf16 step or two at |o| < 1
 
 
-@pytest.mark.parametrize("t,start,heads,kv_heads,window", [(2048, 1000, 64, 8, FULL), (1000, 0, 32, 8, FULL),
-                                                          (2048, 1000, 64, 8, 128), (1000, 37, 24, 4, 100)])
-def test_long_passes_give_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, window, knobs):
+@pytest.mark.parametrize("t,start,heads,kv_heads,window,kernel", [
+    (2048, 1000, 64, 8, FULL, "1"), (1000, 0, 32, 8, FULL, "1"), (2048, 1000, 64, 8, 128, "1"), (1000, 37, 24, 4, 100, "1"),
+    (512, 1536, 64, 8, FULL, "pair"), (300, 2900, 24, 4, 2500, "pair")])
+def test_long_passes_give_the_same_bits_every_launch(gpu, t, start, heads, kv_heads, window, kernel, knobs):
     """The resident kernel's wavefronts pass the tile barrier at two different places of their sequence and share
-    three LDS buffers; the kernel for narrow windows reads rows that other wavefronts' loads wrote straight into
-    LDS: 256 launches over the same inputs, each into its own output, all bit for bit the first (an LDS row
-    overwritten early or read late would show as a launch that differs)."""
-    knobs.setenv("LNG_PREFILL_STREAM", "1")
+    three LDS buffers; the kernel for narrow windows and the one of a workgroup per pair of heads read rows that
+    other wavefronts' loads wrote straight into LDS (the latter into two buffers in turn, and its wavefronts exchange
+    their accumulators through the same memory at the end): 256 launches over the same inputs, each into its own
+    output, all bit for bit the first (an LDS row overwritten early or read late would show as a launch that differs)."""
+    long_causal_kernel(knobs, kernel)
     dim, per_batch, end = 64, 32, start + t
     rows, krows = (t + 31) // 32 * 32, (end + 31) // 32 * 32
     one = rows * heads * dim * 2
