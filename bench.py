@@ -554,8 +554,8 @@ def run_prefill(gpu, steps, warmup, t=8192):
                      "back_to_back_mfma_frac": flops / sustained / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                      "qkvo_bytes": traffic, "hbm_frac": traffic / g / 1e9 / HBM_PEAK_GBS}
     # the same full-causal pass the way the reference makes it: 512 rows at a time (engine.rs:51), 16 calls in
-    # one batch; too few query tiles per call to fill the device, so the library splits the keys of a tile
-    # between workgroups and merges (lng_prefill_merge)
+    # one batch; too few query tiles per call to fill the device, so the library takes the kernel of a workgroup
+    # per pair of heads (lng_prefill_bf16_d64_pair)
     chunk = 512
     pairs = t * (t + 1) // 2
 
