@@ -380,9 +380,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         bad = row_ok ? bad : 0;
         if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) s_again = 1u;
         __syncthreads();
-        again = s_again != 0u;
-        __syncthreads(); // everyone has read it
-        s_again = 0u;
+        again = s_again != 0u; // (written in the first attempt only, which alone has a check: never cleared)
         if (again && a.second_passes && wave == 0u && lane == 0u) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!again) {
