@@ -168,12 +168,17 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         const uint32_t w = (l31 == 0u || l31 == 17u) ? 0x3f803f80u : 0u;
         return as_bf16x8(make_uint4(w, w, w, w));
     };
-    constexpr int ATTEMPTS = 2;
+    // Three ways to make the pass, each a fallback of the one before: (0) every step at the reference point zero, with no
+    // maxima at all, when the run begins with interior steps - the range check below is all that correctness needs (a
+    // softmax does not depend on its reference point, only the number range does), and it passes whenever a row's
+    // largest score is between about -70 and 80 in the exponent's units; (1) the first interior step with the maxima
+    // tracked, the rest fixed there; (2) the maxima tracked throughout.
+    constexpr int ATTEMPTS = 3;
     for (int attempt = 0; attempt < ATTEMPTS; ++attempt) {
-    const bool optimistic = attempt == 0;
+    const bool optimistic = attempt < 2;
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
-        m[h] = LNG_NEG_INF; // the sink joins when the wavefronts' states are put together
+        m[h] = LNG_NEG_INF; // the sink joins when the wavefronts' states are put together (0 below, for way (0))
         l[h] = 0.0f;
         lacc[h] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -317,7 +322,14 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         landed();
     };
     uint32_t s = 0;
-    bool frozen = false;
+    bool frozen = false, at_zero = false;
+    const bool speculate = attempt == 0 && interior(0) && interior(1);
+    if (speculate) {
+        frozen = true;
+        at_zero = true;
+#pragma unroll
+        for (int h = 0; h < NH; ++h) m[h] = 0.0f;
+    } else {
     for (; s < n_steps && !(optimistic && interior(s)); ++s) { // all of a tracked attempt; else up to the first interior step
         any_step(s);
         landed();
@@ -336,7 +348,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         }
         if (__builtin_amdgcn_ballot_w64(!moderate) != 0) s_far = 1u;
         landed();
-        const bool at_zero = s_far == 0u; // (set at most once in a launch: never cleared)
+        at_zero = s_far == 0u; // (never cleared: what it says of the scores holds for a later attempt as well)
         if (at_zero) {
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
@@ -349,6 +361,11 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
                 }
                 m[h] = 0.0f;
             }
+        }
+    }
+    }
+    if (frozen) { // loops of their own: one path through each
+        if (at_zero) {
             for (; s < n_steps && interior(s); ++s) fixed_step(fixed_at_zero{}, s);
         } else {
             for (; s < n_steps && interior(s); ++s) fixed_step(fixed_at_m{}, s);
@@ -380,8 +397,13 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         bad = row_ok ? bad : 0;
         if (__builtin_amdgcn_ballot_w64(bad != 0) != 0) s_again = 1u;
         __syncthreads();
-        again = s_again != 0u; // (written in the first attempt only, which alone has a check: never cleared)
-        if (again && a.second_passes && wave == 0u && lane == 0u) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        again = s_again != 0u;
+        if (again) {
+            __syncthreads(); // everyone has read it
+            s_again = 0u;    // for the next attempt's check: its barriers lie between
+            if (a.second_passes && wave == 0u && lane == 0u) __hip_atomic_fetch_add(a.second_passes, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (!speculate) attempt = 1; // fixing the maxima after a tracked step has failed: track them throughout
+        }
     }
     if (!again) {
         for (; s < n_steps; ++s) { // the diagonal
