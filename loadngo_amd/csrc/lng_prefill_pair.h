@@ -367,6 +367,16 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     if (frozen) { // loops of their own: one path through each
         if (at_zero) {
             for (; s < n_steps && interior(s); ++s) fixed_step(fixed_at_zero{}, s);
+            // the step of the diagonal at the same reference point and ahead of the check, which then covers it (a
+            // masked score is 2^-inf = 0; every sub-tile through the masks, so that there is one more form of the block only)
+            for (; s < n_steps; ++s) {
+                if (s + 1u < n_steps) ask(s + 1u);
+                if (4u * s + kq < all_tiles) {
+                    block(std::true_type{}, fixed_at_zero{}, s, 0);
+                    block(std::true_type{}, fixed_at_zero{}, s, 1);
+                }
+                landed();
+            }
         } else {
             for (; s < n_steps && interior(s); ++s) fixed_step(fixed_at_m{}, s);
         }
