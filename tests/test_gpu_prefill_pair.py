@@ -51,6 +51,28 @@ def test_head_pair_kernel_matches_the_cpu_reference(gpu, t, start, window, slots
         assert not np.isnan(got).any() and max_error(got, want) < BF16_TOL
 
 
+@pytest.mark.parametrize("t,start,window,slots", [(100, 3000, FULL, 3100), (63, 2500, 2000, 2063), (40, 5000, FULL, 5040), (333, 700, FULL, 1033)])
+def test_the_row_by_row_operator_on_the_head_pair_kernel(gpu, t, start, window, slots, knobs):
+    """attention_grouped with tens of rows over thousands of keys goes to a prompt-pass kernel as well (the cache is read
+    once, not once per row); its caches are not padded to 32 rows and hold NaN wherever the operator may not read
+    (attention_grouped.rs:57), its queries and outputs have exactly t rows."""
+    knobs.setenv("LNG_PREFILL_STREAM", "0")
+    knobs.setenv("LNG_PREFILL_PAIR", "1")
+    heads, kv_heads = 64, 8
+    end = start + t
+    q, k, v, sinks = normal_inputs(3 * t + start, t, end, heads, kv_heads, 64, scale=0.5)
+    qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+    kr, vr = ring_layout(kb, t, start, slots, False), ring_layout(vb, t, start, slots, False)
+    first = 0 if window == FULL else max(0, start + 1 - window)
+    if slots >= end:
+        kr[:first] = 0x7FC0
+        vr[:first] = 0x7FC0
+    shape = C.GroupedShape(t, start, heads, kv_heads, 64, window, slots, 0.125)
+    want = from_bf16_bits(oracle.attention_bf16(qb, kb, vb, sinks, start, window=window, scale=0.125, threads=THREADS))
+    got = from_bf16_bits(run_attention(gpu, qb, kr, vr, sinks, shape, False, C.BF16, expect_kernel=PAIR))
+    assert not np.isnan(got).any() and max_error(got, want) < BF16_TOL
+
+
 def test_random_shapes_on_the_head_pair_kernel(gpu, knobs):
     """Seeded random shapes: 1..600 rows after 0..5,000 cached positions, groups of 1..8, windows above 1,024 or none,
     flat caches and rings at every phase, with and without sinks."""
