@@ -2806,7 +2806,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
 
 // Windows of at most 160 positions (unsplit passes): lng_prefill_bf16_d64_h1's arithmetic, block for block, with
 // every K and V row of the workgroup requested at its start. A workgroup of eight wavefronts (a head each) takes 32
-// query rows; they see at most 160 + 31 keys, which lie in at most four tiles of 64 rows from a multiple of 64.
+// query rows; they see at most 160 + 31 keys, which lie in at most seven blocks of 32 rows from a multiple of 32 (five
+// for a window of 128 at a start that is a multiple of 32: 160 rows; whole tiles of 64 from a multiple of 64 were 256).
 // These rows are asked for together with the queries by loads that write LDS directly (global_load_lds_dwordx4: no registers in between, so nothing limits how
 // many are in flight); there is one barrier when they have landed, and the blocks of 32 keys then run without any
 // further wait for memory - tile by tile, such a pass spends a memory round trip per tile: the loads of tile i+1
@@ -2816,15 +2817,15 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
 // rows then fall in 16 different 16-byte bank groups - and piece c of V row r at c ^ (((r >> 1) & 1) << 2): the
 // four rows x 64 bytes that half a wavefront reads transposed fall in four different quarters of the banks.
 // After the last block a barrier says that nobody reads K and V any more, and each wavefront lays its rows down
-// there so that eight lanes store a whole 128-byte row. 64 KiB of LDS: two workgroups per compute unit.
+// there so that eight lanes store a whole 128-byte row. 56 KiB of LDS: two workgroups per compute unit.
 // (Measured and not kept: a first pass around zero - weights 2^score, no maxima, the sums on the matrix unit, a range
 // check and the tracked pass again when it fails: 40 % fewer vector instructions per block, same time; workgroups of
 // four wavefronts with two heads each, three to a compute unit with 48 KiB of LDS each: same time; 64 query rows per
 // workgroup as two blocks of 32, one after the other, over the same K and V rows: 42 against 39 us.)
-#define PW_TILES 4
+#define PW_BLOCKS 7 // blocks of 32 keys a workgroup may see: a window of 160, 32 rows, and up to 31 keys before the first
 extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64_h1w(lng_k_prefill a) {
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[PW_TILES * 64 * 64];
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[PW_TILES * 64 * 64];
+    __shared__ __attribute__((aligned(16))) uint16_t s_k[PW_BLOCKS * 32 * 64];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[PW_BLOCKS * 32 * 64];
     const uint32_t g = blockIdx.x % a.kv_heads;
     const uint32_t qtile = a.q_tiles - 1u - blockIdx.x / a.kv_heads;
     const uint32_t group = a.heads / a.kv_heads;
@@ -2841,8 +2842,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
     const uint32_t pos_last = pos_first + rows_here - 1u;
     const uint32_t window = (uint32_t)a.window; // the host sends windows of 1..160 only
     const uint32_t kfirst = pos_first + 1u > window ? pos_first + 1u - window : 0u;
-    const uint32_t tile0 = kfirst & ~63u;
-    const uint32_t n_tiles = min((pos_last - tile0) / 64u + 1u, (uint32_t)PW_TILES);
+    const uint32_t blk0 = kfirst & ~31u; // the rows in LDS begin at a multiple of 32: 160 of them for a window of 128
+    const uint32_t n_blocks = min((pos_last - blk0) / 32u + 1u, (uint32_t)PW_BLOCKS);
     const bool ring = a.slots < end;
     const uint32_t slots = (uint32_t)a.slots;
     const uint64_t row_bytes = (uint64_t)a.kv_heads * 128u;
@@ -2867,8 +2868,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
         const uint32_t ck = ld_chunk ^ ((ld_row >> 1) & 7u), cv = ld_chunk ^ (((ld_row >> 1) & 1u) << 2);
         typedef __attribute__((address_space(1))) const void *gptr;
         typedef __attribute__((address_space(3))) void *lptr;
-        for (uint32_t i = 0; i < n_tiles; ++i) {
-            uint32_t p = tile0 + 64u * i + ld_row;
+        // (eight wavefronts x eight rows at a time; a wavefront whose eight rows lie past the last block asks for nothing)
+        for (uint32_t i = 0; 64u * i + 8u * wave < 32u * n_blocks; ++i) {
+            uint32_t p = blk0 + 64u * i + ld_row;
             p = p > pos_last ? pos_last : p; // rows past the last needed position are masked anyway,
             p = p < kfirst ? kfirst : p;     // and so are rows before the first one (a ring may not hold them any more)
             const uint32_t r = ring ? p % slots : p;
@@ -2901,8 +2903,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
             for (int i = 0; i < 16; ++i) ot[db][i] = 0.0f;
         }
         // blocks of 32 keys from the one that holds the first visible key to the one that holds the last
-        const uint32_t b_end = min((pos_last - tile0) / 32u + 1u, 2u * PW_TILES);
-        for (uint32_t b = (kfirst - tile0) / 32u; b < b_end; ++b) {
+        for (uint32_t b = 0; b < n_blocks; ++b) {
             bf16x8 ka[4];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) ka[ks] = as_bf16x8(*(const uint4 *)(&s_k[(k_lane_off ^ (16u * ks)) + b * 2048u]));
@@ -2922,7 +2923,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS, 4) void lng_prefill_bf16_d64
                 }
             }
             // key kp = b0 + 4 hh + o_i is visible when 0 <= my_pos - kp < window; a block every row sees whole skips it
-            const uint32_t b0 = tile0 + 32u * b;
+            const uint32_t b0 = blk0 + 32u * b;
             if (b0 + 31u > pos_first || b0 + window < pos_first + 32u) {
                 const int dist = (int)(my_pos - (b0 + 4u * hh));
                 const int below = dist - (int)window;
