@@ -800,23 +800,28 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
         const bool stream = stream_can && (plain_wgs >= g->cus || g->knobs.prefill_stream == 1);
         // Between the two - 64-row tiles, but fewer (query tile, kv head) pairs than compute units (a prompt fed 512 rows
         // at a time) - a workgroup per (query tile, kv head, PAIR of heads) that deals the keys out among its own
-        // wavefronts: four times the workgroups and nothing to merge afterwards. From half the units busy on
+        // wavefronts: four times the workgroups and nothing to merge afterwards
         // (LNG_PREFILL_PAIR: 0 never, 1 whenever it can run).
         const uint64_t head_pairs = (s.heads / s.kv_heads + 1) / 2;
         const bool pair_can = !f32 && !narrow && !stream && g->knobs.prefill_pair != 0 && g->knobs.prefill_splits == 0;
         bool pair = pair_can && g->knobs.prefill_pair == 1;
         if (pair_can && g->knobs.prefill_pair < 0 && plain_wgs < g->cus && head_pairs > 1) {
-            // Which is faster depends on how many keys a call walks: a head-pair workgroup walks all of them (measured
-            // on 64/8 heads: 15 us + 1.9 us per 256 keys, half as much again per key beyond 6,656, where a kv head's K
-            // and V no longer stay in its XCD's L2; as many rounds as the workgroups need on the device's units), a
-            // split workgroup only its share (25 us + 1.6 us per 64 keys of it, and 8 us for the merge dispatch).
+            // Which is faster depends on how many keys a call walks: a head-pair workgroup walks all keys of its query
+            // tile, a split workgroup only its share. Fitted to single calls of 192-1,920 rows after 0-4,096 positions
+            // and to the 16 calls of 512 rows of an 8,192-position prompt (64/8 heads, to within 3 us): head pairs take
+            // 3 us + per round of workgroups on the device's units (9 us + 1.9 us per 256 keys that a row sees on average,
+            // half as much again per key beyond 6,656, where a kv head's K and V no longer stay in its XCD's L2); the
+            // other kernel 10 us + 1.6 us per 64 keys of the longest run, or, with the keys split, 25 us (the merge
+            // dispatch included) + 1.6 us per 64 keys of a split's share.
             // 8,192 positions in calls of 512 rows: 857 -> 735 us; 4,096 in calls of 256: 508 -> 451 us; 2,048 in calls
-            // of 128: 385 -> 313 us; but calls of 256 rows at 8,192 positions and of 512 rows at 16,384 are slower.
-            const double keys = (double)visible;
+            // of 128: 385 -> 313 us; one call of 1,024 rows: 40.8 -> 28.4 us; calls of 256 rows at 8,192 positions, of
+            // 512 rows at 16,384 and one call of 1,920 rows stay with the other kernel.
+            const double seen_avg = (double)visible - (p.window == LNG_WINDOW_FULL ? 0.5 * (double)std::min<uint64_t>(s.t, visible) : 0.0);
             const uint64_t rounds = (plain_wgs * head_pairs + g->cus - 1) / g->cus;
-            const double pair_us = 15.0 + (double)rounds * (1.9 / 256.0) * (keys + (keys > 6656.0 ? 0.5 * (keys - 6656.0) : 0.0));
+            const double pair_us = 3.0 + (double)rounds * (9.0 + (1.9 / 256.0) * (seen_avg + (seen_avg > 6656.0 ? 0.5 * (seen_avg - 6656.0) : 0.0)));
             const uint64_t would_split = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, key_tiles / 4), 64));
-            const double split_us = 25.0 + (would_split > 1 && key_tiles >= 12 ? 8.0 + (1.6 / 64.0) * keys / (double)would_split : (1.6 / 64.0) * keys);
+            const bool splits = would_split > 1 && key_tiles >= 12;
+            const double split_us = splits ? 25.0 + (1.6 / 64.0) * (double)visible / (double)would_split : 10.0 + (1.6 / 64.0) * (double)visible;
             pair = pair_us < split_us;
         }
         if (!stream && !pair && (!narrow || few_rows) && plain_wgs < g->cus && s.t * s.kv_heads <= 65535) {
