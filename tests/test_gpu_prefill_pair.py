@@ -114,6 +114,33 @@ def test_random_shapes_on_the_head_pair_kernel(gpu, knobs):
     assert ran >= 35, ran
 
 
+def test_head_pair_kernel_counts_the_query_tiles_it_makes_again(gpu, knobs):
+    """LNG_COUNT_SECOND_PASSES: a key whose score is about 10,000 above the rest, late in the run, fails the range check
+    of the attempts that fix their reference point (the counter moves, per workgroup and failed attempt); benign scores
+    never do (the counter stays at zero); both results are right."""
+    knobs.setenv("LNG_PREFILL_STREAM", "0")
+    knobs.setenv("LNG_PREFILL_PAIR", "1")
+    knobs.setenv("LNG_COUNT_SECOND_PASSES", "1")
+    t, heads, kv_heads = 1024, 16, 2
+    gpu.debug_get("LNG_COUNT_SECOND_PASSES")
+    for spike in (False, True):
+        q, k, v, sinks = normal_inputs(123, t, t, heads, kv_heads, 64, scale=0.5)
+        if spike:
+            q[:] = np.abs(q) + 1.0
+            k[700] = 30.0
+        qb, kb, vb = to_bf16_bits(q), to_bf16_bits(k), to_bf16_bits(v)
+        shape = C.GroupedShape(t, 0, heads, kv_heads, 64, FULL, t, 0.125)
+        want = from_bf16_bits(oracle.attention_bf16(qb, kb, vb, sinks, 0, scale=0.125, threads=THREADS))
+        got = from_bf16_bits(run_attention(gpu, qb, kb, vb, sinks, shape, True, C.BF16, expect_kernel=PAIR))
+        assert max_error(got, want) < BF16_TOL
+        again = gpu.debug_get("LNG_COUNT_SECOND_PASSES")
+        if spike:
+            # the query tiles that see key 700 behind interior steps: tiles 11..15 of 16, x 2 kv heads x 4 pairs of heads
+            assert again >= 5 * 2 * 4, again
+        else:
+            assert again == 0, again
+
+
 @pytest.mark.parametrize("t,start,slots,expect", [
     (512, 3584, 4096, PAIR),                   # a 512-row chunk of a prompt: 64 (query tile, kv head) pairs on 256 units
     (256, 1024, 1280, PAIR), (128, 1920, 2048, PAIR),
