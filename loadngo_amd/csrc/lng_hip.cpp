@@ -809,16 +809,16 @@ int attention(lng_batch *b, lng_slice q, lng_slice k, lng_slice v, lng_slice out
             // Which is faster depends on how many keys a call walks: a head-pair workgroup walks all keys of its query
             // tile, a split workgroup only its share. Fitted to single calls of 192-1,920 rows after 0-4,096 positions
             // and to the 16 calls of 512 rows of an 8,192-position prompt (64/8 heads, to within 3 us): head pairs take
-            // 3 us + per round of workgroups on the device's units (9 us + 1.9 us per 256 keys that a row sees on average,
-            // half as much again per key beyond 6,656, where a kv head's K and V no longer stay in its XCD's L2); the
-            // other kernel 10 us + 1.6 us per 64 keys of the longest run, or, with the keys split, 25 us (the merge
-            // dispatch included) + 1.6 us per 64 keys of a split's share.
-            // 8,192 positions in calls of 512 rows: 857 -> 735 us; 4,096 in calls of 256: 508 -> 451 us; 2,048 in calls
-            // of 128: 385 -> 313 us; one call of 1,024 rows: 40.8 -> 28.4 us; calls of 256 rows at 8,192 positions, of
-            // 512 rows at 16,384 and one call of 1,920 rows stay with the other kernel.
+            // 3 us + per round of workgroups on the device's units (9 us + 1.9 us per 256 keys that a row sees on
+            // average); the other kernel 10 us + 1.6 us per 64 keys of the longest run, or, with the keys split, 25 us
+            // (the merge dispatch included) + 1.6 us per 64 keys of a split's share.
+            // 8,192 positions in calls of 512 rows: 855 -> 686 us; 16,384 in calls of 512: 2,543 -> 2,364 us (head pairs
+            // up to about 12,000 keys); 4,096 in calls of 256: 506 -> 407 us; 2,048 in calls of 128: 384 -> 277 us; one
+            // call of 1,024 rows: 40.8 -> 28.7 us; calls of 256 rows beyond about 3,300 keys and one call of 1,920 rows
+            // stay with the other kernel.
             const double seen_avg = (double)visible - (p.window == LNG_WINDOW_FULL ? 0.5 * (double)std::min<uint64_t>(s.t, visible) : 0.0);
             const uint64_t rounds = (plain_wgs * head_pairs + g->cus - 1) / g->cus;
-            const double pair_us = 3.0 + (double)rounds * (9.0 + (1.9 / 256.0) * (seen_avg + (seen_avg > 6656.0 ? 0.5 * (seen_avg - 6656.0) : 0.0)));
+            const double pair_us = 3.0 + (double)rounds * (9.0 + (1.9 / 256.0) * seen_avg);
             const uint64_t would_split = std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(g->cus / plain_wgs, key_tiles / 4), 64));
             const bool splits = would_split > 1 && key_tiles >= 12;
             const double split_us = splits ? 25.0 + (1.6 / 64.0) * (double)visible / (double)would_split : 10.0 + (1.6 / 64.0) * (double)visible;

@@ -14,6 +14,11 @@
 // barrier, by loads that write LDS directly and need no registers; the ids put the kv head fastest, so what the 32
 // workgroups of a kv head ask for lies in one XCD's L2.
 //
+// The two staging buffers are two arrays, and the interior loop takes two steps a turn with each buffer named outright:
+// with one array and a computed index the compiler cannot tell the rows a direct load is writing from the rows being
+// read, and makes the first LDS read after the loads wait for all of them (s_waitcnt vmcnt(0)) - the step after next
+// would then arrive before this one's arithmetic starts instead of during it.
+//
 // LDS rows are 128 bytes, unpadded (a direct load puts lane l's 16 bytes at base + 16 l), swizzled as in
 // lng_prefill_bf16_d64_h1w: piece c of K row r at c ^ ((r >> 1) & 7), piece c of V row r at c ^ (((r >> 1) & 1) << 2).
 // The arithmetic of a block of 32 keys is lng_prefill_bf16_d64's (two heads per wavefront), with the same three
@@ -39,7 +44,11 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     constexpr int NH = 2;
     // [buffer][K, V][256 rows x 64]; after the last step: the accumulators being exchanged, then the table of
     // (maximum, sum) and the outputs on their way to whole-row stores
-    __shared__ __attribute__((aligned(16))) uint16_t s_mem[PP_LDS_BYTES / 2u];
+    // Two arrays, not one with an index: where a step's buffers are named outright the compiler can tell that the rows a
+    // direct load is writing are not the rows being read, and does not make every LDS read wait for the loads in flight.
+    __shared__ __attribute__((aligned(16))) uint16_t s_buf0[2u * PP_TILE_ELEMS]; // K then V of the even steps (64 KiB)
+    __shared__ __attribute__((aligned(16))) uint16_t s_buf1[2u * PP_TILE_ELEMS]; // of the odd steps
+    __shared__ __attribute__((aligned(16))) uint16_t s_tail[(PP_LDS_BYTES - PP_ML_OFF) / 2u];
     __shared__ uint32_t s_far, s_again;
 
     const uint32_t group = a.heads / a.kv_heads;
@@ -129,8 +138,9 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     // ---- the 256 rows of step s, K and V, into buffer s & 1: four direct loads of each per wavefront --------------
     typedef __attribute__((address_space(1))) const void *gptr;
     typedef __attribute__((address_space(3))) void *lptr;
-    auto ask = [&](uint32_t s) __attribute__((always_inline)) {
-        const uint32_t kdst = (s & 1u) * (2u * PP_TILE_ELEMS) + wave * 512u, vdst = kdst + PP_TILE_ELEMS; // elements of s_mem
+    auto buf_of = [&](uint32_t s) __attribute__((always_inline)) { return (s & 1u) ? &s_buf1[0] : &s_buf0[0]; };
+    auto ask = [&](uint32_t s, uint16_t *dst) __attribute__((always_inline)) {
+        const uint32_t kdst = wave * 512u, vdst = kdst + PP_TILE_ELEMS; // elements of dst
         const uint32_t p0 = tile0 + PP_STEP * s;
         if (!ring && p0 >= kfirst && p0 + (PP_STEP - 1u) <= pos_last) {
             // every row is there and wanted: one base per load, worked out by the scalar unit, plus the lane's offset
@@ -139,8 +149,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
 #pragma unroll
             for (uint32_t i = 0; i < PP_STEP / 64u; ++i) { // eight wavefronts x eight rows at a time
                 const uint64_t ko = kb + (uint64_t)(64u * i) * row_bytes, vo = vb + (uint64_t)(64u * i) * row_bytes;
-                __builtin_amdgcn_global_load_lds((gptr)(scalar64(ko) + k_ask_off), (lptr)&s_mem[kdst + i * 4096u], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((gptr)(scalar64(vo) + v_ask_off), (lptr)&s_mem[vdst + i * 4096u], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr)(scalar64(ko) + k_ask_off), (lptr)&dst[kdst + i * 4096u], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr)(scalar64(vo) + v_ask_off), (lptr)&dst[vdst + i * 4096u], 16, 0, 0);
             }
         } else {
             const uint32_t kc = k_ask_off - (lane >> 3) * row_bytes, vc = v_ask_off - (lane >> 3) * row_bytes;
@@ -150,8 +160,8 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
                 p = p > pos_last ? pos_last : p; // rows past the last needed position are masked or never used,
                 p = p < kfirst ? kfirst : p;     // and so are rows before the first one (a ring may not hold them any more)
                 const uint32_t r = ring ? p % slots : p;
-                __builtin_amdgcn_global_load_lds((gptr)(a.k + (uint64_t)g * 128u + (uint64_t)r * row_bytes + kc), (lptr)&s_mem[kdst + i * 4096u], 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((gptr)(a.v + (uint64_t)g * 128u + (uint64_t)r * row_bytes + vc), (lptr)&s_mem[vdst + i * 4096u], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr)(a.k + (uint64_t)g * 128u + (uint64_t)r * row_bytes + kc), (lptr)&dst[kdst + i * 4096u], 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr)(a.v + (uint64_t)g * 128u + (uint64_t)r * row_bytes + vc), (lptr)&dst[vdst + i * 4096u], 16, 0, 0);
             }
         }
     };
@@ -187,19 +197,19 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
             for (int i = 0; i < 16; ++i) ot[h][db][i] = 0.0f;
         }
     }
-    ask(0);
+    ask(0, s_buf0);
     landed();
 
     // One block of 32 keys (kb = 0, 1 of the wavefront's sub-tile of step s) for both heads.
     // MODE 0: the running maximum is tracked. MODE 1: it is fixed. MODE 2: it is fixed at zero.
-    auto block = [&](auto mask_tag, auto mode_tag, uint32_t s, int kb) __attribute__((always_inline)) {
+    auto block = [&](auto mask_tag, auto mode_tag, const uint16_t *src, uint32_t s, int kb) __attribute__((always_inline)) {
         constexpr bool MASK = decltype(mask_tag)::value;
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool FIXED = MODE != 0;
-        const uint32_t kt = (s & 1u) * (2u * PP_TILE_ELEMS) + kq * 4096u + kb * 2048, vt = kt + PP_TILE_ELEMS; // elements of s_mem
+        const uint32_t kt = kq * 4096u + kb * 2048, vt = kt + PP_TILE_ELEMS; // elements of src
         bf16x8 ka[4];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) ka[ks] = as_bf16x8(*(const uint4 *)(&s_mem[kt + (k_lane_off ^ (16u * ks))]));
+        for (int ks = 0; ks < 4; ++ks) ka[ks] = as_bf16x8(*(const uint4 *)(&src[kt + (k_lane_off ^ (16u * ks))]));
         floatx16 st[NH];
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
@@ -216,7 +226,7 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         for (int jj = 0; jj < 2; ++jj) {
 #pragma unroll
             for (int db = 0; db < 2; ++db) {
-                const uint16_t *vp = &s_mem[vt + v_lane_off + (16 * jj) * 64u + 32 * (db ^ v_flip)];
+                const uint16_t *vp = &src[vt + v_lane_off + (16 * jj) * 64u + 32 * (db ^ v_flip)];
                 va[jj][db] = lds_read_tr8(vp, vp + 8 * 64);
             }
         }
@@ -303,22 +313,22 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     using fixed_at_zero = std::integral_constant<int, 2>;
     // a step of any kind, the maximum tracked: each wavefront looks at its own sub-tile
     auto any_step = [&](uint32_t s) __attribute__((always_inline)) {
-        if (s + 1u < n_steps) ask(s + 1u);
+        if (s + 1u < n_steps) ask(s + 1u, buf_of(s + 1u));
         const uint32_t j = 4u * s + kq;
         if (j < all_tiles) {
             if (edge(j)) {
-                block(std::true_type{}, tracked{}, s, 0);
-                block(std::true_type{}, tracked{}, s, 1);
+                block(std::true_type{}, tracked{}, buf_of(s), s, 0);
+                block(std::true_type{}, tracked{}, buf_of(s), s, 1);
             } else {
-                block(std::false_type{}, tracked{}, s, 0);
-                block(std::false_type{}, tracked{}, s, 1);
+                block(std::false_type{}, tracked{}, buf_of(s), s, 0);
+                block(std::false_type{}, tracked{}, buf_of(s), s, 1);
             }
         }
     };
     auto fixed_step = [&](auto mode_tag, uint32_t s) __attribute__((always_inline)) {
-        if (s + 1u < n_steps) ask(s + 1u);
-        block(std::false_type{}, mode_tag, s, 0);
-        block(std::false_type{}, mode_tag, s, 1);
+        if (s + 1u < n_steps) ask(s + 1u, buf_of(s + 1u));
+        block(std::false_type{}, mode_tag, buf_of(s), s, 0);
+        block(std::false_type{}, mode_tag, buf_of(s), s, 1);
         landed();
     };
     uint32_t s = 0;
@@ -366,14 +376,28 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     }
     if (frozen) { // loops of their own: one path through each
         if (at_zero) {
+            if ((s & 1u) && s < n_steps && interior(s)) { // to an even step first
+                fixed_step(fixed_at_zero{}, s);
+                ++s;
+            }
+            for (; s + 1u < n_steps && interior(s + 1u); s += 2u) { // two steps a turn, their buffers named outright
+                ask(s + 1u, s_buf1);
+                block(std::false_type{}, fixed_at_zero{}, s_buf0, s, 0);
+                block(std::false_type{}, fixed_at_zero{}, s_buf0, s, 1);
+                landed();
+                if (s + 2u < n_steps) ask(s + 2u, s_buf0);
+                block(std::false_type{}, fixed_at_zero{}, s_buf1, s + 1u, 0);
+                block(std::false_type{}, fixed_at_zero{}, s_buf1, s + 1u, 1);
+                landed();
+            }
             for (; s < n_steps && interior(s); ++s) fixed_step(fixed_at_zero{}, s);
             // the step of the diagonal at the same reference point and ahead of the check, which then covers it (a
             // masked score is 2^-inf = 0; every sub-tile through the masks, so that there is one more form of the block only)
             for (; s < n_steps; ++s) {
-                if (s + 1u < n_steps) ask(s + 1u);
+                if (s + 1u < n_steps) ask(s + 1u, buf_of(s + 1u));
                 if (4u * s + kq < all_tiles) {
-                    block(std::true_type{}, fixed_at_zero{}, s, 0);
-                    block(std::true_type{}, fixed_at_zero{}, s, 1);
+                    block(std::true_type{}, fixed_at_zero{}, buf_of(s), s, 0);
+                    block(std::true_type{}, fixed_at_zero{}, buf_of(s), s, 1);
                 }
                 landed();
             }
@@ -431,15 +455,15 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
     // nobody reads K or V any more.
     lane_values();
     row_values();
-    float *const xch = (float *)&s_mem[0];
-    float2 *const ml = (float2 *)&s_mem[PP_ML_OFF / 2u];
+    float *const xch = (float *)(qb ? &s_buf1[0] : &s_buf0[0]); // a query block's 64 KiB
+    float2 *const ml = (float2 *)&s_tail[0];
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
         const float total = l[h] + __shfl_xor(l[h], 32, 64);
         if (hh == 0u) ml[((qb * 4u + kq) * 2u + h) * 32u + n] = make_float2(m[h], total);
 #pragma unroll
         for (int db = 0; db < 2; ++db) {
-            float *const dst = xch + ((((qb * 4u + (2u * h + db)) * 4u + kq) * 4u) * 64u + lane) * 4u;
+            float *const dst = xch + (((((2u * h + db)) * 4u + kq) * 4u) * 64u + lane) * 4u;
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
                 *(float4 *)(dst + blk * 256u) = make_float4(ot[h][db][4 * blk + 0], ot[h][db][4 * blk + 1], ot[h][db][4 * blk + 2], ot[h][db][4 * blk + 3]);
@@ -467,13 +491,13 @@ extern "C" __global__ __launch_bounds__(PF_THREADS) void lng_prefill_bf16_d64_pa
         total += lk[k] * w[k];
     }
     const float inv = total > 0.0f ? 1.0f / total : 0.0f;
-    uint16_t *const stage = &s_mem[PP_OUT_OFF / 2u + wave * (32u * PP_OUT_STRIDE)];
+    uint16_t *const stage = &s_tail[(PP_OUT_OFF - PP_ML_OFF) / 2u + wave * (32u * PP_OUT_STRIDE)];
 #pragma unroll
     for (int blk = 0; blk < 4; ++blk) {
         float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const float4 piece = *(const float4 *)(xch + ((((qb * 4u + kq) * 4u + k) * 4u + blk) * 64u + lane) * 4u);
+            const float4 piece = *(const float4 *)(xch + (((kq * 4u + k) * 4u + blk) * 64u + lane) * 4u);
             const float wk = w[k] * inv;
             // (a wavefront that saw no key left zeros and has weight 0: no NaN from 0 x inf, its piece is finite)
             sum.x = __builtin_fmaf(piece.x, wk, sum.x);
